@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused linear cross-entropy (forward + backward) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
+
+A step is one forward + backward of ``tiled_linear_cross_entropy`` over one
+synthetic batch that is already resident in HBM.  Prints ONE JSON line:
+tokens/s (loss-bearing rows per second), the roofline of the dominant kernel
+class measured live with HIP events, and the CPU oracle timed on a bounded row
+sample of the same workload on this box's host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+REPO_ROOT = Path(__file__).resolve().parent
+if str(REPO_ROOT) not in sys.path:
+    sys.path.insert(0, str(REPO_ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+
+
+def build_workload(name: str, seed: int):
+    from turbo_dllm_amd import workloads
+
+    if name == "block_diffusion_shard_all_rows":
+        return workloads.block_diffusion_shard(seed=seed, all_rows_loss_bearing=True)
+    return workloads.CONFIGS[name](seed=seed)
+
+
+def cpu_baseline(wl, sample_rows: int):
+    """Oracle (unfused float32 path + analytic gradients) on the first
+    ``sample_rows`` loss-bearing rows, all host threads."""
+    import torch
+
+    sys.path.insert(0, str(REPO_ROOT / "oracle"))
+    import linear_ce_oracle as oracle
+
+    keep = torch.nonzero(wl.labels != -100).flatten()[:sample_rows]
+    hidden = wl.hidden.index_select(0, keep).float()
+    labels = wl.labels.index_select(0, keep)
+    weight = wl.weight.float()
+    cores = torch.get_num_threads()
+    t0 = time.perf_counter()
+    oracle.dense_linear_ce(hidden, weight, labels, logit_softcap=wl.logit_softcap,
+                           dtype=torch.float32)
+    oracle.dense_linear_ce_grads(hidden, weight, labels, logit_softcap=wl.logit_softcap,
+                                 dtype=torch.float32)
+    dt = time.perf_counter() - t0
+    rows = int(keep.numel())
+    return {
+        "value": rows / dt,
+        "unit": "tokens/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"fwd+bwd of the float32 oracle on the first {rows} loss-bearing rows "
+                  f"(full H and V), {dt:.2f} s",
+    }
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="block_diffusion_shard_all_rows")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path "
+              f"(--gpus {args.gpus} is not supported; use --gpus 1)", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from turbo_dllm_amd import _lib
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 1
+    device = torch.device("cuda:0")
+    native.verify_device(0)
+
+    wl = build_workload(args.workload, args.seed)
+    n, m = wl.n_rows, wl.n_loss_rows
+    h, v = wl.hidden.shape[1], wl.weight.shape[0]
+    hidden = wl.hidden.to(device).requires_grad_(True)
+    weight = wl.weight.to(device).requires_grad_(True)
+    labels = wl.labels.to(device)
+
+    def step():
+        hidden.grad = None
+        weight.grad = None
+        loss = tiled_linear_cross_entropy(hidden, weight, labels, reduction="mean",
+                                          logit_softcap=wl.logit_softcap, dtype=hidden.dtype,
+                                          weight_layout="vocab_first")
+        loss.backward()
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        loss = step()
+    stop.record()
+    torch.cuda.synchronize()
+    ms_per_step = start.elapsed_time(stop) / args.steps
+    loss_value = float(loss)
+
+    # per-kernel-class durations of one forward + backward (HIP events on the launch stream)
+    with torch.no_grad():
+        row_idx, m_dev = native.compact_rows(labels, -100)
+        rows = hidden.detach() if m_dev == n else native.gather_rows(hidden.detach(), row_idx)
+        targets = labels if m_dev == n else native.gather_rows(labels, row_idx)
+        idx = None if m_dev == n else row_idx
+        kw = dict(row_block_size=0, ignore_index=-100, exclude_index=-1,
+                  logit_softcap=float(wl.logit_softcap or 0.0), compute_dtype=hidden.dtype,
+                  weight_dim_first=False, row_idx=idx, n_out=n)
+        go = torch.ones(1, device=device)
+        with _lib.kernel_profile() as prof:
+            _, lse, count = native.forward(rows, weight.detach(), None, targets, **kw)
+            native.backward(rows, weight.detach(), None, targets, lse, count, go,
+                            reduction="mean", **kw)
+        torch.cuda.synchronize()
+
+    gemm_classes = ("forward_stats", "grad_logits_panel", "grad_hidden_gemm", "grad_weight_gemm")
+    dominant = max(gemm_classes, key=lambda c: prof.ms[c])
+    contraction_tflop = 2.0 * m * h * v / 1e12          # algorithmic FLOPs of one contraction
+    launches = max(prof.launches[dominant], 1)
+    avg_ms = prof.ms[dominant] / launches
+    achieved = (contraction_tflop / launches) / (avg_ms / 1e3)
+    useful_tflops = 3.0 * contraction_tflop / (ms_per_step / 1e3)
+    executed_tflops = 4.0 * contraction_tflop / (ms_per_step / 1e3)
+    plan = _lib.query_plan(m, h, v, _lib.DTYPE_BF16, True, native.PANEL_BYTES)
+
+    result = {
+        "metric": "fused linear-CE fwd+bwd tokens/s",
+        "value": m / (ms_per_step / 1e3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{wl.name}: N={n} rows, M={m} loss-bearing, H={h}, V={v}, "
+                        f"softcap={wl.logit_softcap}, seed={args.seed}",
+            "input_rows_per_s": n / (ms_per_step / 1e3),
+            "plan": plan,
+        },
+        "loss": loss_value,
+        "tflops_useful_6MHV": useful_tflops,
+        "tflops_executed_8MHV": executed_tflops,
+        "frac_of_bf16_peak_useful": useful_tflops / PEAK_BF16_TFLOPS,
+        "mfma_util_executed": executed_tflops / PEAK_BF16_TFLOPS,
+        "kernel_ms": {k: round(x, 3) for k, x in prof.ms.items()},
+        "kernel_launches": prof.launches,
+        "roofline": {
+            "kernel": dominant,
+            "bound": "mfma",
+            "achieved": achieved,
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved / PEAK_BF16_TFLOPS,
+            "traffic": None,
+            "avg_launch_ms": avg_ms,
+            "launches_per_step": launches,
+            "flops_per_launch": contraction_tflop / launches * 1e12,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(wl, args.cpu_rows)
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,169 @@
+/*
+ * tlce.h — C ABI of the MI355X (gfx950) fused linear cross-entropy library
+ * (libtlce_gfx950.so).
+ *
+ * The library replaces the device half of the reference's
+ * `dllm_fused_linear_ce_v3` extension for the LM-head projection +
+ * masked-token cross-entropy (forward and backward).  Every entry point takes
+ * raw device pointers, sizes and a HIP stream; nothing here allocates, frees or
+ * synchronises: the caller owns outputs and workspaces and sizes them with the
+ * `*_workspace_bytes` helpers.  All matrices are contiguous row-major.
+ *
+ * Reference interfaces replaced (paths relative to the reference tree):
+ *   chunked_linear_ce_forward               dllm_parallel/core/csrc/fused_linear_ce/fused_linear_ce.cpp:94-123
+ *   chunked_linear_ce_backward              dllm_parallel/core/csrc/fused_linear_ce/fused_linear_ce.cpp:125-162
+ *   chunked_linear_ce_backward_frozen_weight dllm_parallel/core/csrc/fused_linear_ce/fused_linear_ce.cpp:164-207
+ *   (their device side: fused_linear_ce_cuda.cu:898-989 and :991-1172)
+ *   row compaction at the loss call sites   dllm_parallel/core/models/backbones/nemotron/model.py:4234-4253
+ *
+ * Conventions
+ *   - every function returning `int` returns 0 on success, non-zero on failure;
+ *     `tlce_last_error()` then holds a thread-local message.
+ *   - `stream` is a `hipStream_t` passed as `void*` (NULL = the null stream).
+ *   - `dtype` is one of TLCE_DTYPE_*; hidden, weight and gradients share it.
+ *   - `bias` is always float32 (the reference converts it the same way,
+ *     fused_linear_ce_cuda.cu:913-916); NULL means "no bias".
+ *   - `row_idx` (int64, ascending, length m) maps compacted row r to its
+ *     position in the un-compacted [n_out] token axis; NULL means rows are
+ *     already in place (n_out == m).
+ *   - `exclude_index < 0` means no excluded vocabulary column;
+ *     `logit_softcap <= 0` means no soft cap.
+ */
+#ifndef TLCE_H_
+#define TLCE_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TLCE_VERSION 1
+
+enum {
+  TLCE_DTYPE_F32 = 0,
+  TLCE_DTYPE_F16 = 1,
+  TLCE_DTYPE_BF16 = 2
+};
+
+/* reduction codes, same numbering as the reference binding shim
+ * (dllm_parallel/core/kernels/chunked_linear_ce_native.py:366-373) */
+enum {
+  TLCE_REDUCTION_NONE = 0,
+  TLCE_REDUCTION_SUM = 1,
+  TLCE_REDUCTION_MEAN = 2
+};
+
+/* Library version (TLCE_VERSION it was built with). */
+int tlce_version(void);
+
+/* Thread-local text of the last failure on the calling thread ("" if none). */
+const char* tlce_last_error(void);
+
+/* 0 when `device` is a gfx950 GPU this library was compiled for.  Replaces
+ * the architecture check of the reference's packaged-kernel loader
+ * (dllm_parallel/core/kernels/runtime.py:189-387). */
+int tlce_check_device(int device);
+
+/* ---- masked-position compaction / gather --------------------------------
+ * Device counterpart of `_compact_valid_loss_rows`
+ * (nemotron/model.py:4234-4253): row_idx = nonzero(labels != ignore_index),
+ * ascending int64, then index_select of the loss-bearing rows. */
+
+/* Bytes of scratch `tlce_compact_rows` needs for `n` labels. */
+int64_t tlce_compact_workspace_bytes(int64_t n);
+
+/* Writes the ascending indices of labels[i] != ignore_index to row_idx_out
+ * (capacity n) and their count to count_out[0] (device int64). */
+int tlce_compact_rows(const int64_t* labels, int64_t n, int64_t ignore_index,
+                      int64_t* row_idx_out, int64_t* count_out,
+                      void* workspace, int64_t workspace_bytes, void* stream);
+
+/* dst[r, :] = src[row_idx[r], :] for r < m; rows are `row_bytes` long and
+ * contiguous in both buffers (index_select along dim 0). */
+int tlce_gather_rows(const void* src, const int64_t* row_idx, int64_t m,
+                     int64_t row_bytes, void* dst, void* stream);
+
+/* dst[row_idx[r], :] = src[r, :] for r < m.  dst is NOT cleared here; rows not
+ * named by row_idx keep their contents (the backward of index_select into a
+ * zero-filled buffer, valid because row_idx has no duplicates). */
+int tlce_scatter_rows(const void* src, const int64_t* row_idx, int64_t m,
+                      int64_t row_bytes, void* dst, void* stream);
+
+/* Zero-fills `bytes` bytes at dst with a kernel (safe inside graph capture). */
+int tlce_fill_zero(void* dst, int64_t bytes, void* stream);
+
+/* ---- forward -------------------------------------------------------------
+ * Replaces chunked_linear_ce_forward (fused_linear_ce.cpp:94-123).
+ *   hidden [m,h], weight [v,h] (vocab-first), labels [m] int64.
+ * Outputs: losses (float32; written at row_idx[r] when row_idx != NULL, in
+ * which case all n_out entries are first cleared; 0 for ignored rows),
+ * lse [m] float32, valid_count [1] float32 (number of rows whose label is not
+ * ignore_index).  No [rows, vocab] logits buffer is used: the workspace holds
+ * only per-row softmax partials. */
+int64_t tlce_forward_workspace_bytes(int64_t m, int64_t h, int64_t v, int dtype);
+
+int tlce_forward(const void* hidden, const void* weight, const float* bias,
+                 const int64_t* labels, const int64_t* row_idx,
+                 int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                 int64_t ignore_index, int64_t exclude_index,
+                 float logit_softcap,
+                 float* losses, float* lse, float* valid_count,
+                 void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- backward ------------------------------------------------------------
+ * Replaces chunked_linear_ce_backward and ..._backward_frozen_weight
+ * (fused_linear_ce.cpp:125-207).  grad_weight == NULL selects the
+ * frozen-weight variant.
+ *   grad_output: float32, [n_out] for TLCE_REDUCTION_NONE, [1] otherwise.
+ *   grad_hidden [n_out,h] (dtype): rows named by row_idx receive the gradient
+ *   and every other row is cleared; grad_weight [v,h] (dtype);
+ *   grad_bias [v] (float32, only when bias != NULL).
+ * The gradient of the logits is rounded to `dtype` before the two gradient
+ * contractions, as the reference does (fused_linear_ce_cuda.cu:1110-1123).
+ * `panel_bytes` bounds the staging panel of vocabulary columns that carries
+ * those rounded logit gradients between the kernels (<= 0: default). */
+int64_t tlce_backward_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                      int dtype, int compute_weight_grad,
+                                      int has_bias, int64_t panel_bytes);
+
+int tlce_backward(const void* hidden, const void* weight, const float* bias,
+                  const int64_t* labels, const int64_t* row_idx,
+                  const float* lse, const float* valid_count,
+                  const float* grad_output,
+                  int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                  int reduction_code, int64_t ignore_index,
+                  int64_t exclude_index, float logit_softcap,
+                  void* grad_hidden, void* grad_weight, float* grad_bias,
+                  int64_t panel_bytes,
+                  void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- introspection used by the benchmark and the tests -------------------
+ * Tile plan the host scheduler would use for a problem; any pointer may be
+ * NULL.  `engine` is 1 for the bf16/f16 MFMA kernels, 0 for the generic
+ * float32-FMA kernels (float32 inputs, or h not a multiple of 8). */
+int tlce_query_plan(int64_t m, int64_t h, int64_t v, int dtype,
+                    int compute_weight_grad, int64_t panel_bytes,
+                    int* engine, int64_t* tile, int64_t* forward_vocab_splits,
+                    int64_t* panel_columns, int64_t* n_panels,
+                    int64_t* grad_hidden_k_splits);
+
+/* ---- per-kernel timing (benchmark support; no reference counterpart) -----
+ * Between tlce_profile_begin() and tlce_profile_end() every kernel the calling
+ * thread launches through this library is bracketed by HIP events on its
+ * stream.  tlce_profile_end waits for them and adds up, per kernel class,
+ * the elapsed milliseconds and the launch count.  Classes:
+ *   0 forward logits+softmax-stats tiles   1 per-row loss merge
+ *   2 backward logit-gradient panel tiles  3 grad_hidden contraction
+ *   4 grad_weight contraction              5 operand transposes
+ *   6 fills, scales and casts
+ * The events allocate driver resources: not for use under graph capture. */
+#define TLCE_PROFILE_CLASSES 7
+int tlce_profile_begin(void);
+int tlce_profile_end(double* class_ms, int64_t* class_launches, int n_classes);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TLCE_H_ */

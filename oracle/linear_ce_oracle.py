@@ -1,0 +1,220 @@
+"""CPU oracle for the fused linear cross-entropy path.  TEST INFRASTRUCTURE ONLY.
+
+Nothing in the product package imports this module: it is the checker for
+``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of
+``bench.py``.  It restates, on the CPU, what the reference computes for this
+path; the reference is Python/CUDA and is read, not run.
+
+What each function follows in the reference (paths relative to its tree):
+
+  dense_linear_ce          the unfused path matmul -> (+bias) -> tanh soft cap ->
+                           excluded column -> log-softmax -> masked NLL, with the
+                           op order of ce_forward_kernel
+                           (dllm_parallel/core/csrc/fused_linear_ce/fused_linear_ce_cuda.cu:156-224)
+                           and the reductions of
+                           dllm_parallel/core/kernels/tiled_linear_cross_entropy.py:327-331.
+  dense_linear_ce_grads    ce_grad_logits_kernel + the two gradient GEMMs
+                           (fused_linear_ce_cuda.cu:226-290, :1049-1170); with
+                           round_grad_logits=True the logit gradient is rounded to
+                           the input dtype before the contractions, as the native
+                           path does (:1110-1123).
+  online_tiled_linear_ce   the streaming (max, sum) algorithm of the reference's
+                           CPU path (tiled_linear_cross_entropy.py:105-149).
+  compact_rows             nonzero(labels != ignore) of _compact_valid_loss_rows
+                           (dllm_parallel/core/models/backbones/nemotron/model.py:4234-4253).
+
+Pinning (tests/test_oracle_pins.py): every function above is checked against
+library routines it does not call (torch.nn.functional.cross_entropy, torch
+autograd through it, torch.nonzero), against brute-force Python loops on tiny
+inputs, against closed forms (uniform logits -> log V, gradient rows summing
+to zero, saturated soft cap), against the committed fixtures under
+tests/golden/, and against the seeded cases of the reference's own test file
+(tests/unit/kernels/test_tiled_linear_cross_entropy.py:61-453), which hold no
+stored vectors and compare to the same library routines.  No function here is
+"parity unpinned".
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import numpy as np
+import torch
+
+
+def _logits(hidden, weight, bias, *, weight_dim_first, logit_softcap, exclude_index, dtype):
+    h = hidden.reshape(-1, hidden.shape[-1]).to(dtype)
+    w = weight.to(dtype)
+    raw = h @ (w if weight_dim_first else w.t())
+    if bias is not None:
+        raw = raw + bias.to(dtype)
+    if logit_softcap and logit_softcap > 0:
+        squashed = torch.tanh(raw / logit_softcap)
+        capped = squashed * logit_softcap
+    else:
+        squashed = None
+        capped = raw
+    if exclude_index is not None and exclude_index >= 0:
+        capped = capped.clone()
+        capped[:, exclude_index] = -float("inf")
+    return capped, squashed
+
+
+def dense_linear_ce(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    bias: Optional[torch.Tensor] = None,
+    reduction: str = "mean",
+    ignore_index: int = -100,
+    exclude_index: Optional[int] = None,
+    logit_softcap: Optional[float] = None,
+    weight_dim_first: bool = False,
+    dtype: torch.dtype = torch.float64,
+    return_lse: bool = False,
+):
+    """Unfused reference value of the loss (and optionally the per-row lse)."""
+    logits, _ = _logits(hidden, weight, bias, weight_dim_first=weight_dim_first,
+                        logit_softcap=logit_softcap, exclude_index=exclude_index, dtype=dtype)
+    y = labels.reshape(-1).to(torch.long)
+    keep = y != ignore_index
+    row_max = logits.max(dim=-1).values
+    lse = row_max + torch.log(torch.exp(logits - row_max[:, None]).sum(dim=-1))
+    safe = torch.where(keep, y, torch.zeros_like(y))
+    target = logits.gather(1, safe[:, None]).squeeze(1)
+    losses = torch.where(keep, lse - target, torch.zeros_like(lse))
+    if reduction == "none":
+        out = losses.reshape(labels.shape)
+    elif reduction == "sum":
+        out = losses.sum()
+    elif reduction == "mean":
+        out = losses.sum() / keep.sum().to(dtype)
+    else:
+        raise ValueError(reduction)
+    return (out, lse) if return_lse else out
+
+
+def dense_linear_ce_grads(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    grad_output: Optional[torch.Tensor] = None,
+    *,
+    bias: Optional[torch.Tensor] = None,
+    reduction: str = "mean",
+    ignore_index: int = -100,
+    exclude_index: Optional[int] = None,
+    logit_softcap: Optional[float] = None,
+    weight_dim_first: bool = False,
+    dtype: torch.dtype = torch.float64,
+    round_grad_logits: Optional[torch.dtype] = None,
+):
+    """Analytic (grad_hidden, grad_weight, grad_bias) of ``dense_linear_ce``.
+
+    grad_output follows autograd: shaped like labels for reduction "none",
+    scalar otherwise (defaults to ones).
+    """
+    logits, squashed = _logits(hidden, weight, bias, weight_dim_first=weight_dim_first,
+                               logit_softcap=logit_softcap, exclude_index=exclude_index,
+                               dtype=dtype)
+    y = labels.reshape(-1).to(torch.long)
+    n = y.numel()
+    keep = y != ignore_index
+    lse = torch.logsumexp(logits, dim=-1)
+    if grad_output is None:
+        grad_output = torch.ones(labels.shape if reduction == "none" else (), dtype=dtype)
+    go = grad_output.to(dtype)
+    if reduction == "none":
+        scale = go.reshape(-1)
+    elif reduction == "sum":
+        scale = go.reshape(()).expand(n)
+    else:
+        scale = (go.reshape(()) / keep.sum().to(dtype)).expand(n)
+    scale = torch.where(keep, scale, torch.zeros_like(scale))
+    g = torch.exp(logits - lse[:, None])
+    rows = torch.nonzero(keep).flatten()
+    g[rows, y[rows]] -= 1.0
+    g = g * scale[:, None]
+    if squashed is not None:
+        g = g * (1.0 - squashed * squashed)
+    if round_grad_logits is not None:
+        g = g.to(round_grad_logits).to(dtype)
+    h = hidden.reshape(-1, hidden.shape[-1]).to(dtype)
+    w = weight.to(dtype)
+    if weight_dim_first:
+        grad_hidden = g @ w.t()
+        grad_weight = h.t() @ g
+    else:
+        grad_hidden = g @ w
+        grad_weight = g.t() @ h
+    grad_bias = g.sum(dim=0) if bias is not None else None
+    return grad_hidden.reshape(hidden.shape), grad_weight, grad_bias
+
+
+def online_tiled_linear_ce(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    vocab_block_size: int,
+    bias: Optional[torch.Tensor] = None,
+    ignore_index: int = -100,
+    exclude_index: Optional[int] = None,
+    logit_softcap: Optional[float] = None,
+    dtype: torch.dtype = torch.float32,
+):
+    """Per-row (losses, lse) by streaming vocabulary tiles with a running
+    (max, sum-of-exponentials) pair -- the algorithm every fused kernel of this
+    path implements.  Exclusion is applied after the soft cap (true removal)."""
+    h = hidden.reshape(-1, hidden.shape[-1]).to(dtype)
+    y = labels.reshape(-1).to(torch.long)
+    keep = y != ignore_index
+    n, vocab = h.shape[0], weight.shape[0]
+    run_max = torch.full((n,), -float("inf"), dtype=dtype)
+    run_sum = torch.zeros(n, dtype=dtype)
+    target = torch.zeros(n, dtype=dtype)
+    for lo in range(0, vocab, vocab_block_size):
+        hi = min(lo + vocab_block_size, vocab)
+        z = h @ weight[lo:hi].to(dtype).t()
+        if bias is not None:
+            z = z + bias[lo:hi].to(dtype)
+        if logit_softcap and logit_softcap > 0:
+            z = torch.tanh(z / logit_softcap) * logit_softcap
+        if exclude_index is not None and lo <= exclude_index < hi:
+            z[:, exclude_index - lo] = -float("inf")
+        new_max = torch.maximum(run_max, z.max(dim=-1).values)
+        finite = new_max > -float("inf")
+        shift = torch.where(finite, new_max, torch.zeros_like(new_max))
+        run_sum = torch.where(
+            finite,
+            run_sum * torch.exp(run_max - shift) + torch.exp(z - shift[:, None]).sum(dim=-1),
+            run_sum,
+        )
+        run_max = new_max
+        here = keep & (y >= lo) & (y < hi)
+        idx = torch.nonzero(here).flatten()
+        target[idx] = z[idx, y[idx] - lo]
+    lse = run_max + torch.log(run_sum)
+    return torch.where(keep, lse - target, torch.zeros_like(lse)), lse
+
+
+def compact_rows(labels, ignore_index: int = -100) -> np.ndarray:
+    """Ascending int64 indices of labels != ignore_index (numpy)."""
+    flat = np.asarray(labels).reshape(-1)
+    return np.flatnonzero(flat != ignore_index).astype(np.int64)
+
+
+def compact_rows_loop(labels, ignore_index: int = -100) -> list[int]:
+    """The same by a plain Python loop (tiny inputs only)."""
+    return [i for i, y in enumerate(np.asarray(labels).reshape(-1).tolist()) if y != ignore_index]
+
+
+def relative_max_error(actual: torch.Tensor, expected: torch.Tensor) -> float:
+    """max|a - e| / max|e|: the "relative max-norm error" of the gradient bars."""
+    a = actual.detach().to(torch.float64).cpu()
+    e = expected.detach().to(torch.float64).cpu()
+    denom = float(e.abs().max())
+    if denom == 0.0:
+        return float(a.abs().max())
+    return float((a - e).abs().max()) / denom

@@ -1,0 +1,82 @@
+"""The C-ABI library loads, exports exactly what include/tlce.h declares, and
+its host-side planning logic behaves (no compute calls: no GPU needed)."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from turbo_dllm_amd import _lib
+
+REPO_ROOT = Path(__file__).resolve().parent.parent
+HEADER = REPO_ROOT / "include" / "tlce.h"
+
+
+def declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    names = re.findall(r"\b(tlce_[a-z_0-9]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_header_and_binding_declare_the_same_entry_points():
+    assert declared_functions() == sorted(_lib.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.library()
+    for name in declared_functions():
+        assert hasattr(lib, name), name
+    assert lib.tlce_version() == 1
+    assert _lib.last_error() == ""
+
+
+def test_argument_counts_match_header():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    for name, (_, argtypes) in _lib.SIGNATURES.items():
+        match = re.search(rf"\b{name}\s*\(([^)]*)\)", text)
+        assert match, name
+        params = match.group(1).strip()
+        count = 0 if params in ("", "void") else len(params.split(","))
+        assert count == len(argtypes), (name, count, len(argtypes))
+
+
+def test_workspace_sizes_and_plan():
+    lib = _lib.library()
+    assert lib.tlce_compact_workspace_bytes(0) >= 4
+    assert lib.tlce_compact_workspace_bytes(32768) >= 32 * 4
+    assert lib.tlce_compact_workspace_bytes(-1) == -1
+    # headline shape: MFMA engine, 256 tiles, vocabulary panels bounded by 1 GiB
+    plan = _lib.query_plan(32768, 4096, 151936, _lib.DTYPE_BF16, True)
+    assert plan["engine"] == "mfma" and plan["tile"] == 256
+    assert plan["forward_vocab_splits"] == 8
+    assert plan["panel_columns"] % 256 == 0
+    assert plan["panel_columns"] * 32768 * 2 * 2 <= (1 << 30)
+    assert plan["n_panels"] * plan["panel_columns"] >= 151936
+    assert plan["grad_hidden_k_splits"] == 1
+    fwd = lib.tlce_forward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16)
+    assert fwd == 2 * 8 * 32768 * 4  # (max, sum) float32 partials only: no logits buffer
+    bwd = lib.tlce_backward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16, 1, 0, 0)
+    logits_bytes = 32768 * 151936 * 4
+    assert bwd < logits_bytes // 4
+    frozen = lib.tlce_backward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16, 0, 0, 0)
+    assert frozen < bwd
+    # few loss rows: the grad-hidden contraction splits K to fill the GPU
+    small = _lib.query_plan(1750, 4096, 151936, _lib.DTYPE_BF16, True)
+    assert small["n_panels"] <= 2 and small["grad_hidden_k_splits"] > 1
+    # float32 inputs and odd hidden sizes take the generic engine
+    assert _lib.query_plan(21, 33, 4097, _lib.DTYPE_F32, True)["engine"] == "generic"
+    assert _lib.query_plan(21, 33, 4097, _lib.DTYPE_BF16, True)["engine"] == "generic"
+    assert _lib.query_plan(31, 96, 1025, _lib.DTYPE_BF16, True)["engine"] == "mfma"
+    # a smaller panel budget means more panels
+    tight = _lib.query_plan(32768, 4096, 151936, _lib.DTYPE_BF16, True, 1 << 28)
+    assert tight["n_panels"] > plan["n_panels"]
+
+
+def test_bad_arguments_report_errors_without_a_gpu():
+    lib = _lib.library()
+    rc = lib.tlce_query_plan(1, 0, 5, _lib.DTYPE_BF16, 1, 0, None, None, None, None, None, None)
+    assert rc != 0 and "bad shape" in _lib.last_error()
+    with pytest.raises(RuntimeError, match="bad shape"):
+        _lib.check(rc, "tlce_query_plan")
+    assert lib.tlce_forward_workspace_bytes(-1, 8, 8, _lib.DTYPE_BF16) == -1

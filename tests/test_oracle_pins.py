@@ -1,0 +1,186 @@
+"""Pins the CPU oracle before anything is compared against it.
+
+Each oracle function is checked against something it does not itself call: a
+library routine (F.cross_entropy, autograd, torch.nonzero), a brute-force
+Python loop, a closed form, or the committed fixtures.  The cases are chosen so
+that a plausible slip (dropped bias, soft cap after the exclusion, onehot with
+the wrong sign, scale missing from mean, transposed grad_weight, ignored rows
+counted in the mean) fails at least one test.
+"""
+
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import linear_ce_oracle as oracle
+
+GOLDEN = Path(__file__).resolve().parent / "golden" / "linear_ce_cases.npz"
+
+
+def _golden_cases():
+    data = np.load(GOLDEN, allow_pickle=False)
+    for entry in data["__cases__"]:
+        name, softcap, exclude = str(entry).split("|")
+        softcap = float(softcap.split("=")[1])
+        exclude = int(exclude.split("=")[1])
+
+        def get(key, _name=name):
+            full = f"{_name}/{key}"
+            return torch.from_numpy(data[full]) if full in data.files else None
+
+        yield name, (softcap or None), (exclude if exclude >= 0 else None), get
+
+
+@pytest.mark.parametrize("reduction", ["none", "sum", "mean"])
+def test_oracle_matches_golden_fixtures(reduction):
+    seen = 0
+    for name, softcap, exclude, get in _golden_cases():
+        hidden, weight, labels, bias = get("hidden"), get("weight"), get("labels"), get("bias")
+        loss = oracle.dense_linear_ce(hidden, weight, labels, bias=bias, reduction=reduction,
+                                      exclude_index=exclude, logit_softcap=softcap)
+        torch.testing.assert_close(loss, get(f"loss_{reduction}"), atol=1e-11, rtol=1e-11,
+                                   msg=f"{name} loss")
+        go = get("grad_out") if reduction == "none" else None
+        dh, dw, db = oracle.dense_linear_ce_grads(
+            hidden, weight, labels, go, bias=bias, reduction=reduction, exclude_index=exclude,
+            logit_softcap=softcap)
+        torch.testing.assert_close(dh, get(f"dh_{reduction}"), atol=1e-11, rtol=1e-10)
+        torch.testing.assert_close(dw, get(f"dw_{reduction}"), atol=1e-11, rtol=1e-10)
+        if bias is not None:
+            torch.testing.assert_close(db, get(f"db_{reduction}"), atol=1e-11, rtol=1e-10)
+        seen += 1
+    assert seen == 6
+
+
+def test_oracle_matches_library_cross_entropy_and_autograd_bf16_inputs():
+    # the shape of the reference's bf16 device test (test_tiled_linear_cross_entropy.py:303-354)
+    torch.manual_seed(52)
+    hidden = (torch.randn(31, 96) * 0.1).bfloat16()
+    weight = (torch.randn(1025, 96) * 0.1).bfloat16()
+    bias = (torch.randn(1025) * 0.1).bfloat16()
+    labels = torch.randint(0, 1024, (31,))
+    labels[::5] = -100
+    h = hidden.double().requires_grad_(True)
+    w = weight.double().requires_grad_(True)
+    b = bias.double().requires_grad_(True)
+    logits = h @ w.t() + b
+    logits = logits + torch.zeros(1025, dtype=torch.float64).index_fill_(
+        0, torch.tensor([1024]), -float("inf"))
+    ref = F.cross_entropy(logits, labels, reduction="mean", ignore_index=-100)
+    ref.backward()
+    got = oracle.dense_linear_ce(hidden, weight, labels, bias=bias, exclude_index=1024)
+    torch.testing.assert_close(got, ref.detach(), atol=1e-12, rtol=1e-12)
+    dh, dw, db = oracle.dense_linear_ce_grads(hidden, weight, labels, bias=bias,
+                                              exclude_index=1024)
+    torch.testing.assert_close(dh, h.grad, atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(dw, w.grad, atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(db, b.grad, atol=1e-12, rtol=1e-10)
+    assert torch.count_nonzero(dw[1024]) == 0
+
+
+def test_oracle_brute_force_tiny():
+    torch.manual_seed(3)
+    n, h, v, cap, excl = 4, 3, 6, 1.5, 2
+    hidden = torch.randn(n, h, dtype=torch.float64)
+    weight = torch.randn(v, h, dtype=torch.float64)
+    bias = torch.randn(v, dtype=torch.float64)
+    labels = torch.tensor([0, -100, 5, 3])
+    expect = []
+    for r in range(n):
+        if labels[r] == -100:
+            expect.append(0.0)
+            continue
+        zs = []
+        for c in range(v):
+            z = sum(float(hidden[r, k]) * float(weight[c, k]) for k in range(h)) + float(bias[c])
+            zs.append(cap * math.tanh(z / cap))
+        denom = sum(math.exp(z) for c, z in enumerate(zs) if c != excl)
+        expect.append(math.log(denom) - zs[int(labels[r])])
+    got = oracle.dense_linear_ce(hidden, weight, labels, bias=bias, reduction="none",
+                                 exclude_index=excl, logit_softcap=cap)
+    torch.testing.assert_close(got, torch.tensor(expect, dtype=torch.float64), atol=1e-12,
+                               rtol=1e-12)
+    mean = oracle.dense_linear_ce(hidden, weight, labels, bias=bias, reduction="mean",
+                                  exclude_index=excl, logit_softcap=cap)
+    assert abs(float(mean) - sum(expect) / 3) < 1e-12  # ignored row not in the denominator
+
+
+def test_oracle_closed_forms():
+    # zero weights -> uniform softmax: loss = log V, and log(V-1) with one column excluded
+    hidden = torch.randn(5, 8, dtype=torch.float64)
+    weight = torch.zeros(17, 8, dtype=torch.float64)
+    labels = torch.tensor([0, 3, 16, 7, 9])
+    loss = oracle.dense_linear_ce(hidden, weight, labels, reduction="none")
+    torch.testing.assert_close(loss, torch.full((5,), math.log(17), dtype=torch.float64))
+    loss = oracle.dense_linear_ce(hidden, weight, labels.clamp(max=15), reduction="none",
+                                  exclude_index=16)
+    torch.testing.assert_close(loss, torch.full((5,), math.log(16), dtype=torch.float64))
+    # without soft cap every row of the logit gradient sums to zero -> grad_bias sums to 0
+    # and grad_hidden of a row equals sum_v g_v W_v
+    torch.manual_seed(1)
+    weight = torch.randn(17, 8, dtype=torch.float64)
+    bias = torch.randn(17, dtype=torch.float64)
+    _, _, db = oracle.dense_linear_ce_grads(hidden, weight, labels, bias=bias, reduction="sum")
+    assert abs(float(db.sum())) < 1e-12
+    # a saturated soft cap kills the gradient: |z| >> cap -> 1 - tanh^2 -> 0
+    dh, dw, _ = oracle.dense_linear_ce_grads(hidden * 1e4, weight, labels, reduction="sum",
+                                             logit_softcap=0.5)
+    assert float(dh.abs().max()) < 1e-9 and float(dw.abs().max()) < 1e-6
+    # lse >= max logit, and ignored rows contribute exactly nothing
+    labels2 = labels.clone()
+    labels2[1] = -100
+    loss, lse = oracle.dense_linear_ce(hidden, weight, labels2, reduction="none", return_lse=True)
+    assert float(loss[1]) == 0.0
+    assert bool((lse >= (hidden @ weight.t()).max(dim=-1).values).all())
+    dh, _, _ = oracle.dense_linear_ce_grads(hidden, weight, labels2, reduction="mean")
+    assert torch.count_nonzero(dh[1]) == 0
+
+
+@pytest.mark.parametrize("tile", [1, 5, 7, 64])
+def test_online_tiled_algorithm_is_tile_invariant(tile):
+    # tile sizes of test_tiled_linear_cross_entropy.py:172-219
+    torch.manual_seed(31)
+    hidden = torch.randn(15, 9, dtype=torch.float64)
+    weight = torch.randn(23, 9, dtype=torch.float64)
+    bias = torch.randn(23, dtype=torch.float64)
+    labels = torch.randint(0, 22, (15,))
+    labels[0] = -100
+    logits = hidden @ weight.t() + bias
+    logits[:, 22] = -float("inf")
+    ref = F.cross_entropy(logits, labels, reduction="none", ignore_index=-100)
+    losses, lse = oracle.online_tiled_linear_ce(hidden, weight, labels, vocab_block_size=tile,
+                                                bias=bias, exclude_index=22, dtype=torch.float64)
+    torch.testing.assert_close(losses, ref, atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(lse, torch.logsumexp(logits, dim=-1), atol=1e-12, rtol=1e-12)
+
+
+def test_rounded_logit_gradient_variant_stays_close_and_differs():
+    torch.manual_seed(11)
+    hidden = torch.randn(16, 32).bfloat16()
+    weight = (torch.randn(200, 32) * 0.1).bfloat16()
+    labels = torch.randint(0, 200, (16,))
+    exact = oracle.dense_linear_ce_grads(hidden, weight, labels, reduction="mean")
+    rounded = oracle.dense_linear_ce_grads(hidden, weight, labels, reduction="mean",
+                                           round_grad_logits=torch.bfloat16)
+    for a, e in zip(rounded[:2], exact[:2]):
+        err = oracle.relative_max_error(a, e)
+        assert 0.0 < err < 2e-2
+
+
+def test_compaction_oracle_matches_nonzero_and_loop():
+    rng = np.random.default_rng(5)
+    for n in (0, 1, 63, 64, 65, 1000, 4097):
+        labels = rng.integers(0, 50, size=n)
+        labels[rng.random(n) < 0.4] = -100
+        got = oracle.compact_rows(labels)
+        assert got.dtype == np.int64
+        ref = torch.nonzero(torch.from_numpy(labels) != -100).flatten().numpy()
+        np.testing.assert_array_equal(got, ref)
+        if n <= 1000:
+            assert got.tolist() == oracle.compact_rows_loop(labels)
+    assert oracle.compact_rows(np.full(10, -100)).size == 0
+    np.testing.assert_array_equal(oracle.compact_rows(np.arange(10)), np.arange(10))

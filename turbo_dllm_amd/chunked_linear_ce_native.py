@@ -1,0 +1,346 @@
+"""Python entry points of the gfx950 fused LM-head cross-entropy library.
+
+Same role and call signatures as the reference's binding shim
+(dllm_parallel/core/kernels/chunked_linear_ce_native.py:61-182): ``forward``,
+``backward`` and ``backward_frozen_weight`` take flattened tensors and return
+``(losses, lse, valid_count)`` / ``(grad_hidden, grad_weight, grad_bias)``.
+Added on top: the device compaction entry points (``compact_rows``,
+``gather_rows``, ``scatter_rows``) and the optional ``row_idx`` / ``n_out``
+arguments that let the kernels read compacted rows and write their results
+straight into the un-compacted token axis.
+
+torch is used here only to allocate outputs and workspaces on the caller's
+device and to hand over the current stream; all arithmetic runs in the HIP
+library through its C ABI.  There is no fallback: a missing library raises.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODES = {
+    torch.float32: _lib.DTYPE_F32,
+    torch.float16: _lib.DTYPE_F16,
+    torch.bfloat16: _lib.DTYPE_BF16,
+}
+
+# Upper bound, in bytes, of the logit-gradient staging panel of the backward
+# pass (0 selects the library default of 1 GiB).
+PANEL_BYTES = 0
+
+
+def _reduction_code(reduction: str) -> int:
+    # same numbering as chunked_linear_ce_native.py:366-373 of the reference
+    if reduction == "none":
+        return _lib.REDUCTION_NONE
+    if reduction == "sum":
+        return _lib.REDUCTION_SUM
+    if reduction == "mean":
+        return _lib.REDUCTION_MEAN
+    raise ValueError(f"unsupported reduction: {reduction}")
+
+
+def _dtype_code(tensor: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODES[tensor.dtype]
+    except KeyError as exc:
+        raise RuntimeError(
+            "native linear CE supports float32, float16, and bfloat16"
+        ) from exc
+
+
+def _ptr(tensor: Optional[torch.Tensor]) -> Optional[int]:
+    if tensor is None or tensor.numel() == 0:
+        return None
+    return tensor.data_ptr()
+
+
+def _stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_device(*tensors: Optional[torch.Tensor]) -> torch.device:
+    device = None
+    for tensor in tensors:
+        if tensor is None:
+            continue
+        if not tensor.is_cuda:
+            raise RuntimeError("native linear CE expects device (HIP) tensors")
+        if device is None:
+            device = tensor.device
+        elif tensor.device != device:
+            raise RuntimeError("native linear CE expects all tensors on one device")
+    assert device is not None
+    return device
+
+
+def _workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    # torch's caching allocator hands out 512-byte aligned blocks
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def verify_device(device: torch.device | int | None = None) -> None:
+    """Raises unless the device is a gfx950 GPU the library has code for."""
+    index = torch.cuda.current_device() if device is None else torch.device(device).index
+    _lib.check(_lib.library().tlce_check_device(int(index or 0)), "tlce_check_device")
+
+
+# ----------------------------------------------------------------- compaction --
+def compact_rows(labels: torch.Tensor, ignore_index: int) -> tuple[torch.Tensor, int]:
+    """``nonzero(labels != ignore_index).flatten()`` on the device.
+
+    Returns the ascending int64 indices (a view of length ``count``) and the
+    count.  Reading the count back is the one host synchronisation of the
+    path, the same one the reference incurs at ``row_indices.numel()``
+    (nemotron/model.py:4244-4248).
+    """
+    device = _require_device(labels)
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    n = labels.numel()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        row_idx = torch.empty(max(n, 1), dtype=torch.long, device=device)
+        count = torch.empty(1, dtype=torch.long, device=device)
+        ws = _workspace(lib.tlce_compact_workspace_bytes(n), device)
+        _lib.check(
+            lib.tlce_compact_rows(
+                _ptr(labels), n, int(ignore_index), row_idx.data_ptr(), count.data_ptr(),
+                ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_compact_rows",
+        )
+        m = int(count.item())
+    return row_idx[:m], m
+
+
+def gather_rows(src: torch.Tensor, row_idx: torch.Tensor) -> torch.Tensor:
+    """``src.index_select(0, row_idx)`` for a contiguous ``src`` (any trailing shape)."""
+    device = _require_device(src, row_idx)
+    src = src.contiguous()
+    m = row_idx.numel()
+    out = torch.empty((m, *src.shape[1:]), dtype=src.dtype, device=device)
+    if m == 0 or src.numel() == 0:
+        return out
+    row_bytes = src.element_size() * (src.numel() // src.shape[0])
+    with torch.cuda.device(device):
+        _lib.check(
+            _lib.library().tlce_gather_rows(
+                src.data_ptr(), row_idx.data_ptr(), m, row_bytes, out.data_ptr(), _stream(device)
+            ),
+            "tlce_gather_rows",
+        )
+    return out
+
+
+def scatter_rows(src: torch.Tensor, row_idx: torch.Tensor, n_rows: int) -> torch.Tensor:
+    """Zero tensor of ``n_rows`` rows with ``out[row_idx[r]] = src[r]``."""
+    device = _require_device(src, row_idx)
+    src = src.contiguous()
+    out = torch.empty((n_rows, *src.shape[1:]), dtype=src.dtype, device=device)
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        if out.numel():
+            _lib.check(
+                lib.tlce_fill_zero(out.data_ptr(), out.numel() * out.element_size(),
+                                   _stream(device)),
+                "tlce_fill_zero",
+            )
+        m = row_idx.numel()
+        if m and src.numel():
+            row_bytes = src.element_size() * (src.numel() // src.shape[0])
+            _lib.check(
+                lib.tlce_scatter_rows(
+                    src.data_ptr(), row_idx.data_ptr(), m, row_bytes, out.data_ptr(),
+                    _stream(device),
+                ),
+                "tlce_scatter_rows",
+            )
+    return out
+
+
+# -------------------------------------------------------------------- forward --
+def _vocab_first(weight: torch.Tensor, weight_dim_first: bool) -> torch.Tensor:
+    # The kernels read the head as [V, H]; a [H, V] head is re-laid once here.
+    return weight.t().contiguous() if weight_dim_first else weight.contiguous()
+
+
+def forward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    labels: torch.Tensor,
+    *,
+    row_block_size: int,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+    compute_dtype: torch.dtype,
+    weight_dim_first: bool,
+    row_idx: torch.Tensor | None = None,
+    n_out: int | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Returns ``(losses [n_out] f32, lse [m] f32, valid_count [1] f32)``.
+
+    ``row_block_size`` and ``compute_dtype`` are accepted for signature parity
+    and ignored, as in the reference shim (chunked_linear_ce_native.py:61-94):
+    tiling is fixed by the library's plan, arithmetic is in the input dtype
+    with float32 accumulation.
+    """
+    del row_block_size, compute_dtype
+    device = _require_device(hidden, weight, bias, labels, row_idx)
+    if hidden.dim() != 2:
+        raise RuntimeError("hidden must be flattened [N, D]")
+    if weight.dim() != 2:
+        raise RuntimeError("weight must be a matrix")
+    if weight.dtype != hidden.dtype:
+        raise RuntimeError("native linear CE expects hidden and weight of one dtype")
+    hidden = hidden.contiguous()
+    weight = _vocab_first(weight, weight_dim_first)
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v = weight.shape[0]
+    if weight.shape[1] != h or labels.numel() != m:
+        raise RuntimeError("native linear CE shape mismatch")
+    n_out = m if n_out is None else int(n_out)
+    bias32 = None if bias is None else bias.to(torch.float32).contiguous()
+    if bias32 is not None and bias32.numel() != v:
+        raise RuntimeError("native linear CE bias shape mismatch")
+    lib = _lib.library()
+    code = _dtype_code(hidden)
+    with torch.cuda.device(device):
+        losses = torch.empty(n_out, dtype=torch.float32, device=device)
+        lse = torch.empty(m, dtype=torch.float32, device=device)
+        valid_count = torch.empty(1, dtype=torch.float32, device=device)
+        ws = _workspace(lib.tlce_forward_workspace_bytes(m, h, v, code), device)
+        _lib.check(
+            lib.tlce_forward(
+                _ptr(hidden), _ptr(weight), _ptr(bias32), _ptr(labels), _ptr(row_idx),
+                m, n_out, h, v, code,
+                int(ignore_index), int(exclude_index), float(logit_softcap),
+                _ptr(losses), _ptr(lse), valid_count.data_ptr(),
+                ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_forward",
+        )
+    return losses, lse, valid_count
+
+
+# ------------------------------------------------------------------- backward --
+def _backward(
+    hidden, weight, bias, labels, lse, valid_count, grad_output, *,
+    reduction, ignore_index, exclude_index, logit_softcap, weight_dim_first,
+    compute_weight_grad, row_idx, n_out,
+):
+    device = _require_device(hidden, weight, bias, labels, lse, valid_count, grad_output, row_idx)
+    hidden = hidden.contiguous()
+    weight_vf = _vocab_first(weight, weight_dim_first)
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v = weight_vf.shape[0]
+    n_out = m if n_out is None else int(n_out)
+    code = _dtype_code(hidden)
+    reduction_code = _reduction_code(reduction)
+    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
+    expected = n_out if reduction_code == _lib.REDUCTION_NONE else 1
+    if grad_output.numel() != expected:
+        raise RuntimeError(
+            f"grad_output has {grad_output.numel()} elements, expected {expected}"
+        )
+    bias32 = None if bias is None else bias.to(torch.float32).contiguous()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        grad_hidden = torch.empty((n_out, h), dtype=hidden.dtype, device=device)
+        grad_weight = (
+            torch.empty((v, h), dtype=weight.dtype, device=device) if compute_weight_grad else None
+        )
+        grad_bias32 = (
+            torch.empty(v, dtype=torch.float32, device=device) if bias is not None else None
+        )
+        ws = _workspace(
+            lib.tlce_backward_workspace_bytes(
+                m, h, v, code, int(compute_weight_grad), int(bias is not None), PANEL_BYTES
+            ),
+            device,
+        )
+        _lib.check(
+            lib.tlce_backward(
+                _ptr(hidden), _ptr(weight_vf), _ptr(bias32), _ptr(labels), _ptr(row_idx),
+                _ptr(lse), valid_count.data_ptr(), _ptr(grad_output),
+                m, n_out, h, v, code,
+                reduction_code, int(ignore_index), int(exclude_index), float(logit_softcap),
+                _ptr(grad_hidden), _ptr(grad_weight), _ptr(grad_bias32),
+                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_backward",
+        )
+    if grad_weight is None:
+        grad_weight = torch.empty(0, dtype=weight.dtype, device=device)
+    elif weight_dim_first:
+        grad_weight = grad_weight.t().contiguous()
+    if grad_bias32 is None:
+        grad_bias = torch.empty(0, dtype=torch.float32, device=device)
+    else:
+        grad_bias = grad_bias32.to(bias.dtype)
+    return grad_hidden, grad_weight, grad_bias
+
+
+def backward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    labels: torch.Tensor,
+    lse: torch.Tensor,
+    valid_count: torch.Tensor,
+    grad_output: torch.Tensor,
+    *,
+    row_block_size: int,
+    reduction: str,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+    compute_dtype: torch.dtype,
+    weight_dim_first: bool,
+    row_idx: torch.Tensor | None = None,
+    n_out: int | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(grad_hidden [n_out, H], grad_weight, grad_bias)`` in the input dtypes."""
+    del row_block_size, compute_dtype
+    return _backward(
+        hidden, weight, bias, labels, lse, valid_count, grad_output,
+        reduction=reduction, ignore_index=ignore_index, exclude_index=exclude_index,
+        logit_softcap=logit_softcap, weight_dim_first=weight_dim_first,
+        compute_weight_grad=True, row_idx=row_idx, n_out=n_out,
+    )
+
+
+def backward_frozen_weight(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    labels: torch.Tensor,
+    lse: torch.Tensor,
+    valid_count: torch.Tensor,
+    grad_output: torch.Tensor,
+    *,
+    row_block_size: int,
+    reduction: str,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+    compute_dtype: torch.dtype,
+    weight_dim_first: bool,
+    row_idx: torch.Tensor | None = None,
+    n_out: int | None = None,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """As ``backward`` with the weight-gradient contraction skipped (empty dW)."""
+    del row_block_size, compute_dtype
+    return _backward(
+        hidden, weight, bias, labels, lse, valid_count, grad_output,
+        reduction=reduction, ignore_index=ignore_index, exclude_index=exclude_index,
+        logit_softcap=logit_softcap, weight_dim_first=weight_dim_first,
+        compute_weight_grad=False, row_idx=row_idx, n_out=n_out,
+    )

@@ -1,0 +1,105 @@
+// Shared host/device helpers for the gfx950 fused linear cross-entropy library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+#include <string.h>
+
+#include <algorithm>
+
+#include "../../include/tlce.h"
+
+namespace tlce {
+
+// ---------------------------------------------------------------- errors ----
+// Thread-local message buffer behind tlce_last_error().  The reference raises
+// through TORCH_CHECK (fused_linear_ce.cpp:107-111); here every entry point
+// returns a code and leaves the text for the host binding to raise.
+char* error_buffer();
+int fail(const char* fmt, ...);
+
+#define TLCE_HIP(expr)                                                        \
+  do {                                                                        \
+    hipError_t tlce_err__ = (expr);                                           \
+    if (tlce_err__ != hipSuccess) {                                           \
+      return ::tlce::fail("%s failed: %s (%s:%d)", #expr,                     \
+                          hipGetErrorString(tlce_err__), __FILE__, __LINE__); \
+    }                                                                         \
+  } while (0)
+
+#define TLCE_REQUIRE(cond, ...)           \
+  do {                                    \
+    if (!(cond)) {                        \
+      return ::tlce::fail(__VA_ARGS__);   \
+    }                                     \
+  } while (0)
+
+#define TLCE_LAUNCH_CHECK() TLCE_HIP(hipGetLastError())
+
+// ----------------------------------------------------------------- sizes ----
+static inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+static inline int64_t ceil_div(int64_t x, int64_t m) { return (x + m - 1) / m; }
+static inline int64_t align256(int64_t x) { return round_up(x, 256); }
+
+static inline int dtype_bytes(int dtype) { return dtype == TLCE_DTYPE_F32 ? 4 : 2; }
+
+constexpr int kXcds = 8;  // MI355X: 8 accelerator dies, workgroups dealt round-robin
+
+// ------------------------------------------------------------- device -------
+#define TLCE_LOG2E 1.4426950408889634f
+#define TLCE_LN2 0.6931471805599453f
+
+// Workgroups are dealt to the 8 XCDs round-robin by blockIdx; each XCD has its
+// own L2.  Map the hardware block id to a logical id so that one XCD works on
+// a contiguous range of logical ids (launch grids are multiples of 8).
+__device__ __forceinline__ int xcd_logical_block(int bid, int nblocks) {
+  const int per = nblocks / kXcds;
+  return (bid % kXcds) * per + (bid / kXcds);
+}
+
+// Grouped tile order: consecutive logical ids walk `group` tiles along i, then
+// step j, so the ~32 workgroups resident on one XCD cover a group x (32/group)
+// block of tiles and share both operands through that XCD's L2.
+__device__ __forceinline__ void grouped_tile(int logical, int ni, int nj, int group,
+                                             int* ti, int* tj) {
+  const int width = group * nj;
+  const int gid = logical / width;
+  const int first = gid * group;
+  const int gsize = min(ni - first, group);
+  const int within = logical - gid * width;
+  *ti = first + within % gsize;
+  *tj = within / gsize;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+// tanh(x) = 1 - 2 / (1 + e^{2x}); saturates cleanly to +-1 for large |x|.
+__device__ __forceinline__ float fast_tanh(float x) {
+  const float e = fast_exp2(x * (2.0f * TLCE_LOG2E));
+  return 1.0f - 2.0f * fast_rcp(1.0f + e);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+template <typename T>
+__device__ __forceinline__ float to_float(T x) { return static_cast<float>(x); }
+template <typename T>
+__device__ __forceinline__ T from_float(float x) { return static_cast<T>(x); }
+
+// Host-side launch grid: a multiple of 8 so xcd_logical_block is a bijection.
+static inline int xcd_grid(int64_t tiles) { return (int)round_up(tiles, kXcds); }
+
+}  // namespace tlce

@@ -1,0 +1,203 @@
+// Masked-position compaction and row gather/scatter for gfx950.
+//
+// Device counterpart of `_compact_valid_loss_rows`
+// (dllm_parallel/core/models/backbones/nemotron/model.py:4234-4253):
+//   row_idx = nonzero(labels != ignore_index)   (ascending int64)
+//   hidden_c = hidden.index_select(0, row_idx), labels_c = labels.index_select(0, row_idx)
+// Two passes over the labels (8 bytes each): a ballot/popcount per 1024-label
+// block, then each block sums the counts before it and writes its indices at
+// wave-ballot prefix positions.  No spin-waits between blocks: the passes are
+// separate launches.
+#include "tlce_common.h"
+
+namespace tlce {
+
+constexpr int kCompactThreads = 256;
+constexpr int kCompactItems = 4;
+constexpr int kCompactBlock = kCompactThreads * kCompactItems;  // labels per block
+
+__global__ __launch_bounds__(kCompactThreads) void compact_count_kernel(
+    const int64_t* __restrict__ labels, int64_t n, int64_t ignore, int* __restrict__ block_counts) {
+  __shared__ int wave_counts[kCompactThreads / 64];
+  const int64_t base = (int64_t)blockIdx.x * kCompactBlock;
+  int count = 0;
+#pragma unroll
+  for (int q = 0; q < kCompactItems; ++q) {
+    const int64_t i = base + q * kCompactThreads + threadIdx.x;
+    const bool keep = (i < n) && (labels[i] != ignore);
+    count += __popcll(__ballot(keep));  // wave-uniform
+  }
+  if ((threadIdx.x & 63) == 0) wave_counts[threadIdx.x >> 6] = count;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int total = 0;
+#pragma unroll
+    for (int w = 0; w < kCompactThreads / 64; ++w) total += wave_counts[w];
+    block_counts[blockIdx.x] = total;
+  }
+}
+
+__global__ __launch_bounds__(kCompactThreads) void compact_write_kernel(
+    const int64_t* __restrict__ labels, int64_t n, int64_t ignore,
+    const int* __restrict__ block_counts, int64_t* __restrict__ row_idx,
+    int64_t* __restrict__ count_out) {
+  constexpr int kWaves = kCompactThreads / 64;
+  __shared__ int64_t wave_partial[kWaves];
+  __shared__ int slot_counts[kCompactItems * kWaves];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+
+  // exclusive prefix of the block counts before this block
+  int64_t before = 0;
+  for (int b = threadIdx.x; b < (int)blockIdx.x; b += kCompactThreads) before += block_counts[b];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o, 64);
+  if (lane == 0) wave_partial[wave] = before;
+
+  const int64_t base = (int64_t)blockIdx.x * kCompactBlock;
+  bool keep[kCompactItems];
+  int rank[kCompactItems];
+#pragma unroll
+  for (int q = 0; q < kCompactItems; ++q) {
+    const int64_t i = base + q * kCompactThreads + threadIdx.x;
+    keep[q] = (i < n) && (labels[i] != ignore);
+    const unsigned long long mask = __ballot(keep[q]);
+    rank[q] = __popcll(mask & ((1ull << lane) - 1ull));
+    if (lane == 0) slot_counts[q * kWaves + wave] = __popcll(mask);
+  }
+  __syncthreads();
+
+  int64_t block_offset = 0;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) block_offset += wave_partial[w];
+
+  int running = 0;
+#pragma unroll
+  for (int q = 0; q < kCompactItems; ++q) {
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      if (w == wave && keep[q]) {
+        const int64_t i = base + q * kCompactThreads + threadIdx.x;
+        row_idx[block_offset + running + rank[q]] = i;
+      }
+      running += slot_counts[q * kWaves + w];
+    }
+  }
+  if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) count_out[0] = block_offset + running;
+}
+
+template <typename V>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const V* __restrict__ src,
+                                                          const int64_t* __restrict__ row_idx,
+                                                          int64_t total, int vecs_per_row,
+                                                          V* __restrict__ dst) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const int64_t r = e / vecs_per_row;
+    const int c = (int)(e - r * vecs_per_row);
+    dst[e] = src[row_idx[r] * vecs_per_row + c];
+  }
+}
+
+template <typename V>
+__global__ __launch_bounds__(256) void scatter_rows_kernel(const V* __restrict__ src,
+                                                           const int64_t* __restrict__ row_idx,
+                                                           int64_t total, int vecs_per_row,
+                                                           V* __restrict__ dst) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+    const int64_t r = e / vecs_per_row;
+    const int c = (int)(e - r * vecs_per_row);
+    dst[row_idx[r] * vecs_per_row + c] = src[e];
+  }
+}
+
+static int pick_vector_bytes(const void* a, const void* b, int64_t row_bytes) {
+  const uintptr_t bits = (uintptr_t)a | (uintptr_t)b | (uintptr_t)row_bytes;
+  if ((bits & 15) == 0) return 16;
+  if ((bits & 7) == 0) return 8;
+  if ((bits & 3) == 0) return 4;
+  if ((bits & 1) == 0) return 2;
+  return 1;
+}
+
+static int move_grid(int64_t total) {
+  return (int)std::min<int64_t>(ceil_div(total, 256), 256 * 32);
+}
+
+template <bool kGather>
+static int move_rows(const void* src, const int64_t* row_idx, int64_t m, int64_t row_bytes,
+                     void* dst, hipStream_t stream) {
+  TLCE_REQUIRE(m >= 0 && row_bytes >= 0, "row move: negative size");
+  if (m == 0 || row_bytes == 0) return 0;
+  TLCE_REQUIRE(src && dst && row_idx, "row move: null pointer");
+  const int vb = pick_vector_bytes(src, dst, row_bytes);
+  const int64_t vpr = row_bytes / vb;
+  TLCE_REQUIRE(vpr <= INT32_MAX, "row move: row too long");
+  const int64_t total = m * vpr;
+  const int grid = move_grid(total);
+#define TLCE_MOVE(V)                                                                        \
+  do {                                                                                      \
+    if (kGather)                                                                            \
+      gather_rows_kernel<V><<<grid, 256, 0, stream>>>((const V*)src, row_idx, total,        \
+                                                      (int)vpr, (V*)dst);                   \
+    else                                                                                    \
+      scatter_rows_kernel<V><<<grid, 256, 0, stream>>>((const V*)src, row_idx, total,       \
+                                                       (int)vpr, (V*)dst);                  \
+  } while (0)
+  switch (vb) {
+    case 16: TLCE_MOVE(uint4); break;
+    case 8: TLCE_MOVE(uint2); break;
+    case 4: TLCE_MOVE(uint32_t); break;
+    case 2: TLCE_MOVE(uint16_t); break;
+    default: TLCE_MOVE(uint8_t); break;
+  }
+#undef TLCE_MOVE
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace tlce
+
+using namespace tlce;
+
+extern "C" int64_t tlce_compact_workspace_bytes(int64_t n) {
+  if (n < 0) return -1;
+  return align256(ceil_div(std::max<int64_t>(n, 1), kCompactBlock) * (int64_t)sizeof(int));
+}
+
+extern "C" int tlce_compact_rows(const int64_t* labels, int64_t n, int64_t ignore_index,
+                                 int64_t* row_idx_out, int64_t* count_out, void* workspace,
+                                 int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  TLCE_REQUIRE(n >= 0 && n < (int64_t)INT32_MAX, "compact: n=%lld out of range", (long long)n);
+  TLCE_REQUIRE(count_out != nullptr, "compact: count_out is null");
+  if (n == 0) {
+    // count = 0 through the fill kernel so the call stays capturable
+    return tlce_fill_zero(count_out, sizeof(int64_t), stream_);
+  }
+  TLCE_REQUIRE(labels && row_idx_out && workspace, "compact: null pointer");
+  TLCE_REQUIRE(workspace_bytes >= tlce_compact_workspace_bytes(n),
+               "compact: workspace too small (%lld < %lld)", (long long)workspace_bytes,
+               (long long)tlce_compact_workspace_bytes(n));
+  const int blocks = (int)ceil_div(n, kCompactBlock);
+  int* block_counts = static_cast<int*>(workspace);
+  compact_count_kernel<<<blocks, kCompactThreads, 0, stream>>>(labels, n, ignore_index,
+                                                               block_counts);
+  TLCE_LAUNCH_CHECK();
+  compact_write_kernel<<<blocks, kCompactThreads, 0, stream>>>(labels, n, ignore_index,
+                                                               block_counts, row_idx_out,
+                                                               count_out);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int tlce_gather_rows(const void* src, const int64_t* row_idx, int64_t m,
+                                int64_t row_bytes, void* dst, void* stream) {
+  return move_rows<true>(src, row_idx, m, row_bytes, dst, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlce_scatter_rows(const void* src, const int64_t* row_idx, int64_t m,
+                                 int64_t row_bytes, void* dst, void* stream) {
+  return move_rows<false>(src, row_idx, m, row_bytes, dst, static_cast<hipStream_t>(stream));
+}

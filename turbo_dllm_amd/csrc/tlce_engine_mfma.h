@@ -1,0 +1,191 @@
+// 256x256x64 bf16/f16 MFMA tile engine for gfx950 (CDNA4), wave64.
+//
+// Computes C[i][j] = sum_k A[i][k] * B[j][k] for one 256x256 tile, A and B both
+// K-contiguous (row-major [rows, K]).  512 threads = 8 waves in a 2 (A rows) x
+// 4 (B rows) grid; each wave owns a 128x64 sub-tile as 4x2
+// v_mfma_f32_32x32x16 blocks (128 fp32 accumulator registers per lane), two
+// waves per SIMD.
+//
+// LDS: two stages of (A 256x64 + B 256x64) 2-byte elements = 2 x 64 KiB of the
+// CU's 160 KiB.  A tile row is 128 bytes = eight 16-byte chunks; chunk c of
+// row r lives at chunk slot c ^ ((r >> 1) & 7), which makes both the 16-byte
+// staging writes and the 16-byte MFMA fragment reads hit all 64 banks.
+//
+// Accumulator layout of one 32x32 block (lane l, register q of 16):
+//   row = 8*(q/4) + 4*(l/32) + q%4,   col = l%32.
+// A/B fragment of one block for K-slice ks: lane l supplies row l%32,
+// K = 16*ks + 8*(l/32) .. +8  (one 16-byte chunk).
+#pragma once
+
+#include "tlce_common.h"
+
+namespace tlce {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+template <typename T> struct MfmaOp;
+template <> struct MfmaOp<__bf16> {
+  using V8 = bf16x8_t;
+  static __device__ __forceinline__ f32x16_t mma(V8 a, V8 b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct MfmaOp<_Float16> {
+  using V8 = f16x8_t;
+  static __device__ __forceinline__ f32x16_t mma(V8 a, V8 b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+template <typename T_>
+struct MfmaEngine {
+  using T = T_;
+  using Op = MfmaOp<T>;
+  using V8 = typename Op::V8;
+
+  static constexpr int kTile = 256;     // BM == BN
+  static constexpr int kBK = 64;
+  static constexpr int kThreads = 512;
+  static constexpr int kWavesN = 4;     // waves along B rows
+  static constexpr int kTM = 4;         // 32-row blocks per wave along A rows
+  static constexpr int kTN = 2;         // 32-col blocks per wave along B rows
+  static constexpr int kRowBytes = kBK * 2;                  // 128
+  static constexpr int kStageBytes = 2 * kTile * kRowBytes;  // 65536
+  static constexpr int kSmemBytes = 2 * kStageBytes;         // 131072
+  static constexpr int kCols = kTN;          // tile columns owned per thread
+  static constexpr int kRows = kTM * 16;     // tile rows held per owned column
+  static constexpr int kShare = 4;           // threads that hold the same column
+
+  struct Acc { f32x16_t c[kTM][kTN]; };
+
+  int lane, wm, wn;
+
+  __device__ __forceinline__ MfmaEngine() {
+    lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    wm = wave / kWavesN;
+    wn = wave % kWavesN;
+  }
+
+  __device__ __forceinline__ int col(int j) const { return wn * 64 + j * 32 + (lane & 31); }
+  __device__ __forceinline__ int row(int i) const {
+    return wm * 128 + (i >> 4) * 32 + ((i >> 2) & 3) * 8 + (lane >> 5) * 4 + (i & 3);
+  }
+  __device__ __forceinline__ int share_slot() const { return wm * 2 + (lane >> 5); }
+  static __device__ __forceinline__ float get(const Acc& a, int j, int i) {
+    return a.c[i >> 4][j][i & 15];
+  }
+  static __device__ __forceinline__ void set(Acc& a, int j, int i, float v) {
+    a.c[i >> 4][j][i & 15] = v;
+  }
+  static __device__ __forceinline__ void zero(Acc& a) {
+#pragma unroll
+    for (int tm = 0; tm < kTM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < kTN; ++tn)
+#pragma unroll
+        for (int q = 0; q < 16; ++q) a.c[tm][tn][q] = 0.0f;
+  }
+  // Sum over the lanes that hold the same tile row (the 32 lanes of a half-wave).
+  __device__ __forceinline__ float reduce_over_cols(float v) const {
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+  }
+  __device__ __forceinline__ bool col_leader() const { return (lane & 31) == 0; }
+
+  // acc += A[a_row0 .. +256, k_begin .. k_end) * B[b_row0 .. +256, same K)^T.
+  // Rows past a_rows / b_rows are clamped to the last valid row (their results
+  // are discarded by the caller); K past k_end is zero-filled.  k_begin and
+  // k_end are multiples of 8 and lda/ldb multiples of 8 (16-byte chunks).
+  __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
+                                           int a_rows, const T* __restrict__ B, int64_t ldb,
+                                           int b_row0, int b_rows, int k_begin, int k_end,
+                                           Acc& acc, char* smem) const {
+    const int tid = threadIdx.x;
+    const int c = tid & 7;
+    const int r0 = tid >> 3;
+    const int pc = c ^ ((tid >> 4) & 7);
+
+    const T* ap[4];
+    const T* bp[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int ar = min(a_row0 + r0 + 64 * j, a_rows - 1);
+      const int br = min(b_row0 + r0 + 64 * j, b_rows - 1);
+      ap[j] = A + (int64_t)ar * lda + k_begin + c * 8;
+      bp[j] = B + (int64_t)br * ldb + k_begin + c * 8;
+    }
+    const int st_off = r0 * kRowBytes + pc * 16;
+
+    const int swz = (lane >> 1) & 7;
+    const int hi = lane >> 5;
+    const int a_frag = (wm * 128 + (lane & 31)) * kRowBytes;
+    const int b_frag = kTile * kRowBytes + (wn * 64 + (lane & 31)) * kRowBytes;
+
+    uint4 ra[4], rb[4];
+
+    // A chunk past k_end re-reads the row's first chunk (always in bounds) and
+    // is zeroed in registers, so the loads stay unconditional global loads.
+    auto gload = [&](int k0) {
+      const bool ok = (k0 + c * 8) < k_end;
+      const int64_t back = ok ? 0 : (int64_t)(k0 - k_begin + c * 8);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        ra[j] = *reinterpret_cast<const uint4*>(ap[j] - back);
+        rb[j] = *reinterpret_cast<const uint4*>(bp[j] - back);
+        if (!ok) {
+          ra[j] = make_uint4(0u, 0u, 0u, 0u);
+          rb[j] = make_uint4(0u, 0u, 0u, 0u);
+        }
+        ap[j] += kBK;
+        bp[j] += kBK;
+      }
+    };
+    auto sstore = [&](int stage) {
+      char* base = smem + stage * kStageBytes + st_off;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        *reinterpret_cast<uint4*>(base + j * 64 * kRowBytes) = ra[j];
+        *reinterpret_cast<uint4*>(base + kTile * kRowBytes + j * 64 * kRowBytes) = rb[j];
+      }
+    };
+    auto compute = [&](int stage) {
+      const char* base = smem + stage * kStageBytes;
+#pragma unroll
+      for (int ks = 0; ks < kBK / 16; ++ks) {
+        const int slot = ((2 * ks + hi) ^ swz) * 16;
+        V8 af[kTM], bf[kTN];
+#pragma unroll
+        for (int tm = 0; tm < kTM; ++tm)
+          af[tm] = __builtin_bit_cast(
+              V8, *reinterpret_cast<const uint4*>(base + a_frag + tm * 32 * kRowBytes + slot));
+#pragma unroll
+        for (int tn = 0; tn < kTN; ++tn)
+          bf[tn] = __builtin_bit_cast(
+              V8, *reinterpret_cast<const uint4*>(base + b_frag + tn * 32 * kRowBytes + slot));
+#pragma unroll
+        for (int tm = 0; tm < kTM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < kTN; ++tn) acc.c[tm][tn] = Op::mma(af[tm], bf[tn], acc.c[tm][tn]);
+      }
+    };
+
+    const int nk = (k_end - k_begin + kBK - 1) / kBK;
+    gload(k_begin);
+    sstore(0);
+    __syncthreads();
+    for (int it = 0; it < nk; ++it) {
+      const int cur = it & 1;
+      const bool more = (it + 1) < nk;
+      if (more) gload(k_begin + (it + 1) * kBK);
+      compute(cur);
+      if (more) sstore(cur ^ 1);
+      __syncthreads();
+    }
+  }
+};
+
+}  // namespace tlce

@@ -1,0 +1,461 @@
+// Device kernels of the fused linear cross-entropy, templated on a tile engine
+// (MfmaEngine for bf16/f16, SimtEngine for the generic float32-FMA path).
+//
+// Orientation used by every logits tile: the engine's "A rows" are vocabulary
+// rows of the LM head and its "B rows" are token rows of hidden, i.e. a tile is
+// logits^T[vocab, token].  A thread then owns a few token columns and holds many
+// vocabulary entries of each in registers, so the softmax reductions over the
+// vocabulary are in-lane and need no cross-lane traffic inside the tile loop.
+#pragma once
+
+#include "tlce_common.h"
+
+namespace tlce {
+
+// ------------------------------------------------------------------ forward --
+// Per (token tile, vocabulary split): stream the split's vocabulary tiles,
+// keeping a running (max, sum-exp) per token in registers (base-2 domain), and
+// write one partial per token.  Math follows ce_forward_kernel
+// (fused_linear_ce_cuda.cu:156-224): bias add, tanh soft cap, excluded column
+// skipped, but as an online single pass instead of two passes over stored
+// logits.
+struct ForwardArgs {
+  const void* hidden;   // [m, h]
+  const void* weight;   // [v, h]
+  const float* bias;    // [v] or null
+  int m, h, v;
+  int64_t exclude;
+  float softcap;
+  int n_ttiles, n_vtiles, nsplit;
+  float* part_max;      // [nsplit, part_ld]  base-2 running max
+  float* part_sum;      // [nsplit, part_ld]
+  int part_ld;
+};
+
+template <class E, bool kSoftcap, bool kBias>
+__global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardArgs p) {
+  extern __shared__ __align__(16) char smem[];
+  using T = typename E::T;
+  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
+  if (logical >= p.n_ttiles * p.nsplit) return;
+  int tt, vs;
+  grouped_tile(logical, p.n_ttiles, p.nsplit, 4, &tt, &vs);
+  const int vt0 = (int)((int64_t)vs * p.n_vtiles / p.nsplit);
+  const int vt1 = (int)((int64_t)(vs + 1) * p.n_vtiles / p.nsplit);
+
+  E eng;
+  const T* hidden = static_cast<const T*>(p.hidden);
+  const T* weight = static_cast<const T*>(p.weight);
+  const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
+
+  float run_max[E::kCols], run_sum[E::kCols];
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    run_max[j] = -INFINITY;
+    run_sum[j] = 0.0f;
+  }
+
+  for (int vt = vt0; vt < vt1; ++vt) {
+    typename E::Acc acc;
+    E::zero(acc);
+    eng.mainloop(weight, p.h, vt * E::kTile, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc,
+                 smem);
+    const int vbase = vt * E::kTile;
+    if (kBias) {
+#pragma unroll
+      for (int i = 0; i < E::kRows; ++i) {
+        const float b = p.bias[min(vbase + eng.row(i), p.v - 1)];
+#pragma unroll
+        for (int j = 0; j < E::kCols; ++j) E::set(acc, j, i, E::get(acc, j, i) + b);
+      }
+    }
+    // logits -> base-2 scaled, masked entries -> -inf
+#pragma unroll
+    for (int i = 0; i < E::kRows; ++i) {
+      const int v = vbase + eng.row(i);
+      const bool ok = (v < p.v) && (v != p.exclude);
+#pragma unroll
+      for (int j = 0; j < E::kCols; ++j) {
+        float z = E::get(acc, j, i);
+        if (kSoftcap) z = p.softcap * fast_tanh(z * inv_cap);
+        E::set(acc, j, i, ok ? z * TLCE_LOG2E : -INFINITY);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      float tile_max = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < E::kRows; ++i) tile_max = fmaxf(tile_max, E::get(acc, j, i));
+      const float new_max = fmaxf(run_max[j], tile_max);
+      if (new_max > -INFINITY) {
+        float s = run_sum[j] * fast_exp2(run_max[j] - new_max);
+#pragma unroll
+        for (int i = 0; i < E::kRows; ++i) s += fast_exp2(E::get(acc, j, i) - new_max);
+        run_sum[j] = s;
+        run_max[j] = new_max;
+      }
+    }
+  }
+
+  // merge the kShare threads that hold the same token column
+  float* sh_max = reinterpret_cast<float*>(smem);
+  float* sh_sum = sh_max + E::kShare * E::kTile;
+  const int slot = eng.share_slot();
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    sh_max[slot * E::kTile + eng.col(j)] = run_max[j];
+    sh_sum[slot * E::kTile + eng.col(j)] = run_sum[j];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < E::kTile; c += E::kThreads) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < E::kShare; ++s) mx = fmaxf(mx, sh_max[s * E::kTile + c]);
+    float sum = 0.0f;
+    if (mx > -INFINITY) {
+#pragma unroll
+      for (int s = 0; s < E::kShare; ++s)
+        sum += sh_sum[s * E::kTile + c] * fast_exp2(sh_max[s * E::kTile + c] - mx);
+    }
+    const int64_t o = (int64_t)vs * p.part_ld + tt * E::kTile + c;
+    p.part_max[o] = mx;
+    p.part_sum[o] = sum;
+  }
+}
+
+// One wave per row: merge the vocabulary-split partials into lse, compute the
+// target logit as a direct dot product hidden[r] . weight[label] (+bias, soft
+// cap), and write loss = lse - target (0 for ignored rows; a label outside
+// [0, v) or equal to the excluded column contributes target 0, as in
+// ce_forward_kernel, fused_linear_ce_cuda.cu:199-219).
+struct CombineArgs {
+  const void* hidden;
+  const void* weight;
+  const float* bias;
+  const int64_t* labels;
+  const int64_t* row_idx;
+  int m, h, v;
+  int64_t ignore, exclude;
+  float softcap;
+  const float* part_max;
+  const float* part_sum;
+  int part_ld, nsplit;
+  float* losses;
+  float* lse;
+  float* valid_count;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= p.m) return;
+  float mx = -INFINITY;
+  for (int s = lane; s < p.nsplit; s += 64) mx = fmaxf(mx, p.part_max[(int64_t)s * p.part_ld + r]);
+  mx = wave_max(mx);
+  float sum = 0.0f;
+  for (int s = lane; s < p.nsplit; s += 64) {
+    const float pm = p.part_max[(int64_t)s * p.part_ld + r];
+    if (pm > -INFINITY) sum += p.part_sum[(int64_t)s * p.part_ld + r] * fast_exp2(pm - mx);
+  }
+  sum = wave_sum(sum);
+  const float lse = (mx + log2f(sum)) * TLCE_LN2;
+
+  const int64_t y = p.labels[r];
+  const bool valid = (y != p.ignore);
+  const bool has_target = valid && y >= 0 && y < p.v && y != p.exclude;
+  float target = 0.0f;
+  if (has_target) {
+    const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
+    const T* wrow = static_cast<const T*>(p.weight) + y * (int64_t)p.h;
+    float dot = 0.0f;
+    for (int k = lane; k < p.h; k += 64) dot = fmaf(to_float<T>(hrow[k]), to_float<T>(wrow[k]), dot);
+    dot = wave_sum(dot);
+    if (p.bias != nullptr) dot += p.bias[y];
+    if (p.softcap > 0.0f) dot = p.softcap * tanhf(dot / p.softcap);
+    target = dot;
+  }
+  if (lane == 0) {
+    p.lse[r] = lse;
+    const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r;
+    p.losses[o] = valid ? (lse - target) : 0.0f;
+    if (valid) atomicAdd(p.valid_count, 1.0f);
+  }
+}
+
+// ----------------------------------------------------------------- backward --
+// scale[r] = d loss / d token_loss[r]  (token_scale_value,
+// fused_linear_ce_cuda.cu:226-238), 0 for ignored and padding rows.
+struct ScaleArgs {
+  const int64_t* labels;
+  const int64_t* row_idx;
+  const float* grad_output;
+  const float* valid_count;
+  int m, mp;
+  int reduction;
+  int64_t ignore;
+  float* scale;
+};
+
+__global__ __launch_bounds__(256) void lce_token_scale_kernel(ScaleArgs p) {
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r >= p.mp) return;
+  float s = 0.0f;
+  if (r < p.m && p.labels[r] != p.ignore) {
+    if (p.reduction == TLCE_REDUCTION_NONE) {
+      s = p.grad_output[(p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r];
+    } else if (p.reduction == TLCE_REDUCTION_SUM) {
+      s = p.grad_output[0];
+    } else {
+      s = p.grad_output[0] / p.valid_count[0];
+    }
+  }
+  p.scale[r] = s;
+}
+
+// Recompute one logits^T tile of a vocabulary panel and turn it, in registers,
+// into the logit gradient of ce_grad_logits_kernel
+// (fused_linear_ce_cuda.cu:240-290):
+//   g = (exp(cap(z) - lse) - [v == label]) * scale * (1 - tanh^2(z / cap)),
+// 0 for ignored rows, the excluded column and padding.  g is rounded to the
+// input dtype and written to the panel in both orientations: G[token, v] feeds
+// the grad-hidden contraction, GT[v, token] the grad-weight contraction.
+struct GradLogitsArgs {
+  const void* hidden;
+  const void* weight;
+  const float* bias;
+  const int64_t* labels;
+  const float* lse;
+  const float* scale;
+  int m, h, v;
+  int64_t ignore, exclude;
+  float softcap;
+  int v0;             // first vocabulary row of the panel
+  int n_ttiles, n_ptiles;
+  void* g;            // [mp, ldg]
+  int64_t ldg;
+  void* gt;           // [panel columns, ldgt] or null
+  int64_t ldgt;
+  float* grad_bias;   // [v] or null
+};
+
+template <typename T>
+__device__ __forceinline__ void store4(T* dst, float a, float b, float c, float d) {
+  if constexpr (sizeof(T) == 2) {
+    typedef T v4_t __attribute__((ext_vector_type(4)));
+    v4_t x;
+    x[0] = from_float<T>(a);
+    x[1] = from_float<T>(b);
+    x[2] = from_float<T>(c);
+    x[3] = from_float<T>(d);
+    *reinterpret_cast<v4_t*>(dst) = x;
+  } else {
+    *reinterpret_cast<float4*>(dst) = make_float4(a, b, c, d);
+  }
+}
+
+template <class E, bool kSoftcap, bool kBias>
+__global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(GradLogitsArgs p) {
+  extern __shared__ __align__(16) char smem[];
+  using T = typename E::T;
+  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
+  if (logical >= p.n_ttiles * p.n_ptiles) return;
+  int tt, pv;
+  grouped_tile(logical, p.n_ttiles, p.n_ptiles, 4, &tt, &pv);
+
+  E eng;
+  const T* hidden = static_cast<const T*>(p.hidden);
+  const T* weight = static_cast<const T*>(p.weight);
+  typename E::Acc acc;
+  E::zero(acc);
+  const int vbase = p.v0 + pv * E::kTile;
+  eng.mainloop(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+
+  const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
+  int64_t label[E::kCols];
+  float lse2[E::kCols], scale[E::kCols];
+  bool live[E::kCols];
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    const int r = tt * E::kTile + eng.col(j);
+    const int rc = min(r, p.m - 1);
+    label[j] = p.labels[rc];
+    live[j] = (r < p.m) && (label[j] != p.ignore);
+    lse2[j] = p.lse[rc] * TLCE_LOG2E;
+    scale[j] = live[j] ? p.scale[rc] : 0.0f;
+  }
+
+  if (kBias) {
+#pragma unroll
+    for (int i = 0; i < E::kRows; ++i) {
+      const float b = p.bias[min(vbase + eng.row(i), p.v - 1)];
+#pragma unroll
+      for (int j = 0; j < E::kCols; ++j) E::set(acc, j, i, E::get(acc, j, i) + b);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < E::kRows; ++i) {
+    const int v = vbase + eng.row(i);
+    const bool vok = (v < p.v) && (v != p.exclude);
+    float row_sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      float z = E::get(acc, j, i);
+      float dcap = 1.0f;
+      if (kSoftcap) {
+        const float t = fast_tanh(z * inv_cap);
+        z = p.softcap * t;
+        dcap = 1.0f - t * t;
+      }
+      float g = fast_exp2(z * TLCE_LOG2E - lse2[j]);
+      if ((int64_t)v == label[j]) g -= 1.0f;
+      g *= scale[j];
+      if (kSoftcap) g *= dcap;
+      g = (vok && live[j]) ? g : 0.0f;
+      E::set(acc, j, i, g);
+      row_sum += g;
+    }
+    if (kBias) {
+      row_sum = eng.reduce_over_cols(row_sum);
+      if (eng.col_leader() && v < p.v && row_sum != 0.0f) atomicAdd(p.grad_bias + v, row_sum);
+    }
+  }
+
+  T* g_out = static_cast<T*>(p.g);
+  T* gt_out = static_cast<T*>(p.gt);
+  const int prow = pv * E::kTile;  // first panel column of this tile
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    const int64_t r = (int64_t)tt * E::kTile + eng.col(j);
+#pragma unroll
+    for (int i = 0; i < E::kRows; i += 4) {
+      store4<T>(g_out + r * p.ldg + prow + eng.row(i), E::get(acc, j, i), E::get(acc, j, i + 1),
+                E::get(acc, j, i + 2), E::get(acc, j, i + 3));
+    }
+    if (gt_out != nullptr) {
+#pragma unroll
+      for (int i = 0; i < E::kRows; ++i)
+        gt_out[(int64_t)(prow + eng.row(i)) * p.ldgt + r] = from_float<T>(E::get(acc, j, i));
+    }
+  }
+}
+
+// C[i][j] (op)= sum_k A[i][k] * B[j][k]  — the two gradient contractions:
+//   grad_hidden: A = G panel [mp, Kv], B = weight^T [h, Kv]   -> C float32 [mp, h]
+//   grad_weight: A = GT panel [pv, Km], B = hidden^T [h, Km]  -> C dtype   [pv, h]
+// (project_grad_hidden / accumulate_grad_weight, fused_linear_ce_cuda.cu:676-791,
+// with float32 accumulation).  blockIdx.y selects a K split.
+enum { kStoreF32 = 0, kAddF32 = 1, kAtomicF32 = 2, kStoreT = 3 };
+
+struct GemmArgs {
+  const void* a;
+  int64_t lda;
+  int a_rows;
+  const void* b;
+  int64_t ldb;
+  int b_rows;
+  int k;            // padded K, multiple of the engine's BK
+  int k_per_split;  // multiple of BK
+  int ni, nj;
+  void* c;
+  int64_t ldc;
+  int c_rows, c_cols;
+  int mode;
+};
+
+template <class E>
+__global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
+  extern __shared__ __align__(16) char smem[];
+  using T = typename E::T;
+  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
+  if (logical >= p.ni * p.nj) return;
+  int ti, tj;
+  grouped_tile(logical, p.ni, p.nj, 4, &ti, &tj);
+  const int k_begin = blockIdx.y * p.k_per_split;
+  const int k_end = min(p.k, k_begin + p.k_per_split);
+  if (k_begin >= k_end) return;
+
+  E eng;
+  typename E::Acc acc;
+  E::zero(acc);
+  eng.mainloop(static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows,
+               static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows, k_begin, k_end, acc,
+               smem);
+
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    const int col = tj * E::kTile + eng.col(j);
+    if (col >= p.c_cols) continue;
+#pragma unroll
+    for (int i = 0; i < E::kRows; ++i) {
+      const int row = ti * E::kTile + eng.row(i);
+      if (row >= p.c_rows) continue;
+      const int64_t o = (int64_t)row * p.ldc + col;
+      const float val = E::get(acc, j, i);
+      if (p.mode == kStoreT) {
+        static_cast<T*>(p.c)[o] = from_float<T>(val);
+      } else if (p.mode == kStoreF32) {
+        static_cast<float*>(p.c)[o] = val;
+      } else if (p.mode == kAddF32) {
+        static_cast<float*>(p.c)[o] += val;
+      } else {
+        atomicAdd(static_cast<float*>(p.c) + o, val);
+      }
+    }
+  }
+}
+
+// out[c][r] = in[r][c] for r < rows, zero for rows <= r < out_cols: the
+// K-contiguous copies (weight^T, hidden^T) the gradient contractions read.
+// The zero padding keeps 0 * garbage out of the padded K range.
+template <typename T>
+__global__ __launch_bounds__(256) void lce_transpose_pad_kernel(const T* __restrict__ in,
+                                                                int64_t ld_in, int rows, int cols,
+                                                                T* __restrict__ out,
+                                                                int64_t ld_out, int out_cols) {
+  __shared__ T tile[64][66];
+  const int tx = threadIdx.x & 63;
+  const int ty = threadIdx.x >> 6;
+  const int c0 = blockIdx.x * 64;
+  const int r0 = blockIdx.y * 64;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int rr = ty + 4 * q;
+    const int r = r0 + rr;
+    const int c = c0 + tx;
+    tile[rr][tx] = (r < rows && c < cols) ? in[(int64_t)r * ld_in + c] : from_float<T>(0.0f);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < 16; ++q) {
+    const int cc = ty + 4 * q;
+    const int c = c0 + cc;
+    const int r = r0 + tx;
+    if (c < cols && r < out_cols) out[(int64_t)c * ld_out + r] = tile[tx][cc];
+  }
+}
+
+// grad_hidden[row_idx[r], :] = dtype(acc32[r, :])  (cast_float_to_scalar_kernel,
+// fused_linear_ce_cuda.cu:144-154, fused with the un-compaction scatter).
+template <typename T>
+__global__ __launch_bounds__(256) void lce_finalize_grad_hidden_kernel(
+    const float* __restrict__ acc32, const int64_t* __restrict__ row_idx, int m, int h,
+    T* __restrict__ out) {
+  const int r = blockIdx.x;
+  if (r >= m) return;
+  const int64_t o = (row_idx != nullptr) ? row_idx[r] : (int64_t)r;
+  const float* src = acc32 + (int64_t)r * h;
+  T* dst = out + o * h;
+  for (int k = threadIdx.x; k < h; k += 256) dst[k] = from_float<T>(src[k]);
+}
+
+__global__ __launch_bounds__(256) void lce_fill_zero_kernel(uint4* __restrict__ dst16,
+                                                            int64_t n16, unsigned char* tail,
+                                                            int ntail) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) dst16[i] = z;
+  if (blockIdx.x == 0 && (int)threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+
+}  // namespace tlce

@@ -1,0 +1,548 @@
+// Host scheduler and C ABI of the fused linear cross-entropy for gfx950.
+//
+// Replaces fused_linear_ce_forward_cuda / fused_linear_ce_backward_cuda
+// (dllm_parallel/core/csrc/fused_linear_ce/fused_linear_ce_cuda.cu:898-989,
+// :991-1172).  Where the reference loops over ~1K-row blocks and round-trips
+// float32 logits through memory three times per block, this scheduler
+//   forward : one launch of the online-softmax tile kernel (+ a per-row merge);
+//   backward: loops over vocabulary panels; per panel one launch recomputes the
+//             logits tiles and writes the dtype-rounded logit gradients of the
+//             panel, one contraction accumulates grad_hidden in float32 and
+//             one writes the panel's rows of grad_weight, complete, in dtype.
+// Nothing here allocates or synchronises.
+#include <algorithm>
+#include <vector>
+
+#include "tlce_common.h"
+#include "tlce_engine_mfma.h"
+#include "tlce_engine_simt.h"
+#include "tlce_kernels.h"
+
+namespace tlce {
+
+char* error_buffer() {
+  static thread_local char buf[512] = {0};
+  return buf;
+}
+
+int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+namespace {
+
+// ------------------------------------------------------------- profiling ----
+// Optional per-kernel-class timing with HIP events on the caller's stream
+// (tlce_profile_begin / tlce_profile_end).  Off by default; when off a launch
+// costs one thread-local pointer test.  One profiling session per thread.
+enum KernelClass {
+  kClassForwardStats = 0,
+  kClassCombine = 1,
+  kClassGradLogits = 2,
+  kClassGradHidden = 3,
+  kClassGradWeight = 4,
+  kClassTranspose = 5,
+  kClassOther = 6,
+  kNumClasses = 7
+};
+
+struct Profiler {
+  struct Record { int cls; hipEvent_t start, stop; };
+  std::vector<Record> records;
+};
+thread_local Profiler* g_profiler = nullptr;
+
+struct ScopedTimer {
+  Profiler* prof;
+  hipStream_t stream;
+  hipEvent_t start = nullptr, stop = nullptr;
+  int cls;
+  ScopedTimer(int cls_, hipStream_t s) : prof(g_profiler), stream(s), cls(cls_) {
+    if (!prof) return;
+    if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) {
+      prof = nullptr;
+      return;
+    }
+    (void)hipEventRecord(start, stream);
+  }
+  ~ScopedTimer() {
+    if (!prof) return;
+    (void)hipEventRecord(stop, stream);
+    prof->records.push_back({cls, start, stop});
+  }
+};
+
+constexpr int64_t kDefaultPanelBytes = 1ll << 30;
+constexpr int kTargetWorkgroups = 1024;  // 4 per CU on a 256-CU MI355X
+
+struct Plan {
+  int engine;  // 1 = MFMA, 0 = generic
+  int tile;
+  int bk;
+  int64_t mp, vp;
+  int n_ttiles, n_vtiles, n_htiles;
+  int nsplit;         // forward vocabulary splits
+  int64_t vc;         // panel columns
+  int n_panels;
+  int dh_ksplit;
+};
+
+Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_grad,
+               int64_t panel_bytes) {
+  Plan p;
+  p.engine = (dtype != TLCE_DTYPE_F32 && (h % 8) == 0) ? 1 : 0;
+  p.tile = p.engine ? 256 : 64;
+  p.bk = p.engine ? 64 : 16;
+  const int64_t mm = std::max<int64_t>(m, 1);
+  p.mp = round_up(mm, p.tile);
+  p.vp = round_up(v, p.tile);
+  p.n_ttiles = (int)(p.mp / p.tile);
+  p.n_vtiles = (int)(p.vp / p.tile);
+  p.n_htiles = (int)ceil_div(h, p.tile);
+  p.nsplit = (int)std::min<int64_t>(p.n_vtiles,
+                                    std::max<int64_t>(1, ceil_div(kTargetWorkgroups, p.n_ttiles)));
+  if (panel_bytes <= 0) panel_bytes = kDefaultPanelBytes;
+  const int64_t col_bytes = p.mp * dtype_bytes(dtype) * (weight_grad ? 2 : 1);
+  int64_t tiles_per_panel = std::max<int64_t>(1, panel_bytes / col_bytes / p.tile);
+  tiles_per_panel = std::min<int64_t>(tiles_per_panel, p.n_vtiles);
+  p.n_panels = (int)ceil_div(p.n_vtiles, tiles_per_panel);
+  p.vc = ceil_div(p.n_vtiles, p.n_panels) * p.tile;  // balanced panels
+  p.n_panels = (int)ceil_div(p.vp, p.vc);
+  p.dh_ksplit = 1;
+  if (p.engine) {
+    const int64_t tiles = (int64_t)p.n_ttiles * p.n_htiles;
+    if (tiles < 256) {
+      const int64_t ksteps = p.vc / p.bk;
+      p.dh_ksplit = (int)std::max<int64_t>(
+          1, std::min<int64_t>(ceil_div(512, tiles), ksteps / 8));
+    }
+  }
+  return p;
+}
+
+struct ForwardLayout {
+  int64_t part_max, part_sum, total;
+};
+ForwardLayout forward_layout(const Plan& p) {
+  ForwardLayout l;
+  const int64_t part = align256((int64_t)p.nsplit * p.mp * 4);
+  l.part_max = 0;
+  l.part_sum = part;
+  l.total = 2 * part;
+  return l;
+}
+
+struct BackwardLayout {
+  int64_t scale, acc32, wt, ht, g, gt, total;
+};
+BackwardLayout backward_layout(const Plan& p, int64_t h, int dtype, bool weight_grad) {
+  BackwardLayout l;
+  const int64_t es = dtype_bytes(dtype);
+  int64_t off = 0;
+  l.scale = off; off += align256(p.mp * 4);
+  l.acc32 = off; off += align256(p.mp * h * 4);
+  l.wt = off;    off += align256(h * p.vp * es);
+  l.ht = off;    off += weight_grad ? align256(h * p.mp * es) : 0;
+  l.g = off;     off += align256(p.mp * p.vc * es);
+  l.gt = off;    off += weight_grad ? align256(p.vc * p.mp * es) : 0;
+  l.total = off;
+  return l;
+}
+
+template <typename K>
+int enable_large_lds(K kernel, int bytes) {
+  if (bytes <= 64 * 1024) return 0;
+  TLCE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  return 0;
+}
+
+int validate_common(const void* hidden, const void* weight, int64_t m, int64_t h, int64_t v,
+                    int dtype) {
+  TLCE_REQUIRE(dtype == TLCE_DTYPE_F32 || dtype == TLCE_DTYPE_F16 || dtype == TLCE_DTYPE_BF16,
+               "unsupported dtype code %d", dtype);
+  TLCE_REQUIRE(m >= 0 && h > 0 && v > 0, "bad shape m=%lld h=%lld v=%lld", (long long)m,
+               (long long)h, (long long)v);
+  TLCE_REQUIRE(m < (1ll << 30) && h < (1ll << 30) && v < (1ll << 30),
+               "shape exceeds 32-bit tile indexing");
+  TLCE_REQUIRE(weight != nullptr && (hidden != nullptr || m == 0), "null input pointer");
+  TLCE_REQUIRE(((uintptr_t)hidden & 15) == 0 && ((uintptr_t)weight & 15) == 0,
+               "hidden and weight must be 16-byte aligned");
+  return 0;
+}
+
+// ---------------------------------------------------------------- launches --
+template <class E, bool kSoftcap, bool kBias>
+int launch_forward_variant(const Plan& p, const ForwardArgs& a, hipStream_t stream) {
+  static int rc = enable_large_lds(lce_forward_stats_kernel<E, kSoftcap, kBias>, E::kSmemBytes);
+  if (rc) return rc;
+  const int grid = xcd_grid((int64_t)p.n_ttiles * p.nsplit);
+  ScopedTimer timer(kClassForwardStats, stream);
+  lce_forward_stats_kernel<E, kSoftcap, kBias><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+template <class E>
+int launch_forward(const Plan& p, const ForwardArgs& a, hipStream_t stream) {
+  const bool softcap = a.softcap > 0.0f, bias = a.bias != nullptr;
+  if (softcap && bias) return launch_forward_variant<E, true, true>(p, a, stream);
+  if (softcap) return launch_forward_variant<E, true, false>(p, a, stream);
+  if (bias) return launch_forward_variant<E, false, true>(p, a, stream);
+  return launch_forward_variant<E, false, false>(p, a, stream);
+}
+
+template <class E, bool kSoftcap, bool kBias>
+int launch_grad_logits_variant(const GradLogitsArgs& a, hipStream_t stream) {
+  static int rc =
+      enable_large_lds(lce_grad_logits_panel_kernel<E, kSoftcap, kBias>, E::kSmemBytes);
+  if (rc) return rc;
+  const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
+  ScopedTimer timer(kClassGradLogits, stream);
+  lce_grad_logits_panel_kernel<E, kSoftcap, kBias>
+      <<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+template <class E>
+int launch_grad_logits(const GradLogitsArgs& a, hipStream_t stream) {
+  const bool softcap = a.softcap > 0.0f, bias = a.bias != nullptr;
+  if (softcap && bias) return launch_grad_logits_variant<E, true, true>(a, stream);
+  if (softcap) return launch_grad_logits_variant<E, true, false>(a, stream);
+  if (bias) return launch_grad_logits_variant<E, false, true>(a, stream);
+  return launch_grad_logits_variant<E, false, false>(a, stream);
+}
+
+template <class E>
+int launch_gemm(GemmArgs a, int ksplit, int cls, hipStream_t stream) {
+  static int rc = enable_large_lds(lce_gemm_nt_kernel<E>, E::kSmemBytes);
+  if (rc) return rc;
+  const int ksteps = a.k / E::kBK;
+  a.k_per_split = (int)ceil_div(ksteps, ksplit) * E::kBK;
+  dim3 grid(xcd_grid((int64_t)a.ni * a.nj), ksplit, 1);
+  ScopedTimer timer(cls, stream);
+  lce_gemm_nt_kernel<E><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+template <typename T>
+int launch_transpose(const T* in, int64_t ld_in, int64_t rows, int64_t cols, T* out,
+                     int64_t ld_out, int64_t out_cols, hipStream_t stream) {
+  dim3 grid((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(out_cols, 64), 1);
+  TLCE_REQUIRE(grid.y <= 65535, "transpose: too many row tiles");
+  ScopedTimer timer(kClassTranspose, stream);
+  lce_transpose_pad_kernel<T><<<grid, 256, 0, stream>>>(in, ld_in, (int)rows, (int)cols, out,
+                                                        ld_out, (int)out_cols);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+int fill_zero(void* dst, int64_t bytes, hipStream_t stream) {
+  if (bytes <= 0) return 0;
+  TLCE_REQUIRE(((uintptr_t)dst & 15) == 0 || bytes < 16, "fill_zero: dst must be 16-byte aligned");
+  const int64_t n16 = (((uintptr_t)dst & 15) == 0) ? bytes / 16 : 0;
+  const int ntail = (int)(bytes - n16 * 16);
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n16, 256), 256 * 16));
+  ScopedTimer timer(kClassOther, stream);
+  lce_fill_zero_kernel<<<grid, 256, 0, stream>>>(static_cast<uint4*>(dst), n16,
+                                                 static_cast<unsigned char*>(dst) + n16 * 16, ntail);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+// ----------------------------------------------------------------- forward --
+template <class E>
+int forward_impl(const Plan& p, const void* hidden, const void* weight, const float* bias,
+                 const int64_t* labels, const int64_t* row_idx, int64_t m, int64_t h, int64_t v,
+                 int64_t ignore, int64_t exclude, float softcap, float* losses, float* lse,
+                 float* valid_count, char* ws, hipStream_t stream) {
+  using T = typename E::T;
+  const ForwardLayout l = forward_layout(p);
+  ForwardArgs fa;
+  fa.hidden = hidden; fa.weight = weight; fa.bias = bias;
+  fa.m = (int)m; fa.h = (int)h; fa.v = (int)v;
+  fa.exclude = exclude; fa.softcap = softcap;
+  fa.n_ttiles = p.n_ttiles; fa.n_vtiles = p.n_vtiles; fa.nsplit = p.nsplit;
+  fa.part_max = reinterpret_cast<float*>(ws + l.part_max);
+  fa.part_sum = reinterpret_cast<float*>(ws + l.part_sum);
+  fa.part_ld = (int)p.mp;
+  if (int rc = launch_forward<E>(p, fa, stream)) return rc;
+
+  CombineArgs ca;
+  ca.hidden = hidden; ca.weight = weight; ca.bias = bias; ca.labels = labels;
+  ca.row_idx = row_idx;
+  ca.m = (int)m; ca.h = (int)h; ca.v = (int)v;
+  ca.ignore = ignore; ca.exclude = exclude; ca.softcap = softcap;
+  ca.part_max = fa.part_max; ca.part_sum = fa.part_sum;
+  ca.part_ld = fa.part_ld; ca.nsplit = p.nsplit;
+  ca.losses = losses; ca.lse = lse; ca.valid_count = valid_count;
+  {
+    ScopedTimer timer(kClassCombine, stream);
+    lce_combine_loss_kernel<T><<<(int)ceil_div(m, 4), 256, 0, stream>>>(ca);
+  }
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------- backward --
+template <class E>
+int backward_impl(const Plan& p, const void* hidden, const void* weight, const float* bias,
+                  const int64_t* labels, const int64_t* row_idx, const float* lse,
+                  const float* valid_count, const float* grad_output, int64_t m, int64_t n_out,
+                  int64_t h, int64_t v, int dtype, int reduction, int64_t ignore, int64_t exclude,
+                  float softcap, void* grad_hidden, void* grad_weight, float* grad_bias, char* ws,
+                  hipStream_t stream) {
+  using T = typename E::T;
+  const bool weight_grad = grad_weight != nullptr;
+  const BackwardLayout l = backward_layout(p, h, dtype, weight_grad);
+  float* scale = reinterpret_cast<float*>(ws + l.scale);
+  float* acc32 = reinterpret_cast<float*>(ws + l.acc32);
+  T* wt = reinterpret_cast<T*>(ws + l.wt);
+  T* ht = reinterpret_cast<T*>(ws + l.ht);
+  T* g = reinterpret_cast<T*>(ws + l.g);
+  T* gt = weight_grad ? reinterpret_cast<T*>(ws + l.gt) : nullptr;
+
+  ScaleArgs sa;
+  sa.labels = labels; sa.row_idx = row_idx; sa.grad_output = grad_output;
+  sa.valid_count = valid_count; sa.m = (int)m; sa.mp = (int)p.mp; sa.reduction = reduction;
+  sa.ignore = ignore; sa.scale = scale;
+  {
+    ScopedTimer timer(kClassOther, stream);
+    lce_token_scale_kernel<<<(int)ceil_div(p.mp, 256), 256, 0, stream>>>(sa);
+  }
+  TLCE_LAUNCH_CHECK();
+
+  // K-contiguous operands of the two gradient contractions
+  if (int rc = launch_transpose<T>(static_cast<const T*>(weight), h, v, h, wt, p.vp, p.vp, stream))
+    return rc;
+  if (weight_grad) {
+    if (int rc = launch_transpose<T>(static_cast<const T*>(hidden), h, m, h, ht, p.mp, p.mp,
+                                     stream))
+      return rc;
+  }
+  if (p.dh_ksplit > 1) {
+    if (int rc = fill_zero(acc32, p.mp * h * 4, stream)) return rc;
+  }
+  if (grad_bias != nullptr) {
+    if (int rc = fill_zero(grad_bias, v * 4, stream)) return rc;
+  }
+
+  for (int panel = 0; panel < p.n_panels; ++panel) {
+    const int64_t v0 = (int64_t)panel * p.vc;
+    const int64_t width = std::min<int64_t>(p.vc, p.vp - v0);   // multiple of tile
+    const int64_t rows_valid = std::min<int64_t>(p.vc, v - v0);  // real vocabulary rows
+    GradLogitsArgs ga;
+    ga.hidden = hidden; ga.weight = weight; ga.bias = bias; ga.labels = labels;
+    ga.lse = lse; ga.scale = scale;
+    ga.m = (int)m; ga.h = (int)h; ga.v = (int)v;
+    ga.ignore = ignore; ga.exclude = exclude; ga.softcap = softcap;
+    ga.v0 = (int)v0;
+    ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
+    ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
+    ga.grad_bias = (bias != nullptr) ? grad_bias : nullptr;
+    if (int rc = launch_grad_logits<E>(ga, stream)) return rc;
+
+    GemmArgs dh;
+    dh.a = g; dh.lda = p.vc; dh.a_rows = (int)p.mp;
+    dh.b = wt + v0; dh.ldb = p.vp; dh.b_rows = (int)h;
+    dh.k = (int)width; dh.k_per_split = 0;
+    dh.ni = p.n_ttiles; dh.nj = p.n_htiles;
+    dh.c = acc32; dh.ldc = h; dh.c_rows = (int)p.mp; dh.c_cols = (int)h;
+    dh.mode = (p.dh_ksplit > 1) ? kAtomicF32 : (panel == 0 ? kStoreF32 : kAddF32);
+    if (int rc = launch_gemm<E>(dh, p.dh_ksplit, kClassGradHidden, stream)) return rc;
+
+    if (weight_grad) {
+      GemmArgs dw;
+      dw.a = gt; dw.lda = p.mp; dw.a_rows = (int)width;
+      dw.b = ht; dw.ldb = p.mp; dw.b_rows = (int)h;
+      dw.k = (int)p.mp; dw.k_per_split = 0;
+      dw.ni = (int)(width / p.tile); dw.nj = p.n_htiles;
+      dw.c = static_cast<T*>(grad_weight) + v0 * h; dw.ldc = h;
+      dw.c_rows = (int)rows_valid; dw.c_cols = (int)h;
+      dw.mode = kStoreT;
+      if (int rc = launch_gemm<E>(dw, 1, kClassGradWeight, stream)) return rc;
+    }
+  }
+
+  if (row_idx != nullptr) {
+    if (int rc = fill_zero(grad_hidden, n_out * h * dtype_bytes(dtype), stream)) return rc;
+  }
+  {
+    ScopedTimer timer(kClassOther, stream);
+    lce_finalize_grad_hidden_kernel<T><<<(int)m, 256, 0, stream>>>(acc32, row_idx, (int)m, (int)h,
+                                                                 static_cast<T*>(grad_hidden));
+  }
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace
+}  // namespace tlce
+
+using namespace tlce;
+
+#define TLCE_DISPATCH(plan, dtype, CALL)                                                  \
+  do {                                                                                    \
+    if ((plan).engine) {                                                                  \
+      if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaEngine<__bf16>; return CALL; }      \
+      { using E = MfmaEngine<_Float16>; return CALL; }                                    \
+    }                                                                                     \
+    if ((dtype) == TLCE_DTYPE_F32) { using E = SimtEngine<float>; return CALL; }          \
+    if ((dtype) == TLCE_DTYPE_BF16) { using E = SimtEngine<__bf16>; return CALL; }        \
+    { using E = SimtEngine<_Float16>; return CALL; }                                      \
+  } while (0)
+
+extern "C" int tlce_version(void) { return TLCE_VERSION; }
+
+extern "C" const char* tlce_last_error(void) { return error_buffer(); }
+
+extern "C" int tlce_check_device(int device) {
+  hipDeviceProp_t prop;
+  TLCE_HIP(hipGetDeviceProperties(&prop, device));
+  TLCE_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0,
+               "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+  return 0;
+}
+
+extern "C" int tlce_fill_zero(void* dst, int64_t bytes, void* stream) {
+  TLCE_REQUIRE(bytes >= 0 && (dst != nullptr || bytes == 0), "fill_zero: bad arguments");
+  return fill_zero(dst, bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlce_query_plan(int64_t m, int64_t h, int64_t v, int dtype, int compute_weight_grad,
+                               int64_t panel_bytes, int* engine, int64_t* tile,
+                               int64_t* forward_vocab_splits, int64_t* panel_columns,
+                               int64_t* n_panels, int64_t* grad_hidden_k_splits) {
+  TLCE_REQUIRE(m >= 0 && h > 0 && v > 0, "query_plan: bad shape");
+  const Plan p = make_plan(m, h, v, dtype, compute_weight_grad != 0, panel_bytes);
+  if (engine) *engine = p.engine;
+  if (tile) *tile = p.tile;
+  if (forward_vocab_splits) *forward_vocab_splits = p.nsplit;
+  if (panel_columns) *panel_columns = p.vc;
+  if (n_panels) *n_panels = p.n_panels;
+  if (grad_hidden_k_splits) *grad_hidden_k_splits = p.dh_ksplit;
+  return 0;
+}
+
+extern "C" int64_t tlce_forward_workspace_bytes(int64_t m, int64_t h, int64_t v, int dtype) {
+  if (m < 0 || h <= 0 || v <= 0) return -1;
+  return forward_layout(make_plan(m, h, v, dtype, false, 0)).total;
+}
+
+extern "C" int tlce_forward(const void* hidden, const void* weight, const float* bias,
+                            const int64_t* labels, const int64_t* row_idx, int64_t m,
+                            int64_t n_out, int64_t h, int64_t v, int dtype, int64_t ignore_index,
+                            int64_t exclude_index, float logit_softcap, float* losses, float* lse,
+                            float* valid_count, void* workspace, int64_t workspace_bytes,
+                            void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  TLCE_REQUIRE(valid_count != nullptr, "forward: valid_count is null");
+  TLCE_REQUIRE(n_out >= m, "forward: n_out=%lld < m=%lld", (long long)n_out, (long long)m);
+  TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
+               "forward: n_out != m without row_idx");
+  if (int rc = fill_zero(valid_count, 4, stream)) return rc;
+  if (row_idx != nullptr || m == 0) {
+    TLCE_REQUIRE(losses != nullptr || n_out == 0, "forward: losses is null");
+    if (int rc = fill_zero(losses, n_out * 4, stream)) return rc;
+  }
+  if (m == 0) return 0;
+  TLCE_REQUIRE(labels && losses && lse && workspace, "forward: null pointer");
+  const Plan p = make_plan(m, h, v, dtype, false, 0);
+  TLCE_REQUIRE(workspace_bytes >= forward_layout(p).total,
+               "forward: workspace too small (%lld < %lld)", (long long)workspace_bytes,
+               (long long)forward_layout(p).total);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0, "forward: workspace must be 256-byte aligned");
+  TLCE_DISPATCH(p, dtype,
+                forward_impl<E>(p, hidden, weight, bias, labels, row_idx, m, h, v, ignore_index,
+                                exclude_index, logit_softcap, losses, lse, valid_count,
+                                static_cast<char*>(workspace), stream));
+}
+
+extern "C" int64_t tlce_backward_workspace_bytes(int64_t m, int64_t h, int64_t v, int dtype,
+                                                 int compute_weight_grad, int has_bias,
+                                                 int64_t panel_bytes) {
+  (void)has_bias;
+  if (m < 0 || h <= 0 || v <= 0) return -1;
+  const Plan p = make_plan(m, h, v, dtype, compute_weight_grad != 0, panel_bytes);
+  return backward_layout(p, h, dtype, compute_weight_grad != 0).total;
+}
+
+extern "C" int tlce_backward(const void* hidden, const void* weight, const float* bias,
+                             const int64_t* labels, const int64_t* row_idx, const float* lse,
+                             const float* valid_count, const float* grad_output, int64_t m,
+                             int64_t n_out, int64_t h, int64_t v, int dtype, int reduction_code,
+                             int64_t ignore_index, int64_t exclude_index, float logit_softcap,
+                             void* grad_hidden, void* grad_weight, float* grad_bias,
+                             int64_t panel_bytes, void* workspace, int64_t workspace_bytes,
+                             void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  TLCE_REQUIRE(reduction_code >= TLCE_REDUCTION_NONE && reduction_code <= TLCE_REDUCTION_MEAN,
+               "backward: bad reduction code %d", reduction_code);
+  TLCE_REQUIRE(n_out >= m, "backward: n_out=%lld < m=%lld", (long long)n_out, (long long)m);
+  TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
+               "backward: n_out != m without row_idx");
+  TLCE_REQUIRE(grad_hidden != nullptr || n_out == 0, "backward: grad_hidden is null");
+  TLCE_REQUIRE((bias == nullptr) || (grad_bias != nullptr), "backward: bias without grad_bias");
+  const int64_t es = dtype_bytes(dtype);
+  if (m == 0) {
+    if (int rc = fill_zero(grad_hidden, n_out * h * es, stream)) return rc;
+    if (grad_weight != nullptr) {
+      if (int rc = fill_zero(grad_weight, v * h * es, stream)) return rc;
+    }
+    if (bias != nullptr) return fill_zero(grad_bias, v * 4, stream);
+    return 0;
+  }
+  TLCE_REQUIRE(labels && lse && valid_count && grad_output && workspace, "backward: null pointer");
+  TLCE_REQUIRE(((uintptr_t)grad_hidden & 15) == 0 && ((uintptr_t)grad_weight & 15) == 0,
+               "backward: gradients must be 16-byte aligned");
+  const Plan p = make_plan(m, h, v, dtype, grad_weight != nullptr, panel_bytes);
+  const int64_t need = backward_layout(p, h, dtype, grad_weight != nullptr).total;
+  TLCE_REQUIRE(workspace_bytes >= need, "backward: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0, "backward: workspace must be 256-byte aligned");
+  TLCE_DISPATCH(p, dtype,
+                backward_impl<E>(p, hidden, weight, bias, labels, row_idx, lse, valid_count,
+                                 grad_output, m, n_out, h, v, dtype, reduction_code, ignore_index,
+                                 exclude_index, logit_softcap, grad_hidden, grad_weight,
+                                 (bias != nullptr) ? grad_bias : nullptr,
+                                 static_cast<char*>(workspace), stream));
+}
+
+extern "C" int tlce_profile_begin(void) {
+  TLCE_REQUIRE(g_profiler == nullptr, "profile_begin: a session is already open on this thread");
+  g_profiler = new Profiler();
+  return 0;
+}
+
+extern "C" int tlce_profile_end(double* class_ms, int64_t* class_launches, int n_classes) {
+  TLCE_REQUIRE(g_profiler != nullptr, "profile_end: no session is open on this thread");
+  Profiler* prof = g_profiler;
+  g_profiler = nullptr;
+  for (int c = 0; c < n_classes; ++c) {
+    if (class_ms) class_ms[c] = 0.0;
+    if (class_launches) class_launches[c] = 0;
+  }
+  int rc = 0;
+  for (auto& r : prof->records) {
+    float ms = 0.0f;
+    if (rc == 0 && hipEventSynchronize(r.stop) != hipSuccess) rc = fail("profile_end: event sync failed");
+    if (rc == 0 && hipEventElapsedTime(&ms, r.start, r.stop) != hipSuccess)
+      rc = fail("profile_end: elapsed time failed");
+    if (rc == 0 && r.cls < n_classes) {
+      if (class_ms) class_ms[r.cls] += ms;
+      if (class_launches) class_launches[r.cls] += 1;
+    }
+    (void)hipEventDestroy(r.start);
+    (void)hipEventDestroy(r.stop);
+  }
+  delete prof;
+  return rc;
+}
