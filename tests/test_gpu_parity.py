@@ -239,13 +239,29 @@ def test_reductions_and_dtypes(gpu_device, reduction, dtype):
 def test_dim_first_and_non_contiguous(gpu_device):
     say("dim_first / non-contiguous")
     torch.manual_seed(11)
-    hidden = torch.randn(2, 64, 72)[:, ::2, :].bfloat16()      # H=72: K tail inside one slab
-    labels = torch.randint(0, 300, (2, 64))[:, ::2]
+    base_hidden = torch.randn(2, 64, 72).bfloat16()            # H=72: K tail inside one slab
+    base_labels = torch.randint(0, 300, (2, 64))
     weight = (torch.randn(72, 300) * 0.2).bfloat16()
-    assert not hidden.is_contiguous()
-    loss, dh, dw, _ = check_against_oracle(gpu_device, hidden, weight, labels,
-                                           weight_layout="dim_first", reduction="sum")
-    assert dw.shape == (72, 300)
+    hidden, labels = base_hidden[:, ::2, :], base_labels[:, ::2]
+    # strided views on the device, as in test_tiled_linear_cross_entropy.py:153-169
+    h = base_hidden.to(gpu_device)[:, ::2, :].requires_grad_(True)
+    y = base_labels.to(gpu_device)[:, ::2]
+    w = weight.to(gpu_device).requires_grad_(True)
+    assert not h.is_contiguous() and not y.is_contiguous()
+    loss = tiled_linear_cross_entropy(h, w, y, reduction="sum", dtype=torch.bfloat16,
+                                      weight_layout="dim_first")
+    loss.backward()
+    ref = oracle.dense_linear_ce(hidden, weight, labels, reduction="sum", weight_dim_first=True)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, reduction="sum",
+                                               weight_dim_first=True)
+    torch.testing.assert_close(loss.cpu().double(), ref, rtol=LOSS_RTOL, atol=1e-5)
+    assert h.grad.shape == (2, 32, 72) and w.grad.shape == (72, 300)
+    assert oracle.relative_max_error(h.grad, rdh) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(w.grad, rdw) <= GRAD_REL_MAX
+    # layout inference from shapes gives the same answer
+    auto = tiled_linear_cross_entropy(h.detach(), w.detach(), y, reduction="sum",
+                                      dtype=torch.bfloat16)
+    assert torch.equal(auto, loss.detach())
 
 
 def test_softcap_with_bias_and_exclusion(gpu_device):
@@ -270,7 +286,7 @@ def test_empty_and_fully_ignored_inputs(gpu_device):
     assert none.shape == (10,) and torch.count_nonzero(none) == 0
     total = tiled_linear_cross_entropy(hidden, weight, labels, reduction="sum")
     total.backward()
-    assert float(total) == 0.0
+    assert float(total.detach()) == 0.0
     assert torch.count_nonzero(hidden.grad) == 0 and torch.count_nonzero(weight.grad) == 0
     assert torch.isnan(tiled_linear_cross_entropy(hidden, weight, labels, reduction="mean"))
     zero = tiled_linear_cross_entropy(hidden[:0], weight, labels[:0], reduction="sum")

@@ -85,6 +85,10 @@ def library() -> ctypes.CDLL:
             "Run `python -m turbo_dllm_amd.build` (or __graft_entry__.build()). "
             "Device tensors are never routed to a CPU or PyTorch fallback."
         )
+    # torch ships its own HIP runtime.  Loading it first makes this library bind
+    # to that same runtime; two runtimes in one process do not share the GPU.
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(str(LIBRARY_PATH))
     for name, (restype, argtypes) in SIGNATURES.items():
         try:
