@@ -1,6 +1,6 @@
-// 256x256x64 bf16/f16 MFMA tile engine for gfx950 (CDNA4), wave64.
+// 256x256 bf16/f16 MFMA tile engines for gfx950 (CDNA4), wave64.
 //
-// Computes C[i][j] = sum_k A[i][k] * B[j][k] for one 256x256 tile, A and B both
+// Both compute C[i][j] = sum_k A[i][k] * B[j][k] for one 256x256 tile, A and B both
 // K-contiguous (row-major [rows, K]).  512 threads = 8 waves in a 2 (A rows) x
 // 4 (B rows) grid; each wave owns a 128x64 sub-tile as 4x2
 // v_mfma_f32_32x32x16 blocks (128 fp32 accumulator registers per lane), two
@@ -39,32 +39,30 @@ template <> struct MfmaOp<_Float16> {
   }
 };
 
+// Thread <-> tile-element mapping shared by the MFMA engines: 8 waves as
+// 2 (A rows) x 4 (B rows), each wave 4x2 blocks of 32x32.
 template <typename T_>
-struct MfmaEngine {
+struct MfmaTileLayout {
   using T = T_;
   using Op = MfmaOp<T>;
   using V8 = typename Op::V8;
 
   static constexpr int kTile = 256;     // BM == BN
-  static constexpr int kBK = 64;
   static constexpr int kThreads = 512;
   static constexpr int kWavesN = 4;     // waves along B rows
   static constexpr int kTM = 4;         // 32-row blocks per wave along A rows
   static constexpr int kTN = 2;         // 32-col blocks per wave along B rows
-  static constexpr int kRowBytes = kBK * 2;                  // 128
-  static constexpr int kStageBytes = 2 * kTile * kRowBytes;  // 65536
-  static constexpr int kSmemBytes = 2 * kStageBytes;         // 131072
   static constexpr int kCols = kTN;          // tile columns owned per thread
   static constexpr int kRows = kTM * 16;     // tile rows held per owned column
   static constexpr int kShare = 4;           // threads that hold the same column
 
   struct Acc { f32x16_t c[kTM][kTN]; };
 
-  int lane, wm, wn;
+  int lane, wave, wm, wn;
 
-  __device__ __forceinline__ MfmaEngine() {
+  __device__ __forceinline__ MfmaTileLayout() {
     lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    wave = threadIdx.x >> 6;
     wm = wave / kWavesN;
     wn = wave % kWavesN;
   }
@@ -95,6 +93,28 @@ struct MfmaEngine {
     return v;
   }
   __device__ __forceinline__ bool col_leader() const { return (lane & 31) == 0; }
+};
+
+// Register-staged engine: global -> VGPR -> LDS, two 64-wide K stages.  Takes
+// any K that is a multiple of 8 (zero-fills the tail); used when the hidden
+// size is not a multiple of 32.
+template <typename T_>
+struct MfmaEngine : MfmaTileLayout<T_> {
+  using Base = MfmaTileLayout<T_>;
+  using T = T_;
+  using Op = typename Base::Op;
+  using V8 = typename Base::V8;
+  using Acc = typename Base::Acc;
+  using Base::kTile;
+  using Base::kTM;
+  using Base::kTN;
+  using Base::lane;
+  using Base::wm;
+  using Base::wn;
+  static constexpr int kBK = 64;
+  static constexpr int kRowBytes = kBK * 2;                  // 128
+  static constexpr int kStageBytes = 2 * kTile * kRowBytes;  // 65536
+  static constexpr int kSmemBytes = 2 * kStageBytes;         // 131072
 
   // acc += A[a_row0 .. +256, k_begin .. k_end) * B[b_row0 .. +256, same K)^T.
   // Rows past a_rows / b_rows are clamped to the last valid row (their results
@@ -185,6 +205,145 @@ struct MfmaEngine {
       if (more) sstore(cur ^ 1);
       __syncthreads();
     }
+  }
+};
+
+// Direct-to-LDS engine: the operand tiles go global -> LDS with
+// global_load_lds_dwordx4 (no VGPR staging, no ds_write), through a ring of
+// four 32-wide K stages (4 x 32 KiB), so a tile is requested three K steps
+// before it is consumed and HBM/L2 latency hides behind ~48 MFMAs per wave.
+// Needs K (k_end - k_begin) to be a multiple of 32.
+//
+// A stage row is 64 bytes = four 16-byte chunks; chunk c of row r sits in slot
+// c ^ ((r >> 2) & 3): the 16 lanes of one LDS read phase (16 rows, one chunk)
+// then cover all 64 banks.  A wave's load instruction fills 1 KiB = 16 rows:
+// lane i lands in row i/4, slot i%4, so it fetches logical chunk
+// (i%4) ^ ((i>>4)&3) of that row.
+//
+// Ordering: loads are counted per wave by vmcnt and complete in order.  Before
+// using tile k a wave waits until at most the loads of the (up to two) younger
+// tiles are outstanding, then the workgroup barrier publishes every wave's
+// part of tile k and retires stage (k-1)%4, which the loads of tile k+3 refill.
+template <typename T_>
+struct MfmaDirectEngine : MfmaTileLayout<T_> {
+  using Base = MfmaTileLayout<T_>;
+  using T = T_;
+  using Op = typename Base::Op;
+  using V8 = typename Base::V8;
+  using Acc = typename Base::Acc;
+  using Base::kTile;
+  using Base::kTM;
+  using Base::kTN;
+  using Base::lane;
+  using Base::wave;
+  using Base::wm;
+  using Base::wn;
+  static constexpr int kBK = 32;
+  static constexpr int kStages = 4;
+  static constexpr int kRowBytes = kBK * 2;                  // 64
+  static constexpr int kOperandBytes = kTile * kRowBytes;    // 16384
+  static constexpr int kStageBytes = 2 * kOperandBytes;      // 32768
+  static constexpr int kSmemBytes = kStages * kStageBytes;   // 131072
+
+  static __device__ __forceinline__ void load_to_lds(unsigned lds_addr, const T* src) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_addr), "v"(src)
+                 : "memory", "m0");
+  }
+
+  __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
+                                           int a_rows, const T* __restrict__ B, int64_t ldb,
+                                           int b_row0, int b_rows, int k_begin, int k_end,
+                                           Acc& acc, char* smem) const {
+    // loader role: this wave fills rows [32*wave, 32*wave+32) of both operands
+    const int lrow = lane >> 2;
+    const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const T* ap[2];
+    const T* bp[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r = wave * 32 + j * 16 + lrow;
+      const int ar = min(a_row0 + r, a_rows - 1);
+      const int br = min(b_row0 + r, b_rows - 1);
+      ap[j] = A + (int64_t)ar * lda + k_begin + chunk * 8;
+      bp[j] = B + (int64_t)br * ldb + k_begin + chunk * 8;
+    }
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;
+    const unsigned fill =
+        __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(wave * 32 * kRowBytes));
+
+    auto issue = [&](int stage) {
+      const unsigned dst = fill + (unsigned)(stage * kStageBytes);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        load_to_lds(dst + j * 16 * kRowBytes, ap[j]);
+        load_to_lds(dst + kOperandBytes + j * 16 * kRowBytes, bp[j]);
+        ap[j] += kBK;
+        bp[j] += kBK;
+      }
+    };
+
+    // consumer role: fragment addresses of this wave's 128x64 sub-tile
+    const int swz = (lane >> 2) & 3;
+    const int hi = lane >> 5;
+    const int a_frag = (wm * 128 + (lane & 31)) * kRowBytes;
+    const int b_frag = kOperandBytes + (wn * 64 + (lane & 31)) * kRowBytes;
+
+    auto compute = [&](int stage) {
+      const char* base = smem + stage * kStageBytes;
+      V8 af[kTM], bf[kTN];
+#pragma unroll
+      for (int ks = 0; ks < kBK / 16; ++ks) {
+        const int slot = ((2 * ks + hi) ^ swz) * 16;
+#ifdef TLCE_EXP_HALFLDS
+        if (ks == 0) {
+#endif
+#pragma unroll
+        for (int tm = 0; tm < kTM; ++tm)
+          af[tm] = __builtin_bit_cast(
+              V8, *reinterpret_cast<const uint4*>(base + a_frag + tm * 32 * kRowBytes + slot));
+#pragma unroll
+        for (int tn = 0; tn < kTN; ++tn)
+          bf[tn] = __builtin_bit_cast(
+              V8, *reinterpret_cast<const uint4*>(base + b_frag + tn * 32 * kRowBytes + slot));
+#ifdef TLCE_EXP_HALFLDS
+        }
+#endif
+#pragma unroll
+        for (int tm = 0; tm < kTM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < kTN; ++tn) acc.c[tm][tn] = Op::mma(af[tm], bf[tn], acc.c[tm][tn]);
+      }
+    };
+
+    const int nk = (k_end - k_begin) / kBK;
+#pragma unroll
+    for (int t = 0; t < kStages - 1; ++t)
+      if (t < nk) issue(t);
+    for (int k = 0; k < nk; ++k) {
+      const int younger = min(nk - 1 - k, kStages - 2);   // tiles in flight behind tile k
+#ifdef TLCE_EXP_NOWAIT
+      if (k + 1 == nk) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (false) {
+#else
+      if (younger >= 2) {
+#endif
+        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      } else if (younger == 1) {
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+#ifndef TLCE_EXP_NOBARRIER
+      __syncthreads();
+#endif
+#ifndef TLCE_EXP_NOLOAD
+      if (k + kStages - 1 < nk) issue((k + kStages - 1) & (kStages - 1));
+#endif
+      compute(k & (kStages - 1));
+    }
+    __syncthreads();
   }
 };
 

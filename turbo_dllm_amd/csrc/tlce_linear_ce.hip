@@ -80,7 +80,7 @@ constexpr int64_t kDefaultPanelBytes = 1ll << 30;
 constexpr int kTargetWorkgroups = 1024;  // 4 per CU on a 256-CU MI355X
 
 struct Plan {
-  int engine;  // 1 = MFMA, 0 = generic
+  int engine;  // 2 = direct-to-LDS MFMA, 1 = register-staged MFMA, 0 = generic
   int tile;
   int bk;
   int64_t mp, vp;
@@ -94,9 +94,10 @@ struct Plan {
 Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_grad,
                int64_t panel_bytes) {
   Plan p;
-  p.engine = (dtype != TLCE_DTYPE_F32 && (h % 8) == 0) ? 1 : 0;
+  // 2: direct-to-LDS MFMA (h % 32 == 0), 1: register-staged MFMA (h % 8 == 0), 0: generic
+  p.engine = (dtype == TLCE_DTYPE_F32 || (h % 8) != 0) ? 0 : ((h % 32) == 0 ? 2 : 1);
   p.tile = p.engine ? 256 : 64;
-  p.bk = p.engine ? 64 : 16;
+  p.bk = p.engine == 2 ? 32 : (p.engine == 1 ? 64 : 16);
   const int64_t mm = std::max<int64_t>(m, 1);
   p.mp = round_up(mm, p.tile);
   p.vp = round_up(v, p.tile);
@@ -389,7 +390,11 @@ using namespace tlce;
 
 #define TLCE_DISPATCH(plan, dtype, CALL)                                                  \
   do {                                                                                    \
-    if ((plan).engine) {                                                                  \
+    if ((plan).engine == 2) {                                                             \
+      if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaDirectEngine<__bf16>; return CALL; } \
+      { using E = MfmaDirectEngine<_Float16>; return CALL; }                              \
+    }                                                                                     \
+    if ((plan).engine == 1) {                                                             \
       if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaEngine<__bf16>; return CALL; }      \
       { using E = MfmaEngine<_Float16>; return CALL; }                                    \
     }                                                                                     \
