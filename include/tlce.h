@@ -140,8 +140,9 @@ int tlce_backward(const void* hidden, const void* weight, const float* bias,
 
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be
- * NULL.  `engine` is 1 for the bf16/f16 MFMA kernels, 0 for the generic
- * float32-FMA kernels (float32 inputs, or h not a multiple of 8). */
+ * NULL.  `engine` is 2 for the bf16/f16 MFMA kernels with direct-to-LDS loads
+ * (h a multiple of 32), 1 for the register-staged MFMA kernels (h a multiple of
+ * 8), 0 for the generic float32-FMA kernels (float32 inputs, other h). */
 int tlce_query_plan(int64_t m, int64_t h, int64_t v, int dtype,
                     int compute_weight_grad, int64_t panel_bytes,
                     int* engine, int64_t* tile, int64_t* forward_vocab_splits,

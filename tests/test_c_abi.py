@@ -48,7 +48,7 @@ def test_workspace_sizes_and_plan():
     assert lib.tlce_compact_workspace_bytes(-1) == -1
     # headline shape: MFMA engine, 256 tiles, vocabulary panels bounded by 1 GiB
     plan = _lib.query_plan(32768, 4096, 151936, _lib.DTYPE_BF16, True)
-    assert plan["engine"] == "mfma" and plan["tile"] == 256
+    assert plan["engine"] == "mfma_direct" and plan["tile"] == 256
     assert plan["forward_vocab_splits"] == 8
     assert plan["panel_columns"] % 256 == 0
     assert plan["panel_columns"] * 32768 * 2 * 2 <= (1 << 30)
@@ -67,7 +67,8 @@ def test_workspace_sizes_and_plan():
     # float32 inputs and odd hidden sizes take the generic engine
     assert _lib.query_plan(21, 33, 4097, _lib.DTYPE_F32, True)["engine"] == "generic"
     assert _lib.query_plan(21, 33, 4097, _lib.DTYPE_BF16, True)["engine"] == "generic"
-    assert _lib.query_plan(31, 96, 1025, _lib.DTYPE_BF16, True)["engine"] == "mfma"
+    assert _lib.query_plan(31, 96, 1025, _lib.DTYPE_BF16, True)["engine"] == "mfma_direct"
+    assert _lib.query_plan(64, 72, 300, _lib.DTYPE_BF16, True)["engine"] == "mfma"  # K tail
     # a smaller panel budget means more panels
     tight = _lib.query_plan(32768, 4096, 151936, _lib.DTYPE_BF16, True, 1 << 28)
     assert tight["n_panels"] > plan["n_panels"]
