@@ -17,6 +17,8 @@
 // K = 16*ks + 8*(l/32) .. +8  (one 16-byte chunk).
 #pragma once
 
+#include <type_traits>
+
 #include "tlce_common.h"
 
 namespace tlce {
@@ -39,22 +41,24 @@ template <> struct MfmaOp<_Float16> {
   }
 };
 
-// Thread <-> tile-element mapping shared by the MFMA engines: 8 waves as
-// 2 (A rows) x 4 (B rows), each wave 4x2 blocks of 32x32.
-template <typename T_>
+// Thread <-> tile-element mapping shared by the MFMA engines: 2 waves along
+// the A rows, kWavesN_ along the B rows, each wave 4 x kTN_ blocks of 32x32
+// (8 waves of 128x64, or 4 waves of 128x128).
+template <typename T_, int kWavesN_ = 4, int kTN_ = 2>
 struct MfmaTileLayout {
   using T = T_;
   using Op = MfmaOp<T>;
   using V8 = typename Op::V8;
 
   static constexpr int kTile = 256;     // BM == BN
-  static constexpr int kThreads = 512;
-  static constexpr int kWavesN = 4;     // waves along B rows
+  static constexpr int kWavesN = kWavesN_;   // waves along B rows
+  static constexpr int kThreads = 2 * kWavesN * 64;
   static constexpr int kTM = 4;         // 32-row blocks per wave along A rows
-  static constexpr int kTN = 2;         // 32-col blocks per wave along B rows
+  static constexpr int kTN = kTN_;      // 32-col blocks per wave along B rows
   static constexpr int kCols = kTN;          // tile columns owned per thread
   static constexpr int kRows = kTM * 16;     // tile rows held per owned column
   static constexpr int kShare = 4;           // threads that hold the same column
+  static_assert(kWavesN * kTN * 32 == kTile, "waves must tile the 256 B rows");
 
   struct Acc { f32x16_t c[kTM][kTN]; };
 
@@ -67,7 +71,9 @@ struct MfmaTileLayout {
     wn = wave % kWavesN;
   }
 
-  __device__ __forceinline__ int col(int j) const { return wn * 64 + j * 32 + (lane & 31); }
+  __device__ __forceinline__ int col(int j) const {
+    return wn * (kTN * 32) + j * 32 + (lane & 31);
+  }
   __device__ __forceinline__ int row(int i) const {
     return wm * 128 + (i >> 4) * 32 + ((i >> 2) & 3) * 8 + (lane >> 5) * 4 + (i & 3);
   }
@@ -290,59 +296,243 @@ struct MfmaDirectEngine : MfmaTileLayout<T_> {
     const int a_frag = (wm * 128 + (lane & 31)) * kRowBytes;
     const int b_frag = kOperandBytes + (wn * 64 + (lane & 31)) * kRowBytes;
 
-    auto compute = [&](int stage) {
+    // Fragments of one 16-wide K slice: 4 A blocks + 2 B blocks, 24 VGPRs.
+    struct Frags { V8 a[kTM]; V8 b[kTN]; };
+    auto read_slice = [&](Frags& f, int stage, int ks) {
       const char* base = smem + stage * kStageBytes;
-      V8 af[kTM], bf[kTN];
+      const int slot = ((2 * ks + hi) ^ swz) * 16;
 #pragma unroll
-      for (int ks = 0; ks < kBK / 16; ++ks) {
-        const int slot = ((2 * ks + hi) ^ swz) * 16;
-#ifdef TLCE_EXP_HALFLDS
-        if (ks == 0) {
-#endif
+      for (int tm = 0; tm < kTM; ++tm)
+        f.a[tm] = __builtin_bit_cast(
+            V8, *reinterpret_cast<const uint4*>(base + a_frag + tm * 32 * kRowBytes + slot));
 #pragma unroll
-        for (int tm = 0; tm < kTM; ++tm)
-          af[tm] = __builtin_bit_cast(
-              V8, *reinterpret_cast<const uint4*>(base + a_frag + tm * 32 * kRowBytes + slot));
+      for (int tn = 0; tn < kTN; ++tn)
+        f.b[tn] = __builtin_bit_cast(
+            V8, *reinterpret_cast<const uint4*>(base + b_frag + tn * 32 * kRowBytes + slot));
+    };
+    auto mma_slice = [&](const Frags& f) {
 #pragma unroll
-        for (int tn = 0; tn < kTN; ++tn)
-          bf[tn] = __builtin_bit_cast(
-              V8, *reinterpret_cast<const uint4*>(base + b_frag + tn * 32 * kRowBytes + slot));
-#ifdef TLCE_EXP_HALFLDS
-        }
-#endif
+      for (int tm = 0; tm < kTM; ++tm)
 #pragma unroll
-        for (int tm = 0; tm < kTM; ++tm)
-#pragma unroll
-          for (int tn = 0; tn < kTN; ++tn) acc.c[tm][tn] = Op::mma(af[tm], bf[tn], acc.c[tm][tn]);
-      }
+        for (int tn = 0; tn < kTN; ++tn) acc.c[tm][tn] = Op::mma(f.a[tm], f.b[tn], acc.c[tm][tn]);
     };
 
+    // Software pipeline: the fragments of the next K slice are always in flight
+    // while the MFMAs of the current one issue, also across K steps.  The
+    // barrier that publishes tile k+1 sits in the middle of step k, after the
+    // last LDS reads of tile k have been issued and before slice 0 of tile k+1
+    // is read; the stage refilled after it, (k+3)%4 == (k-1)%4, was last read
+    // in step k-1.
     const int nk = (k_end - k_begin) / kBK;
 #pragma unroll
     for (int t = 0; t < kStages - 1; ++t)
       if (t < nk) issue(t);
-    for (int k = 0; k < nk; ++k) {
-      const int younger = min(nk - 1 - k, kStages - 2);   // tiles in flight behind tile k
-#ifdef TLCE_EXP_NOWAIT
-      if (k + 1 == nk) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (false) {
-#else
-      if (younger >= 2) {
-#endif
-        asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-      } else if (younger == 1) {
+    if (nk >= 3) {
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    } else if (nk == 2) {
+      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+    Frags f0, f1;
+    read_slice(f0, 0, 0);
+    for (int k = 0; k + 1 < nk; ++k) {
+      read_slice(f1, k & (kStages - 1), 1);
+      __builtin_amdgcn_sched_barrier(0);   // keep the LDS reads ahead of the MFMA batch
+      mma_slice(f0);
+      // tile k+1 must have landed; tile k+2 (if any) may stay in flight
+      if (k + 2 < nk) {
         asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
       } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       }
-#ifndef TLCE_EXP_NOBARRIER
       __syncthreads();
-#endif
-#ifndef TLCE_EXP_NOLOAD
       if (k + kStages - 1 < nk) issue((k + kStages - 1) & (kStages - 1));
-#endif
-      compute(k & (kStages - 1));
+      read_slice(f0, (k + 1) & (kStages - 1), 0);
+      __builtin_amdgcn_sched_barrier(0);
+      mma_slice(f1);
     }
+    read_slice(f1, (nk - 1) & (kStages - 1), 1);
+    mma_slice(f0);
+    mma_slice(f1);
+    __syncthreads();
+  }
+};
+
+// Four-wave direct-to-LDS engine (K multiple of 64): 256 threads, each wave a
+// 128x128 sub-tile (4x4 MFMA blocks, 256 accumulator registers, one wave per
+// SIMD), which halves the LDS fragment traffic per MFMA of the 8-wave layout.
+// Two 64-wide K stages of 64 KiB; stage rows are 128 bytes, so every
+// global_load_lds_dwordx4 wave instruction moves eight full 128-byte lines.
+//
+// Loads use the scalar-base form: the tile's base address and K position live
+// in SGPRs, the per-lane byte offsets (row clamp and chunk swizzle folded in)
+// are computed once per tile, so a load costs two scalar moves and no VALU work.
+//
+// Software pipeline of one wave (the only wave on its SIMD): the fragments of
+// K slice s+1 are read while the 16 MFMAs of slice s issue; the next tile's
+// 16 load instructions are spread over slices 0-2; the barrier that publishes
+// the next tile sits in the middle of slice 3, so the first fragments of the
+// next tile are in flight under the last 8 MFMAs of the current one.
+template <typename T_>
+struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
+  using Base = MfmaTileLayout<T_, 2, 4>;
+  using T = T_;
+  using Op = typename Base::Op;
+  using V8 = typename Base::V8;
+  using Acc = typename Base::Acc;
+  using Base::kTile;
+  using Base::kTM;
+  using Base::kTN;
+  using Base::lane;
+  using Base::wave;
+  using Base::wm;
+  using Base::wn;
+  static constexpr int kBK = 64;
+  static constexpr int kRowBytes = kBK * 2;                  // 128
+  static constexpr int kOperandBytes = kTile * kRowBytes;    // 32768
+  static constexpr int kStageBytes = 2 * kOperandBytes;      // 65536
+  static constexpr int kSmemBytes = 2 * kStageBytes;         // 131072
+  static constexpr int kLoadsPerOperand = 8;                 // per wave per tile
+
+  static __device__ __forceinline__ void load_to_lds(unsigned lds_addr, unsigned byte_offset,
+                                                     const char* base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(byte_offset), "s"(base)
+                 : "memory", "m0");
+  }
+
+  struct Frags { V8 a[kTM]; V8 b[kTN]; };
+
+  __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
+                                           int a_rows, const T* __restrict__ B, int64_t ldb,
+                                           int b_row0, int b_rows, int k_begin, int k_end,
+                                           Acc& acc, char* smem) const {
+    // loader role: this wave fills rows [64*wave, 64*wave+64) of both operands,
+    // eight rows (1 KiB) per instruction; lane i lands in row i/8, slot i%8
+    unsigned aoff[kLoadsPerOperand], boff[kLoadsPerOperand];
+#pragma unroll
+    for (int j = 0; j < kLoadsPerOperand; ++j) {
+      const int r = wave * 64 + j * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ ((r >> 1) & 7);
+      const int ar = min(a_row0 + r, a_rows - 1) - a_row0;
+      const int br = min(b_row0 + r, b_rows - 1) - b_row0;
+      aoff[j] = (unsigned)((int64_t)ar * lda * 2 + chunk * 16);
+      boff[j] = (unsigned)((int64_t)br * ldb * 2 + chunk * 16);
+    }
+    const char* abase = reinterpret_cast<const char*>(A + (int64_t)a_row0 * lda + k_begin);
+    const char* bbase = reinterpret_cast<const char*>(B + (int64_t)b_row0 * ldb + k_begin);
+    const unsigned lds0 = (unsigned)(uintptr_t)smem;
+    const unsigned fill =
+        __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(wave * 64 * kRowBytes));
+
+    // load number q (0..15) of K tile `tile` into `stage`: even q -> operand A,
+    // odd q -> operand B, instruction q/2 of this wave's eight per operand
+    auto issue_one = [&](int stage, int tile, int q) {
+      const unsigned dst = fill + (unsigned)(stage * kStageBytes) + (unsigned)((q >> 1) * 8 * kRowBytes);
+      if (q & 1) {
+        load_to_lds(dst + kOperandBytes, boff[q >> 1], bbase + (int64_t)tile * kRowBytes);
+      } else {
+        load_to_lds(dst, aoff[q >> 1], abase + (int64_t)tile * kRowBytes);
+      }
+    };
+
+    // consumer role: fragment addresses of this wave's 128x128 sub-tile
+    const int swz = (lane >> 1) & 7;
+    const int hi = lane >> 5;
+    const int a_frag = (wm * 128 + (lane & 31)) * kRowBytes;
+    const int b_frag = kOperandBytes + (wn * 128 + (lane & 31)) * kRowBytes;
+
+    auto read_a = [&](Frags& f, int stage, int ks, int tm) {
+      const int slot = ((2 * ks + hi) ^ swz) * 16;
+      f.a[tm] = __builtin_bit_cast(
+          V8, *reinterpret_cast<const uint4*>(smem + stage * kStageBytes + a_frag +
+                                              tm * 32 * kRowBytes + slot));
+    };
+    auto read_b = [&](Frags& f, int stage, int ks, int tn) {
+      const int slot = ((2 * ks + hi) ^ swz) * 16;
+      f.b[tn] = __builtin_bit_cast(
+          V8, *reinterpret_cast<const uint4*>(smem + stage * kStageBytes + b_frag +
+                                              tn * 32 * kRowBytes + slot));
+    };
+    // fragment r (0..7) of a slice in the order the next slice consumes them:
+    // b0..b3 first (every MFMA group needs all four), then a0..a3
+    auto read_frag = [&](Frags& f, int stage, int ks, int r) {
+      if (r < 4) read_b(f, stage, ks, r); else read_a(f, stage, ks, r - 4);
+    };
+    auto mma_group = [&](const Frags& f, int tm) {
+#pragma unroll
+      for (int tn = 0; tn < kTN; ++tn) acc.c[tm][tn] = Op::mma(f.a[tm], f.b[tn], acc.c[tm][tn]);
+    };
+
+    // One K step = 16 groups of 4 MFMAs (slice s = g/4, A block g%4).  Every
+    // group also carries two LDS fragment reads of the next slice and, in the
+    // first half of the step, two of the next tile's 16 load instructions, so
+    // neither the LDS nor the vector-memory issue ever comes in bursts that
+    // would hold up this wave's (in-order) MFMA issue.  Loads 0..3 of tile
+    // k+2 go out right after the barrier of step k, loads 4..15 in the first
+    // six groups of step k+1; the last load is then 40 MFMAs (~1300 cycles)
+    // ahead of the barrier that needs it.
+    const int nk = (k_end - k_begin) / kBK;
+    auto step = [&](int k, Frags& fa, Frags& fb, auto has_next_tag) {
+      constexpr bool kHasNext = decltype(has_next_tag)::value;
+      const int cur = k & 1;
+      const int nxt = cur ^ 1;
+#pragma unroll
+      for (int g = 0; g < 16; ++g) {
+        const int sl = g >> 2;
+        const int q = g & 3;
+        Frags& fcur = (sl & 1) ? fb : fa;
+        Frags& fnext = (sl & 1) ? fa : fb;
+        if (kHasNext && g < 6) {
+          issue_one(nxt, k + 1, 4 + 2 * g);
+          issue_one(nxt, k + 1, 5 + 2 * g);
+        }
+        if (sl < 3) {
+          read_frag(fnext, cur, sl + 1, 2 * q);
+          read_frag(fnext, cur, sl + 1, 2 * q + 1);
+        } else if (kHasNext) {
+          if (q == 2) {
+            // tile k+1 is complete and visible from here on; stage `cur` is free
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (k + 2 < nk) {
+              issue_one(cur, k + 2, 0);
+              issue_one(cur, k + 2, 1);
+            }
+#pragma unroll
+            for (int r = 0; r < 5; ++r) read_frag(fnext, nxt, 0, r);
+          } else if (q == 3) {
+            if (k + 2 < nk) {
+              issue_one(cur, k + 2, 2);
+              issue_one(cur, k + 2, 3);
+            }
+#pragma unroll
+            for (int r = 5; r < 8; ++r) read_frag(fnext, nxt, 0, r);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mma_group(fcur, q);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+
+#pragma unroll
+    for (int q = 0; q < 16; ++q) issue_one(0, 0, q);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (nk > 1) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) issue_one(1, 1, q);
+    }
+    Frags f0, f1;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) read_frag(f0, 0, 0, r);
+    // a step consumes slices from f0,f1,f0,f1 and leaves the next tile's slice 0 in f0
+    for (int k = 0; k + 1 < nk; ++k) step(k, f0, f1, std::true_type{});
+    step(nk - 1, f0, f1, std::false_type{});
     __syncthreads();
   }
 };

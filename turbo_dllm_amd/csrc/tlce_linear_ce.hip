@@ -10,6 +10,8 @@
 //             panel, one contraction accumulates grad_hidden in float32 and
 //             one writes the panel's rows of grad_weight, complete, in dtype.
 // Nothing here allocates or synchronises.
+#include <stdlib.h>
+
 #include <algorithm>
 #include <vector>
 
@@ -80,7 +82,7 @@ constexpr int64_t kDefaultPanelBytes = 1ll << 30;
 constexpr int kTargetWorkgroups = 1024;  // 4 per CU on a 256-CU MI355X
 
 struct Plan {
-  int engine;  // 2 = direct-to-LDS MFMA, 1 = register-staged MFMA, 0 = generic
+  int engine;  // 3/2 = direct-to-LDS MFMA (4/8 waves), 1 = register-staged MFMA, 0 = generic
   int tile;
   int bk;
   int64_t mp, vp;
@@ -94,10 +96,18 @@ struct Plan {
 Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_grad,
                int64_t panel_bytes) {
   Plan p;
-  // 2: direct-to-LDS MFMA (h % 32 == 0), 1: register-staged MFMA (h % 8 == 0), 0: generic
-  p.engine = (dtype == TLCE_DTYPE_F32 || (h % 8) != 0) ? 0 : ((h % 32) == 0 ? 2 : 1);
+  // 3: four-wave direct-to-LDS MFMA (h % 64 == 0), 2: eight-wave direct-to-LDS MFMA
+  // (h % 32 == 0), 1: register-staged MFMA (h % 8 == 0), 0: generic
+  if (dtype == TLCE_DTYPE_F32 || (h % 8) != 0) p.engine = 0;
+  else if ((h % 64) == 0) p.engine = 3;
+  else if ((h % 32) == 0) p.engine = 2;
+  else p.engine = 1;
+  if (const char* forced = getenv("TLCE_FORCE_ENGINE")) {
+    const int e = atoi(forced);           // debugging aid: only to a less demanding engine
+    if (e >= 0 && e < p.engine) p.engine = e;
+  }
   p.tile = p.engine ? 256 : 64;
-  p.bk = p.engine == 2 ? 32 : (p.engine == 1 ? 64 : 16);
+  p.bk = p.engine == 3 ? 64 : (p.engine == 2 ? 32 : (p.engine == 1 ? 64 : 16));
   const int64_t mm = std::max<int64_t>(m, 1);
   p.mp = round_up(mm, p.tile);
   p.vp = round_up(v, p.tile);
@@ -390,6 +400,10 @@ using namespace tlce;
 
 #define TLCE_DISPATCH(plan, dtype, CALL)                                                  \
   do {                                                                                    \
+    if ((plan).engine == 3) {                                                             \
+      if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaDirect4Engine<__bf16>; return CALL; } \
+      { using E = MfmaDirect4Engine<_Float16>; return CALL; }                             \
+    }                                                                                     \
     if ((plan).engine == 2) {                                                             \
       if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaDirectEngine<__bf16>; return CALL; } \
       { using E = MfmaDirectEngine<_Float16>; return CALL; }                              \
