@@ -432,11 +432,21 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
     // odd q -> operand B, instruction q/2 of this wave's eight per operand
     auto issue_one = [&](int stage, int tile, int q) {
       const unsigned dst = fill + (unsigned)(stage * kStageBytes) + (unsigned)((q >> 1) * 8 * kRowBytes);
+#if defined(TLCE_EXP_SAMELINE)
+      // every load re-reads this wave's first 1 KiB: stays in the vector L1
+      if (q & 1) load_to_lds(dst + kOperandBytes, (unsigned)(lane * 16), bbase);
+      else load_to_lds(dst, (unsigned)(lane * 16), abase);
+#elif defined(TLCE_EXP_SAMETILE)
+      // no K advance: the tile's first 64-wide slab again (L2 hits)
+      if (q & 1) load_to_lds(dst + kOperandBytes, boff[q >> 1], bbase);
+      else load_to_lds(dst, aoff[q >> 1], abase);
+#else
       if (q & 1) {
         load_to_lds(dst + kOperandBytes, boff[q >> 1], bbase + (int64_t)tile * kRowBytes);
       } else {
         load_to_lds(dst, aoff[q >> 1], abase + (int64_t)tile * kRowBytes);
       }
+#endif
     };
 
     // consumer role: fragment addresses of this wave's 128x128 sub-tile
@@ -462,60 +472,62 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
     auto read_frag = [&](Frags& f, int stage, int ks, int r) {
       if (r < 4) read_b(f, stage, ks, r); else read_a(f, stage, ks, r - 4);
     };
-    auto mma_group = [&](const Frags& f, int tm) {
-#pragma unroll
-      for (int tn = 0; tn < kTN; ++tn) acc.c[tm][tn] = Op::mma(f.a[tm], f.b[tn], acc.c[tm][tn]);
-    };
 
-    // One K step = 16 groups of 4 MFMAs (slice s = g/4, A block g%4).  Every
-    // group also carries two LDS fragment reads of the next slice and, in the
-    // first half of the step, two of the next tile's 16 load instructions, so
-    // neither the LDS nor the vector-memory issue ever comes in bursts that
-    // would hold up this wave's (in-order) MFMA issue.  Loads 0..3 of tile
-    // k+2 go out right after the barrier of step k, loads 4..15 in the first
-    // six groups of step k+1; the last load is then 40 MFMAs (~1300 cycles)
-    // ahead of the barrier that needs it.
+    // One K step = 64 MFMAs = 16 groups of 4 (slice sl = g/4, A block q = g%4,
+    // B block t = 0..3).  A wave issues in order and an MFMA occupies its pipe
+    // for 32 cycles, so everything else has to fit into those shadows a few
+    // instructions at a time: after every MFMA at most one LDS fragment read
+    // or one load instruction (three scalar + one vector instruction) follows.
+    //   reads : the 8 fragments of the next slice, two per group (slots 0, 2);
+    //           the next tile's slice 0 is read in the two groups after the
+    //           barrier (5 + 3);
+    //   loads : of the next tile's 16, six go out right after the barrier of
+    //           the previous step, ten in groups 0..9 (slot 1) - the last one
+    //           16 MFMAs (~500 cycles) before the barrier that waits for it.
     const int nk = (k_end - k_begin) / kBK;
     auto step = [&](int k, Frags& fa, Frags& fb, auto has_next_tag) {
       constexpr bool kHasNext = decltype(has_next_tag)::value;
       const int cur = k & 1;
       const int nxt = cur ^ 1;
+      const bool more = (k + 2 < nk);
 #pragma unroll
       for (int g = 0; g < 16; ++g) {
         const int sl = g >> 2;
         const int q = g & 3;
         Frags& fcur = (sl & 1) ? fb : fa;
         Frags& fnext = (sl & 1) ? fa : fb;
-        if (kHasNext && g < 6) {
-          issue_one(nxt, k + 1, 4 + 2 * g);
-          issue_one(nxt, k + 1, 5 + 2 * g);
+        const bool after_barrier = kHasNext && sl == 3 && q >= 2;
+        if (kHasNext && sl == 3 && q == 2) {
+          // tile k+1 is complete and visible from here on; stage `cur` is free
+#ifndef TLCE_EXP_NOWAIT
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+#ifndef TLCE_EXP_NOBARRIER
+          __syncthreads();
+#endif
         }
-        if (sl < 3) {
-          read_frag(fnext, cur, sl + 1, 2 * q);
-          read_frag(fnext, cur, sl + 1, 2 * q + 1);
-        } else if (kHasNext) {
-          if (q == 2) {
-            // tile k+1 is complete and visible from here on; stage `cur` is free
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            __syncthreads();
-            if (k + 2 < nk) {
-              issue_one(cur, k + 2, 0);
-              issue_one(cur, k + 2, 1);
-            }
 #pragma unroll
-            for (int r = 0; r < 5; ++r) read_frag(fnext, nxt, 0, r);
-          } else if (q == 3) {
-            if (k + 2 < nk) {
-              issue_one(cur, k + 2, 2);
-              issue_one(cur, k + 2, 3);
+        for (int t = 0; t < kTN; ++t) {
+          acc.c[q][t] = Op::mma(fcur.a[q], fcur.b[t], acc.c[q][t]);
+          if (sl < 3) {
+            if (t == 0) read_frag(fnext, cur, sl + 1, 2 * q);
+            if (t == 2) read_frag(fnext, cur, sl + 1, 2 * q + 1);
+#ifndef TLCE_EXP_NOLOAD
+            if (kHasNext && t == 1 && g < 10) issue_one(nxt, k + 1, 6 + g);
+#endif
+          } else if (after_barrier) {
+            if (q == 2) {
+              if (t == 0) { read_frag(fnext, nxt, 0, 0); read_frag(fnext, nxt, 0, 1); }
+              else read_frag(fnext, nxt, 0, t + 1);
+            } else {
+              if (t < 3) read_frag(fnext, nxt, 0, 5 + t);
             }
-#pragma unroll
-            for (int r = 5; r < 8; ++r) read_frag(fnext, nxt, 0, r);
+#ifndef TLCE_EXP_NOLOAD
+            if (t >= 1 && more) issue_one(cur, k + 2, (q - 2) * 3 + (t - 1));
+#endif
           }
+          __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        mma_group(fcur, q);
-        __builtin_amdgcn_sched_barrier(0);
       }
     };
 
@@ -525,7 +537,7 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
     __syncthreads();
     if (nk > 1) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) issue_one(1, 1, q);
+      for (int q = 0; q < 6; ++q) issue_one(1, 1, q);
     }
     Frags f0, f1;
 #pragma unroll

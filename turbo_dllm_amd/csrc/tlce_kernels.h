@@ -321,6 +321,9 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
     }
   }
 
+#ifdef TLCE_EXP_NOSTORE
+  if (p.m != 123457) return;
+#endif
   T* g_out = static_cast<T*>(p.g);
   T* gt_out = static_cast<T*>(p.gt);
   const int prow = pv * E::kTile;  // first panel column of this tile
@@ -340,11 +343,14 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   }
 }
 
-// C[i][j] (op)= sum_k A[i][k] * B[j][k]  — the two gradient contractions:
-//   grad_hidden: A = G panel [mp, Kv], B = weight^T [h, Kv]   -> C float32 [mp, h]
-//   grad_weight: A = GT panel [pv, Km], B = hidden^T [h, Km]  -> C dtype   [pv, h]
+// C[j][i] (op)= sum_k A[i][k] * B[j][k]  - the two gradient contractions, with
+// the "A rows" on the output's contiguous axis (the hidden dimension):
+//   grad_hidden: A = weight^T [h, Kv], B = G panel [mp, Kv]   -> C float32 [mp, h]
+//   grad_weight: A = hidden^T [h, Km], B = GT panel [pv, Km]  -> C dtype   [pv, h]
 // (project_grad_hidden / accumulate_grad_weight, fused_linear_ce_cuda.cu:676-791,
-// with float32 accumulation).  blockIdx.y selects a K split.
+// with float32 accumulation).  A thread holds runs of 4 consecutive A rows per
+// owned B row, so it reads and writes the output 16 (float32) or 8 (dtype)
+// bytes at a time.  blockIdx.y selects a K split.
 enum { kStoreF32 = 0, kAddF32 = 1, kAtomicF32 = 2, kStoreT = 3 };
 
 struct GemmArgs {
@@ -356,8 +362,8 @@ struct GemmArgs {
   int b_rows;
   int k;            // padded K, multiple of the engine's BK
   int k_per_split;  // multiple of BK
-  int ni, nj;
-  void* c;
+  int ni, nj;       // tiles along A rows / B rows
+  void* c;          // [c_rows, ldc]: row = B row, column = A row
   int64_t ldc;
   int c_rows, c_cols;
   int mode;
@@ -382,24 +388,54 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
                static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows, k_begin, k_end, acc,
                smem);
 
+#ifdef TLCE_EXP_NOSTORE
+  if (p.k != 123457) return;
+#endif
+  // runs of 4 can be moved as one vector when every row start keeps them aligned
+  const bool vec_ok = (p.ldc % 4 == 0) && (p.c_cols % 4 == 0) &&
+                      (reinterpret_cast<uintptr_t>(p.c) % 16 == 0);
 #pragma unroll
   for (int j = 0; j < E::kCols; ++j) {
-    const int col = tj * E::kTile + eng.col(j);
-    if (col >= p.c_cols) continue;
+    const int out_row = tj * E::kTile + eng.col(j);
+    if (out_row >= p.c_rows) continue;
 #pragma unroll
-    for (int i = 0; i < E::kRows; ++i) {
-      const int row = ti * E::kTile + eng.row(i);
-      if (row >= p.c_rows) continue;
-      const int64_t o = (int64_t)row * p.ldc + col;
-      const float val = E::get(acc, j, i);
-      if (p.mode == kStoreT) {
-        static_cast<T*>(p.c)[o] = from_float<T>(val);
-      } else if (p.mode == kStoreF32) {
-        static_cast<float*>(p.c)[o] = val;
-      } else if (p.mode == kAddF32) {
-        static_cast<float*>(p.c)[o] += val;
+    for (int i = 0; i < E::kRows; i += 4) {
+      const int out_col = ti * E::kTile + eng.row(i);
+      if (out_col >= p.c_cols) continue;
+      const int64_t o = (int64_t)out_row * p.ldc + out_col;
+      const float v0 = E::get(acc, j, i), v1 = E::get(acc, j, i + 1);
+      const float v2 = E::get(acc, j, i + 2), v3 = E::get(acc, j, i + 3);
+      if (vec_ok) {
+        if (p.mode == kStoreT) {
+          store4<T>(static_cast<T*>(p.c) + o, v0, v1, v2, v3);
+        } else if (p.mode == kStoreF32) {
+          *reinterpret_cast<float4*>(static_cast<float*>(p.c) + o) = make_float4(v0, v1, v2, v3);
+        } else if (p.mode == kAddF32) {
+          float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.c) + o);
+          float4 old = *dst;
+          *dst = make_float4(old.x + v0, old.y + v1, old.z + v2, old.w + v3);
+        } else {
+          float* dst = static_cast<float*>(p.c) + o;
+          atomicAdd(dst, v0);
+          atomicAdd(dst + 1, v1);
+          atomicAdd(dst + 2, v2);
+          atomicAdd(dst + 3, v3);
+        }
       } else {
-        atomicAdd(static_cast<float*>(p.c) + o, val);
+        const float vals[4] = {v0, v1, v2, v3};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (out_col + e >= p.c_cols) continue;
+          if (p.mode == kStoreT) {
+            static_cast<T*>(p.c)[o + e] = from_float<T>(vals[e]);
+          } else if (p.mode == kStoreF32) {
+            static_cast<float*>(p.c)[o + e] = vals[e];
+          } else if (p.mode == kAddF32) {
+            static_cast<float*>(p.c)[o + e] += vals[e];
+          } else {
+            atomicAdd(static_cast<float*>(p.c) + o + e, vals[e]);
+          }
+        }
       }
     }
   }

@@ -360,20 +360,20 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     if (int rc = launch_grad_logits<E>(ga, stream)) return rc;
 
     GemmArgs dh;
-    dh.a = g; dh.lda = p.vc; dh.a_rows = (int)p.mp;
-    dh.b = wt + v0; dh.ldb = p.vp; dh.b_rows = (int)h;
+    dh.a = wt + v0; dh.lda = p.vp; dh.a_rows = (int)h;
+    dh.b = g; dh.ldb = p.vc; dh.b_rows = (int)p.mp;
     dh.k = (int)width; dh.k_per_split = 0;
-    dh.ni = p.n_ttiles; dh.nj = p.n_htiles;
+    dh.ni = p.n_htiles; dh.nj = p.n_ttiles;
     dh.c = acc32; dh.ldc = h; dh.c_rows = (int)p.mp; dh.c_cols = (int)h;
     dh.mode = (p.dh_ksplit > 1) ? kAtomicF32 : (panel == 0 ? kStoreF32 : kAddF32);
     if (int rc = launch_gemm<E>(dh, p.dh_ksplit, kClassGradHidden, stream)) return rc;
 
     if (weight_grad) {
       GemmArgs dw;
-      dw.a = gt; dw.lda = p.mp; dw.a_rows = (int)width;
-      dw.b = ht; dw.ldb = p.mp; dw.b_rows = (int)h;
+      dw.a = ht; dw.lda = p.mp; dw.a_rows = (int)h;
+      dw.b = gt; dw.ldb = p.mp; dw.b_rows = (int)width;
       dw.k = (int)p.mp; dw.k_per_split = 0;
-      dw.ni = (int)(width / p.tile); dw.nj = p.n_htiles;
+      dw.ni = p.n_htiles; dw.nj = (int)(width / p.tile);
       dw.c = static_cast<T*>(grad_weight) + v0 * h; dw.ldc = h;
       dw.c_rows = (int)rows_valid; dw.c_cols = (int)h;
       dw.mode = kStoreT;
