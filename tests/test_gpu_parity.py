@@ -353,6 +353,32 @@ def test_panel_count_does_not_change_results(gpu_device):
     assert oracle.relative_max_error(multi[1], base[1].double()) < 1e-2   # grad_hidden: split differs
 
 
+@pytest.mark.parametrize("m,h,v,panel_tiles", [
+    (5, 64, 64, 0), (64, 128, 1024, 0), (100, 128, 1088, 2), (300, 256, 2048, 3),
+    (513, 192, 4160, 4), (1000, 320, 1536, 0),
+])
+def test_direct_engine_in_place_operands(gpu_device, m, h, v, panel_tiles):
+    # h % 64 == 0 and v % 64 == 0: the gradient contractions read weight, hidden and the
+    # logit-gradient panel K-major (no transposed copies); m % 64 != 0 pads hidden rows,
+    # v % 256 != 0 ends a panel inside a tile, panel_tiles forces several panels
+    say("in-place operands", m, h, v, panel_tiles)
+    torch.manual_seed(m + v)
+    hidden = torch.randn(m + 7, h).bfloat16()
+    weight = (torch.randn(v, h) * 0.2).bfloat16()
+    labels = torch.randint(0, v, (m + 7,))
+    labels[torch.randperm(m + 7)[:7]] = -100
+    old = native.PANEL_BYTES
+    try:
+        if panel_tiles:
+            mp = -(-m // 256) * 256
+            native.PANEL_BYTES = mp * 256 * 2 * panel_tiles
+        check_against_oracle(gpu_device, hidden, weight, labels, reduction="mean")
+        check_against_oracle(gpu_device, hidden, weight, labels, reduction="sum", frozen=True,
+                             logit_softcap=4.0)
+    finally:
+        native.PANEL_BYTES = old
+
+
 # ------------------------------------------- benchmark configurations, scaled ----
 @pytest.mark.parametrize("name", list(workloads.CONFIGS))
 def test_scaled_benchmark_configurations(gpu_device, name):

@@ -127,7 +127,7 @@ def query_plan(m: int, h: int, v: int, dtype_code: int, compute_weight_grad: boo
         "tlce_query_plan",
     )
     return {
-        "engine": {0: "generic", 1: "mfma", 2: "mfma_direct", 3: "mfma_direct4"}[engine.value],
+        "engine": {0: "generic", 1: "mfma", 2: "mfma_direct"}[engine.value],
         "tile": tile.value,
         "forward_vocab_splits": splits.value,
         "panel_columns": columns.value,

@@ -121,6 +121,7 @@ struct MfmaEngine : MfmaTileLayout<T_> {
   static constexpr int kRowBytes = kBK * 2;                  // 128
   static constexpr int kStageBytes = 2 * kTile * kRowBytes;  // 65536
   static constexpr int kSmemBytes = 2 * kStageBytes;         // 131072
+  static constexpr bool kHasKMajor = false;
 
   // acc += A[a_row0 .. +256, k_begin .. k_end) * B[b_row0 .. +256, same K)^T.
   // Rows past a_rows / b_rows are clamped to the last valid row (their results
@@ -214,167 +215,54 @@ struct MfmaEngine : MfmaTileLayout<T_> {
   }
 };
 
-// Direct-to-LDS engine: the operand tiles go global -> LDS with
-// global_load_lds_dwordx4 (no VGPR staging, no ds_write), through a ring of
-// four 32-wide K stages (4 x 32 KiB), so a tile is requested three K steps
-// before it is consumed and HBM/L2 latency hides behind ~48 MFMAs per wave.
-// Needs K (k_end - k_begin) to be a multiple of 32.
-//
-// A stage row is 64 bytes = four 16-byte chunks; chunk c of row r sits in slot
-// c ^ ((r >> 2) & 3): the 16 lanes of one LDS read phase (16 rows, one chunk)
-// then cover all 64 banks.  A wave's load instruction fills 1 KiB = 16 rows:
-// lane i lands in row i/4, slot i%4, so it fetches logical chunk
-// (i%4) ^ ((i>>4)&3) of that row.
-//
-// Ordering: loads are counted per wave by vmcnt and complete in order.  Before
-// using tile k a wave waits until at most the loads of the (up to two) younger
-// tiles are outstanding, then the workgroup barrier publishes every wave's
-// part of tile k and retires stage (k-1)%4, which the loads of tile k+3 refill.
-template <typename T_>
-struct MfmaDirectEngine : MfmaTileLayout<T_> {
-  using Base = MfmaTileLayout<T_>;
-  using T = T_;
-  using Op = typename Base::Op;
-  using V8 = typename Base::V8;
-  using Acc = typename Base::Acc;
-  using Base::kTile;
-  using Base::kTM;
-  using Base::kTN;
-  using Base::lane;
-  using Base::wave;
-  using Base::wm;
-  using Base::wn;
-  static constexpr int kBK = 32;
-  static constexpr int kStages = 4;
-  static constexpr int kRowBytes = kBK * 2;                  // 64
-  static constexpr int kOperandBytes = kTile * kRowBytes;    // 16384
-  static constexpr int kStageBytes = 2 * kOperandBytes;      // 32768
-  static constexpr int kSmemBytes = kStages * kStageBytes;   // 131072
-
-  static __device__ __forceinline__ void load_to_lds(unsigned lds_addr, const T* src) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
-                 :
-                 : "s"(lds_addr), "v"(src)
-                 : "memory", "m0");
-  }
-
-  __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
-                                           int a_rows, const T* __restrict__ B, int64_t ldb,
-                                           int b_row0, int b_rows, int k_begin, int k_end,
-                                           Acc& acc, char* smem) const {
-    // loader role: this wave fills rows [32*wave, 32*wave+32) of both operands
-    const int lrow = lane >> 2;
-    const int chunk = (lane & 3) ^ ((lane >> 4) & 3);
-    const T* ap[2];
-    const T* bp[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int r = wave * 32 + j * 16 + lrow;
-      const int ar = min(a_row0 + r, a_rows - 1);
-      const int br = min(b_row0 + r, b_rows - 1);
-      ap[j] = A + (int64_t)ar * lda + k_begin + chunk * 8;
-      bp[j] = B + (int64_t)br * ldb + k_begin + chunk * 8;
-    }
-    const unsigned lds0 = (unsigned)(uintptr_t)smem;
-    const unsigned fill =
-        __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(wave * 32 * kRowBytes));
-
-    auto issue = [&](int stage) {
-      const unsigned dst = fill + (unsigned)(stage * kStageBytes);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        load_to_lds(dst + j * 16 * kRowBytes, ap[j]);
-        load_to_lds(dst + kOperandBytes + j * 16 * kRowBytes, bp[j]);
-        ap[j] += kBK;
-        bp[j] += kBK;
-      }
-    };
-
-    // consumer role: fragment addresses of this wave's 128x64 sub-tile
-    const int swz = (lane >> 2) & 3;
-    const int hi = lane >> 5;
-    const int a_frag = (wm * 128 + (lane & 31)) * kRowBytes;
-    const int b_frag = kOperandBytes + (wn * 64 + (lane & 31)) * kRowBytes;
-
-    // Fragments of one 16-wide K slice: 4 A blocks + 2 B blocks, 24 VGPRs.
-    struct Frags { V8 a[kTM]; V8 b[kTN]; };
-    auto read_slice = [&](Frags& f, int stage, int ks) {
-      const char* base = smem + stage * kStageBytes;
-      const int slot = ((2 * ks + hi) ^ swz) * 16;
-#pragma unroll
-      for (int tm = 0; tm < kTM; ++tm)
-        f.a[tm] = __builtin_bit_cast(
-            V8, *reinterpret_cast<const uint4*>(base + a_frag + tm * 32 * kRowBytes + slot));
-#pragma unroll
-      for (int tn = 0; tn < kTN; ++tn)
-        f.b[tn] = __builtin_bit_cast(
-            V8, *reinterpret_cast<const uint4*>(base + b_frag + tn * 32 * kRowBytes + slot));
-    };
-    auto mma_slice = [&](const Frags& f) {
-#pragma unroll
-      for (int tm = 0; tm < kTM; ++tm)
-#pragma unroll
-        for (int tn = 0; tn < kTN; ++tn) acc.c[tm][tn] = Op::mma(f.a[tm], f.b[tn], acc.c[tm][tn]);
-    };
-
-    // Software pipeline: the fragments of the next K slice are always in flight
-    // while the MFMAs of the current one issue, also across K steps.  The
-    // barrier that publishes tile k+1 sits in the middle of step k, after the
-    // last LDS reads of tile k have been issued and before slice 0 of tile k+1
-    // is read; the stage refilled after it, (k+3)%4 == (k-1)%4, was last read
-    // in step k-1.
-    const int nk = (k_end - k_begin) / kBK;
-#pragma unroll
-    for (int t = 0; t < kStages - 1; ++t)
-      if (t < nk) issue(t);
-    if (nk >= 3) {
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    } else if (nk == 2) {
-      asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __syncthreads();
-    Frags f0, f1;
-    read_slice(f0, 0, 0);
-    for (int k = 0; k + 1 < nk; ++k) {
-      read_slice(f1, k & (kStages - 1), 1);
-      __builtin_amdgcn_sched_barrier(0);   // keep the LDS reads ahead of the MFMA batch
-      mma_slice(f0);
-      // tile k+1 must have landed; tile k+2 (if any) may stay in flight
-      if (k + 2 < nk) {
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
-      __syncthreads();
-      if (k + kStages - 1 < nk) issue((k + kStages - 1) & (kStages - 1));
-      read_slice(f0, (k + 1) & (kStages - 1), 0);
-      __builtin_amdgcn_sched_barrier(0);
-      mma_slice(f1);
-    }
-    read_slice(f1, (nk - 1) & (kStages - 1), 1);
-    mma_slice(f0);
-    mma_slice(f1);
-    __syncthreads();
-  }
-};
-
 // Four-wave direct-to-LDS engine (K multiple of 64): 256 threads, each wave a
 // 128x128 sub-tile (4x4 MFMA blocks, 256 accumulator registers, one wave per
-// SIMD), which halves the LDS fragment traffic per MFMA of the 8-wave layout.
-// Two 64-wide K stages of 64 KiB; stage rows are 128 bytes, so every
-// global_load_lds_dwordx4 wave instruction moves eight full 128-byte lines.
+// SIMD).  Operands go global -> LDS with global_load_lds_dwordx4 (no VGPR
+// staging, no ds_write) into two 64-wide K stages of 64 KiB; every wave load
+// instruction moves 1 KiB made of full 128-byte (or 512-byte) row segments.
 //
-// Loads use the scalar-base form: the tile's base address and K position live
-// in SGPRs, the per-lane byte offsets (row clamp and chunk swizzle folded in)
-// are computed once per tile, so a load costs two scalar moves and no VALU work.
+// Either operand can be stored in one of two ways:
+//   K-contiguous  X[row][k]  (the projection's hidden and weight rows, the
+//                 logit-gradient panel as seen by grad_hidden);
+//   K-major       X[k][row]  (weight as seen by grad_hidden, hidden and the
+//                 logit-gradient panel as seen by grad_weight), read from LDS
+//                 with the transposing ds_read_b64_tr_b16, so no transposed
+//                 copy of any matrix is ever made in HBM.
 //
-// Software pipeline of one wave (the only wave on its SIMD): the fragments of
-// K slice s+1 are read while the 16 MFMAs of slice s issue; the next tile's
-// 16 load instructions are spread over slices 0-2; the barrier that publishes
-// the next tile sits in the middle of slice 3, so the first fragments of the
-// next tile are in flight under the last 8 MFMAs of the current one.
+// LDS layouts of one operand stage (32 KiB):
+//   K-contiguous: 256 rows x 128 B; 16-byte chunk c of row r in slot
+//                 c ^ ((r >> 1) & 7).
+//   K-major:      64 K rows x 512 B; 16-byte chunk c of K row k in slot
+//                 c ^ (2 * ((k & 3) | (((k >> 3) & 1) << 2))); the even XOR
+//                 keeps 32-byte pairs together for the transposing read.
+// ds_read_b64_tr_b16 works on groups of 16 lanes: lane i of a group addresses
+// 4 consecutive elements, and lane l receives element l%4 of the chunks of
+// lanes l/4, 4 + l/4, 8 + l/4, 12 + l/4.  With lane i addressing K row i/4,
+// columns 4*(i%4).. of a 4 x 16 block, lane l ends up with 4 consecutive K
+// values of column l: half an MFMA fragment.
+//
+// Loads use the scalar-base form: tile base and K position live in SGPRs, the
+// per-lane byte offsets (row clamp and slot swizzle folded in) are computed
+// once per tile, so a load costs three scalar instructions and no VALU work.
+//
+// Software pipeline of one wave (the only wave on its SIMD; it issues in
+// order and an MFMA occupies its pipe for 32 cycles): one K step = 64 MFMAs
+// = 16 groups of 4 (slice sl = g/4, A block q = g%4, B block t).  After every
+// MFMA at most one fragment read and one load instruction follow.
+//   reads : the fragments of the next slice, spread over the groups of the
+//           current one; slice 0 of the next tile is read in the two groups
+//           after the barrier, which sits in the middle of slice 3;
+//   loads : of the next tile's 16, six go out right after the barrier of the
+//           previous step, ten in groups 0..9 - the last one 16 MFMAs before
+//           the barrier that waits for it.
+template <typename T>
+struct Operand {
+  const T* ptr;   // matrix base
+  int64_t ld;     // elements between consecutive stored rows
+  int row0;       // first tile row (K-contiguous) or first tile column (K-major)
+  int rows;       // valid rows / columns of the matrix; accesses beyond are clamped
+};
+
 template <typename T_>
 struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
   using Base = MfmaTileLayout<T_, 2, 4>;
@@ -390,11 +278,14 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
   using Base::wm;
   using Base::wn;
   static constexpr int kBK = 64;
-  static constexpr int kRowBytes = kBK * 2;                  // 128
-  static constexpr int kOperandBytes = kTile * kRowBytes;    // 32768
+  static constexpr int kOperandBytes = kTile * kBK * 2;      // 32768
   static constexpr int kStageBytes = 2 * kOperandBytes;      // 65536
   static constexpr int kSmemBytes = 2 * kStageBytes;         // 131072
-  static constexpr int kLoadsPerOperand = 8;                 // per wave per tile
+  static constexpr int kLoads = 8;                           // per wave, operand and K tile
+  static constexpr bool kHasKMajor = true;
+
+  typedef short v4s_t __attribute__((ext_vector_type(4)));
+  typedef short v8s_t __attribute__((ext_vector_type(8)));
 
   static __device__ __forceinline__ void load_to_lds(unsigned lds_addr, unsigned byte_offset,
                                                      const char* base) {
@@ -404,86 +295,130 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
                  : "memory", "m0");
   }
 
+  // Loader state of one operand: where this wave's eight 1 KiB pieces of a K
+  // tile come from and where they land.
+  struct Loader {
+    unsigned off[kLoads];   // per-lane byte offsets from the K tile's base
+    unsigned fill;          // LDS address of this wave's first piece in stage 0
+    const char* next;       // base address of the next K tile to request
+    int64_t step;           // bytes between consecutive K tiles
+  };
+
+  template <bool kKMajor>
+  __device__ __forceinline__ Loader make_loader(const Operand<T>& x, int k_begin, unsigned lds_op,
+                                                bool second_operand) const {
+    Loader ld;
+    (void)second_operand;
+    if (!kKMajor) {
+      // this wave fills tile rows [64w, 64w+64), eight rows per instruction
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) {
+        const int r = wave * 64 + j * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ ((r >> 1) & 7);
+        const int rr = min(x.row0 + r, x.rows - 1) - x.row0;
+        ld.off[j] = (unsigned)((int64_t)rr * x.ld * 2 + chunk * 16);
+      }
+      ld.fill = __builtin_amdgcn_readfirstlane(lds_op + (unsigned)(wave * 64 * 128));
+      ld.next = reinterpret_cast<const char*>(x.ptr + (int64_t)x.row0 * x.ld + k_begin);
+      ld.step = kBK * 2;
+    } else {
+      // this wave fills K rows [16w, 16w+16) of the slab, two rows per instruction
+      const int last_chunk = x.rows / 8 - 1 - x.row0 / 8;   // relative to the tile
+#pragma unroll
+      for (int j = 0; j < kLoads; ++j) {
+        const int kr = wave * 16 + j * 2 + (lane >> 5);
+        const int swz = 2 * ((kr & 3) | (((kr >> 3) & 1) << 2));
+        const int chunk = min((lane & 31) ^ swz, last_chunk);
+        ld.off[j] = (unsigned)((int64_t)kr * x.ld * 2 + chunk * 16);
+      }
+      ld.fill = __builtin_amdgcn_readfirstlane(lds_op + (unsigned)(wave * 16 * 512));
+      ld.next = reinterpret_cast<const char*>(x.ptr + (int64_t)k_begin * x.ld + x.row0);
+      ld.step = (int64_t)kBK * x.ld * 2;
+    }
+    return ld;
+  }
+
+  // Fragment addressing of one operand for this lane.
+  struct Reader {
+    int base[4];   // LDS byte offset of block 0..3 within the operand stage
+  };
+
+  template <bool kKMajor>
+  __device__ __forceinline__ Reader make_reader(int wave_block) const {
+    Reader rd;
+    if (!kKMajor) {
+      const int swz = (lane >> 1) & 7;
+      (void)swz;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) rd.base[b] = (wave_block * 128 + b * 32 + (lane & 31)) * 128;
+    } else {
+      const int g = lane >> 4;          // 16-lane group
+      const int i = lane & 15;
+      const int hi = g >> 1;
+      const int swz = 2 * ((i >> 2) | (hi << 2));
+      const int kr = 8 * hi + (i >> 2);  // K row within a 16-wide slice, first half
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int col = wave_block * 128 + b * 32 + 16 * (g & 1) + 4 * (i & 3);
+        const int slot = (col >> 3) ^ swz;
+        rd.base[b] = kr * 512 + slot * 16 + (col & 7) * 2;
+      }
+    }
+    return rd;
+  }
+
+  template <bool kKMajor>
+  __device__ __forceinline__ V8 read_frag(const char* op_stage, const Reader& rd, int ks,
+                                          int b) const {
+    if (!kKMajor) {
+      const int slot = ((2 * ks + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16;
+      return __builtin_bit_cast(V8, *reinterpret_cast<const uint4*>(op_stage + rd.base[b] + slot));
+    } else {
+      typedef __attribute__((address_space(3))) v4s_t* lds_v4s_ptr;
+      const char* p0 = op_stage + rd.base[b] + ks * 16 * 512;
+      const v4s_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (lds_v4s_ptr)(uintptr_t)(unsigned)(uintptr_t)p0);
+      const v4s_t hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+          (lds_v4s_ptr)(uintptr_t)(unsigned)(uintptr_t)(p0 + 4 * 512));
+      v8s_t v;
+      v[0] = lo[0]; v[1] = lo[1]; v[2] = lo[2]; v[3] = lo[3];
+      v[4] = hi4[0]; v[5] = hi4[1]; v[6] = hi4[2]; v[7] = hi4[3];
+      return __builtin_bit_cast(V8, v);
+    }
+  }
+
   struct Frags { V8 a[kTM]; V8 b[kTN]; };
 
-  __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
-                                           int a_rows, const T* __restrict__ B, int64_t ldb,
-                                           int b_row0, int b_rows, int k_begin, int k_end,
-                                           Acc& acc, char* smem) const {
-    // loader role: this wave fills rows [64*wave, 64*wave+64) of both operands,
-    // eight rows (1 KiB) per instruction; lane i lands in row i/8, slot i%8
-    unsigned aoff[kLoadsPerOperand], boff[kLoadsPerOperand];
-#pragma unroll
-    for (int j = 0; j < kLoadsPerOperand; ++j) {
-      const int r = wave * 64 + j * 8 + (lane >> 3);
-      const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-      const int ar = min(a_row0 + r, a_rows - 1) - a_row0;
-      const int br = min(b_row0 + r, b_rows - 1) - b_row0;
-      aoff[j] = (unsigned)((int64_t)ar * lda * 2 + chunk * 16);
-      boff[j] = (unsigned)((int64_t)br * ldb * 2 + chunk * 16);
-    }
-    const char* abase = reinterpret_cast<const char*>(A + (int64_t)a_row0 * lda + k_begin);
-    const char* bbase = reinterpret_cast<const char*>(B + (int64_t)b_row0 * ldb + k_begin);
+  // acc += A-tile * B-tile^T over K in [k_begin, k_end), a multiple of 64 wide.
+  // K-contiguous operand: tile rows row0 .. row0+256 of x (rows clamped to
+  // x.rows - 1).  K-major operand: tile columns row0 .. row0+256 of x (16-byte
+  // column chunks clamped to the last valid one; x.rows is a multiple of 8);
+  // all K rows in [k_begin, k_end) must exist.
+  template <bool kAKMajor, bool kBKMajor>
+  __device__ __forceinline__ void mainloop_ex(const Operand<T>& A, const Operand<T>& B,
+                                              int k_begin, int k_end, Acc& acc,
+                                              char* smem) const {
     const unsigned lds0 = (unsigned)(uintptr_t)smem;
-    const unsigned fill =
-        __builtin_amdgcn_readfirstlane(lds0 + (unsigned)(wave * 64 * kRowBytes));
+    Loader la = make_loader<kAKMajor>(A, k_begin, lds0, false);
+    Loader lb = make_loader<kBKMajor>(B, k_begin, lds0 + kOperandBytes, true);
+    const Reader ra = make_reader<kAKMajor>(wm);
+    const Reader rb = make_reader<kBKMajor>(wn);
 
-    // load number q (0..15) of K tile `tile` into `stage`: even q -> operand A,
-    // odd q -> operand B, instruction q/2 of this wave's eight per operand
-    auto issue_one = [&](int stage, int tile, int q) {
-      const unsigned dst = fill + (unsigned)(stage * kStageBytes) + (unsigned)((q >> 1) * 8 * kRowBytes);
-#if defined(TLCE_EXP_SAMELINE)
-      // every load re-reads this wave's first 1 KiB: stays in the vector L1
-      if (q & 1) load_to_lds(dst + kOperandBytes, (unsigned)(lane * 16), bbase);
-      else load_to_lds(dst, (unsigned)(lane * 16), abase);
-#elif defined(TLCE_EXP_SAMETILE)
-      // no K advance: the tile's first 64-wide slab again (L2 hits)
-      if (q & 1) load_to_lds(dst + kOperandBytes, boff[q >> 1], bbase);
-      else load_to_lds(dst, aoff[q >> 1], abase);
-#else
-      if (q & 1) {
-        load_to_lds(dst + kOperandBytes, boff[q >> 1], bbase + (int64_t)tile * kRowBytes);
-      } else {
-        load_to_lds(dst, aoff[q >> 1], abase + (int64_t)tile * kRowBytes);
-      }
-#endif
-    };
-
-    // consumer role: fragment addresses of this wave's 128x128 sub-tile
-    const int swz = (lane >> 1) & 7;
-    const int hi = lane >> 5;
-    const int a_frag = (wm * 128 + (lane & 31)) * kRowBytes;
-    const int b_frag = kOperandBytes + (wn * 128 + (lane & 31)) * kRowBytes;
-
-    auto read_a = [&](Frags& f, int stage, int ks, int tm) {
-      const int slot = ((2 * ks + hi) ^ swz) * 16;
-      f.a[tm] = __builtin_bit_cast(
-          V8, *reinterpret_cast<const uint4*>(smem + stage * kStageBytes + a_frag +
-                                              tm * 32 * kRowBytes + slot));
-    };
-    auto read_b = [&](Frags& f, int stage, int ks, int tn) {
-      const int slot = ((2 * ks + hi) ^ swz) * 16;
-      f.b[tn] = __builtin_bit_cast(
-          V8, *reinterpret_cast<const uint4*>(smem + stage * kStageBytes + b_frag +
-                                              tn * 32 * kRowBytes + slot));
+    // load number q (0..15) of the next K tile into `stage`, `ahead` K tiles
+    // past the loaders' current position: even q -> A, odd q -> B
+    auto issue_one = [&](int stage, int ahead, int q) {
+      const unsigned s_off = (unsigned)(stage * kStageBytes) + (unsigned)((q >> 1) * 1024);
+      if (q & 1) load_to_lds(lb.fill + s_off, lb.off[q >> 1], lb.next + ahead * lb.step);
+      else load_to_lds(la.fill + s_off, la.off[q >> 1], la.next + ahead * la.step);
     };
     // fragment r (0..7) of a slice in the order the next slice consumes them:
     // b0..b3 first (every MFMA group needs all four), then a0..a3
-    auto read_frag = [&](Frags& f, int stage, int ks, int r) {
-      if (r < 4) read_b(f, stage, ks, r); else read_a(f, stage, ks, r - 4);
+    auto read_one = [&](Frags& f, int stage, int ks, int r) {
+      const char* st = smem + stage * kStageBytes;
+      if (r < 4) f.b[r] = read_frag<kBKMajor>(st + kOperandBytes, rb, ks, r);
+      else f.a[r - 4] = read_frag<kAKMajor>(st, ra, ks, r - 4);
     };
 
-    // One K step = 64 MFMAs = 16 groups of 4 (slice sl = g/4, A block q = g%4,
-    // B block t = 0..3).  A wave issues in order and an MFMA occupies its pipe
-    // for 32 cycles, so everything else has to fit into those shadows a few
-    // instructions at a time: after every MFMA at most one LDS fragment read
-    // or one load instruction (three scalar + one vector instruction) follows.
-    //   reads : the 8 fragments of the next slice, two per group (slots 0, 2);
-    //           the next tile's slice 0 is read in the two groups after the
-    //           barrier (5 + 3);
-    //   loads : of the next tile's 16, six go out right after the barrier of
-    //           the previous step, ten in groups 0..9 (slot 1) - the last one
-    //           16 MFMAs (~500 cycles) before the barrier that waits for it.
     const int nk = (k_end - k_begin) / kBK;
     auto step = [&](int k, Frags& fa, Frags& fb, auto has_next_tag) {
       constexpr bool kHasNext = decltype(has_next_tag)::value;
@@ -499,53 +434,60 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
         const bool after_barrier = kHasNext && sl == 3 && q >= 2;
         if (kHasNext && sl == 3 && q == 2) {
           // tile k+1 is complete and visible from here on; stage `cur` is free
-#ifndef TLCE_EXP_NOWAIT
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-#ifndef TLCE_EXP_NOBARRIER
           __syncthreads();
-#endif
+          la.next += la.step;
+          lb.next += lb.step;
         }
 #pragma unroll
         for (int t = 0; t < kTN; ++t) {
           acc.c[q][t] = Op::mma(fcur.a[q], fcur.b[t], acc.c[q][t]);
           if (sl < 3) {
-            if (t == 0) read_frag(fnext, cur, sl + 1, 2 * q);
-            if (t == 2) read_frag(fnext, cur, sl + 1, 2 * q + 1);
-#ifndef TLCE_EXP_NOLOAD
-            if (kHasNext && t == 1 && g < 10) issue_one(nxt, k + 1, 6 + g);
-#endif
+            if (t == 0) read_one(fnext, cur, sl + 1, 2 * q);
+            if (t == 2) read_one(fnext, cur, sl + 1, 2 * q + 1);
+            if (kHasNext && t == 1 && g < 10) issue_one(nxt, 0, 6 + g);
           } else if (after_barrier) {
             if (q == 2) {
-              if (t == 0) { read_frag(fnext, nxt, 0, 0); read_frag(fnext, nxt, 0, 1); }
-              else read_frag(fnext, nxt, 0, t + 1);
+              if (t == 0) { read_one(fnext, nxt, 0, 0); read_one(fnext, nxt, 0, 1); }
+              else read_one(fnext, nxt, 0, t + 1);
             } else {
-              if (t < 3) read_frag(fnext, nxt, 0, 5 + t);
+              if (t < 3) read_one(fnext, nxt, 0, 5 + t);
             }
-#ifndef TLCE_EXP_NOLOAD
-            if (t >= 1 && more) issue_one(cur, k + 2, (q - 2) * 3 + (t - 1));
-#endif
+            if (t >= 1 && more) issue_one(cur, 0, (q - 2) * 3 + (t - 1));
           }
           __builtin_amdgcn_sched_barrier(0);
         }
       }
     };
 
+    // tile 0 entirely, then the first six loads of tile 1 (la.next / lb.next
+    // always point at the tile whose loads are being issued)
 #pragma unroll
     for (int q = 0; q < 16; ++q) issue_one(0, 0, q);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
+    la.next += la.step;
+    lb.next += lb.step;
     if (nk > 1) {
 #pragma unroll
-      for (int q = 0; q < 6; ++q) issue_one(1, 1, q);
+      for (int q = 0; q < 6; ++q) issue_one(1, 0, q);
     }
     Frags f0, f1;
 #pragma unroll
-    for (int r = 0; r < 8; ++r) read_frag(f0, 0, 0, r);
+    for (int r = 0; r < 8; ++r) read_one(f0, 0, 0, r);
     // a step consumes slices from f0,f1,f0,f1 and leaves the next tile's slice 0 in f0
     for (int k = 0; k + 1 < nk; ++k) step(k, f0, f1, std::true_type{});
     step(nk - 1, f0, f1, std::false_type{});
     __syncthreads();
+  }
+
+  __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
+                                           int a_rows, const T* __restrict__ B, int64_t ldb,
+                                           int b_row0, int b_rows, int k_begin, int k_end,
+                                           Acc& acc, char* smem) const {
+    const Operand<T> a = {A, lda, a_row0, a_rows};
+    const Operand<T> b = {B, ldb, b_row0, b_rows};
+    mainloop_ex<false, false>(a, b, k_begin, k_end, acc, smem);
   }
 };
 

@@ -23,6 +23,7 @@ struct SimtEngine {
   static constexpr int kCols = 1;
   static constexpr int kRows = 16;
   static constexpr int kShare = 4;
+  static constexpr bool kHasKMajor = false;
 
   struct Acc { float c[kRows]; };
 

@@ -321,21 +321,51 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
     }
   }
 
-#ifdef TLCE_EXP_NOSTORE
-  if (p.m != 123457) return;
-#endif
   T* g_out = static_cast<T*>(p.g);
   T* gt_out = static_cast<T*>(p.gt);
   const int prow = pv * E::kTile;  // first panel column of this tile
+  if constexpr (E::kHasKMajor && sizeof(T) == 2) {
+    // The MFMA engine's LDS is free after the main loop: stage the tile there
+    // as [token][vocab] (512-byte rows, 16-byte chunk c of token t in slot
+    // c ^ (t & 31)) and write G in whole 512-byte rows.
 #pragma unroll
-  for (int j = 0; j < E::kCols; ++j) {
-    const int64_t r = (int64_t)tt * E::kTile + eng.col(j);
+    for (int j = 0; j < E::kCols; ++j) {
+      const int tok = eng.col(j);
 #pragma unroll
-    for (int i = 0; i < E::kRows; i += 4) {
-      store4<T>(g_out + r * p.ldg + prow + eng.row(i), E::get(acc, j, i), E::get(acc, j, i + 1),
-                E::get(acc, j, i + 2), E::get(acc, j, i + 3));
+      for (int i = 0; i < E::kRows; i += 4) {
+        const int vq = eng.row(i) >> 2;
+        T* dst = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
+                                      (vq & 1) * 8);
+        store4<T>(dst, E::get(acc, j, i), E::get(acc, j, i + 1), E::get(acc, j, i + 2),
+                  E::get(acc, j, i + 3));
+      }
     }
-    if (gt_out != nullptr) {
+    __syncthreads();
+#pragma unroll 4
+    for (int it = 0; it < (E::kTile * 32) / E::kThreads; ++it) {
+      const int c = it * E::kThreads + threadIdx.x;
+      const int tok = c >> 5;
+      const int ch = c & 31;
+      const uint4 val =
+          *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16));
+      *reinterpret_cast<uint4*>(g_out + ((int64_t)tt * E::kTile + tok) * p.ldg + prow + ch * 8) =
+          val;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      const int64_t r = (int64_t)tt * E::kTile + eng.col(j);
+#pragma unroll
+      for (int i = 0; i < E::kRows; i += 4) {
+        store4<T>(g_out + r * p.ldg + prow + eng.row(i), E::get(acc, j, i),
+                  E::get(acc, j, i + 1), E::get(acc, j, i + 2), E::get(acc, j, i + 3));
+      }
+    }
+  }
+  if (gt_out != nullptr) {
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      const int64_t r = (int64_t)tt * E::kTile + eng.col(j);
 #pragma unroll
       for (int i = 0; i < E::kRows; ++i)
         gt_out[(int64_t)(prow + eng.row(i)) * p.ldgt + r] = from_float<T>(E::get(acc, j, i));
@@ -347,6 +377,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 // the "A rows" on the output's contiguous axis (the hidden dimension):
 //   grad_hidden: A = weight^T [h, Kv], B = G panel [mp, Kv]   -> C float32 [mp, h]
 //   grad_weight: A = hidden^T [h, Km], B = GT panel [pv, Km]  -> C dtype   [pv, h]
+// An engine with K-major operand support reads the "transposed" operands
+// straight from their stored form (kAKMajor / kBKMajor: the operand is given
+// as X[k][row], `rows` = its valid columns): weight [v, h] for grad_hidden,
+// hidden [m, h] and the G panel [mp, Kv] for grad_weight.
 // (project_grad_hidden / accumulate_grad_weight, fused_linear_ce_cuda.cu:676-791,
 // with float32 accumulation).  A thread holds runs of 4 consecutive A rows per
 // owned B row, so it reads and writes the output 16 (float32) or 8 (dtype)
@@ -369,7 +403,7 @@ struct GemmArgs {
   int mode;
 };
 
-template <class E>
+template <class E, bool kAKMajor, bool kBKMajor>
 __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
@@ -384,13 +418,16 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
   E eng;
   typename E::Acc acc;
   E::zero(acc);
-  eng.mainloop(static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows,
-               static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows, k_begin, k_end, acc,
-               smem);
+  if constexpr (E::kHasKMajor) {
+    const Operand<T> a = {static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows};
+    const Operand<T> b = {static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows};
+    eng.template mainloop_ex<kAKMajor, kBKMajor>(a, b, k_begin, k_end, acc, smem);
+  } else {
+    eng.mainloop(static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows,
+                 static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows, k_begin, k_end,
+                 acc, smem);
+  }
 
-#ifdef TLCE_EXP_NOSTORE
-  if (p.k != 123457) return;
-#endif
   // runs of 4 can be moved as one vector when every row start keeps them aligned
   const bool vec_ok = (p.ldc % 4 == 0) && (p.c_cols % 4 == 0) &&
                       (reinterpret_cast<uintptr_t>(p.c) % 16 == 0);

@@ -82,7 +82,8 @@ constexpr int64_t kDefaultPanelBytes = 1ll << 30;
 constexpr int kTargetWorkgroups = 1024;  // 4 per CU on a 256-CU MI355X
 
 struct Plan {
-  int engine;  // 3/2 = direct-to-LDS MFMA (4/8 waves), 1 = register-staged MFMA, 0 = generic
+  int engine;   // 2 = direct-to-LDS MFMA, 1 = register-staged MFMA, 0 = generic
+  bool kmajor;  // gradient contractions read K-major operands in place
   int tile;
   int bk;
   int64_t mp, vp;
@@ -96,18 +97,21 @@ struct Plan {
 Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_grad,
                int64_t panel_bytes) {
   Plan p;
-  // 3: four-wave direct-to-LDS MFMA (h % 64 == 0), 2: eight-wave direct-to-LDS MFMA
-  // (h % 32 == 0), 1: register-staged MFMA (h % 8 == 0), 0: generic
+  // 2: four-wave direct-to-LDS MFMA (h % 64 == 0), 1: register-staged MFMA
+  // (h % 8 == 0), 0: generic float32-FMA tiles
   if (dtype == TLCE_DTYPE_F32 || (h % 8) != 0) p.engine = 0;
-  else if ((h % 64) == 0) p.engine = 3;
-  else if ((h % 32) == 0) p.engine = 2;
+  else if ((h % 64) == 0) p.engine = 2;
   else p.engine = 1;
   if (const char* forced = getenv("TLCE_FORCE_ENGINE")) {
     const int e = atoi(forced);           // debugging aid: only to a less demanding engine
     if (e >= 0 && e < p.engine) p.engine = e;
   }
+  // The direct engine reads weight, hidden and the logit-gradient panel in
+  // their stored form for the gradient contractions (no transposed copies) as
+  // long as every 64-row K slab of weight exists.
+  p.kmajor = (p.engine == 2) && (v % 64) == 0;
   p.tile = p.engine ? 256 : 64;
-  p.bk = p.engine == 3 ? 64 : (p.engine == 2 ? 32 : (p.engine == 1 ? 64 : 16));
+  p.bk = p.engine ? 64 : 16;
   const int64_t mm = std::max<int64_t>(m, 1);
   p.mp = round_up(mm, p.tile);
   p.vp = round_up(v, p.tile);
@@ -117,7 +121,7 @@ Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_grad,
   p.nsplit = (int)std::min<int64_t>(p.n_vtiles,
                                     std::max<int64_t>(1, ceil_div(kTargetWorkgroups, p.n_ttiles)));
   if (panel_bytes <= 0) panel_bytes = kDefaultPanelBytes;
-  const int64_t col_bytes = p.mp * dtype_bytes(dtype) * (weight_grad ? 2 : 1);
+  const int64_t col_bytes = p.mp * dtype_bytes(dtype) * ((weight_grad && !p.kmajor) ? 2 : 1);
   int64_t tiles_per_panel = std::max<int64_t>(1, panel_bytes / col_bytes / p.tile);
   tiles_per_panel = std::min<int64_t>(tiles_per_panel, p.n_vtiles);
   p.n_panels = (int)ceil_div(p.n_vtiles, tiles_per_panel);
@@ -150,16 +154,23 @@ ForwardLayout forward_layout(const Plan& p) {
 struct BackwardLayout {
   int64_t scale, acc32, wt, ht, g, gt, total;
 };
-BackwardLayout backward_layout(const Plan& p, int64_t h, int dtype, bool weight_grad) {
+// wt / gt exist only on the transposed-copy path; ht is hidden^T there and, on
+// the K-major path, a copy of hidden padded to a multiple of 64 rows (only when
+// m is not one already).
+BackwardLayout backward_layout(const Plan& p, int64_t m, int64_t h, int dtype, bool weight_grad) {
   BackwardLayout l;
   const int64_t es = dtype_bytes(dtype);
   int64_t off = 0;
   l.scale = off; off += align256(p.mp * 4);
   l.acc32 = off; off += align256(p.mp * h * 4);
-  l.wt = off;    off += align256(h * p.vp * es);
-  l.ht = off;    off += weight_grad ? align256(h * p.mp * es) : 0;
+  l.wt = off;    off += p.kmajor ? 0 : align256(h * p.vp * es);
+  l.ht = off;
+  if (weight_grad) {
+    if (!p.kmajor) off += align256(h * p.mp * es);
+    else if (m % 64 != 0) off += align256(round_up(m, 64) * h * es);
+  }
   l.g = off;     off += align256(p.mp * p.vc * es);
-  l.gt = off;    off += weight_grad ? align256(p.vc * p.mp * es) : 0;
+  l.gt = off;    off += (weight_grad && !p.kmajor) ? align256(p.vc * p.mp * es) : 0;
   l.total = off;
   return l;
 }
@@ -229,15 +240,15 @@ int launch_grad_logits(const GradLogitsArgs& a, hipStream_t stream) {
   return launch_grad_logits_variant<E, false, false>(a, stream);
 }
 
-template <class E>
+template <class E, bool kAKMajor, bool kBKMajor>
 int launch_gemm(GemmArgs a, int ksplit, int cls, hipStream_t stream) {
-  static int rc = enable_large_lds(lce_gemm_nt_kernel<E>, E::kSmemBytes);
+  static int rc = enable_large_lds(lce_gemm_nt_kernel<E, kAKMajor, kBKMajor>, E::kSmemBytes);
   if (rc) return rc;
   const int ksteps = a.k / E::kBK;
   a.k_per_split = (int)ceil_div(ksteps, ksplit) * E::kBK;
   dim3 grid(xcd_grid((int64_t)a.ni * a.nj), ksplit, 1);
   ScopedTimer timer(cls, stream);
-  lce_gemm_nt_kernel<E><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  lce_gemm_nt_kernel<E, kAKMajor, kBKMajor><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
@@ -311,13 +322,13 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
                   hipStream_t stream) {
   using T = typename E::T;
   const bool weight_grad = grad_weight != nullptr;
-  const BackwardLayout l = backward_layout(p, h, dtype, weight_grad);
+  const BackwardLayout l = backward_layout(p, m, h, dtype, weight_grad);
   float* scale = reinterpret_cast<float*>(ws + l.scale);
   float* acc32 = reinterpret_cast<float*>(ws + l.acc32);
   T* wt = reinterpret_cast<T*>(ws + l.wt);
   T* ht = reinterpret_cast<T*>(ws + l.ht);
   T* g = reinterpret_cast<T*>(ws + l.g);
-  T* gt = weight_grad ? reinterpret_cast<T*>(ws + l.gt) : nullptr;
+  T* gt = (weight_grad && !p.kmajor) ? reinterpret_cast<T*>(ws + l.gt) : nullptr;
 
   ScaleArgs sa;
   sa.labels = labels; sa.row_idx = row_idx; sa.grad_output = grad_output;
@@ -329,13 +340,22 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
   }
   TLCE_LAUNCH_CHECK();
 
-  // K-contiguous operands of the two gradient contractions
-  if (int rc = launch_transpose<T>(static_cast<const T*>(weight), h, v, h, wt, p.vp, p.vp, stream))
-    return rc;
-  if (weight_grad) {
-    if (int rc = launch_transpose<T>(static_cast<const T*>(hidden), h, m, h, ht, p.mp, p.mp,
-                                     stream))
-      return rc;
+  const T* hidden_t = static_cast<const T*>(hidden);
+  const T* weight_t = static_cast<const T*>(weight);
+  const T* hidden_k = hidden_t;          // K-major operand of grad_weight
+  const int64_t m64 = round_up(m, 64);
+  if (!p.kmajor) {
+    // K-contiguous copies for engines that cannot read K-major operands
+    if (int rc = launch_transpose<T>(weight_t, h, v, h, wt, p.vp, p.vp, stream)) return rc;
+    if (weight_grad) {
+      if (int rc = launch_transpose<T>(hidden_t, h, m, h, ht, p.mp, p.mp, stream)) return rc;
+    }
+  } else if (weight_grad && m64 != m) {
+    // whole 64-row K slabs must exist: pad hidden with zero rows
+    TLCE_HIP(hipMemcpyAsync(ht, hidden_t, (size_t)(m * h * sizeof(T)), hipMemcpyDeviceToDevice,
+                            stream));
+    if (int rc = fill_zero(ht + m * h, (m64 - m) * h * (int64_t)sizeof(T), stream)) return rc;
+    hidden_k = ht;
   }
   if (p.dh_ksplit > 1) {
     if (int rc = fill_zero(acc32, p.mp * h * 4, stream)) return rc;
@@ -360,24 +380,43 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     if (int rc = launch_grad_logits<E>(ga, stream)) return rc;
 
     GemmArgs dh;
-    dh.a = wt + v0; dh.lda = p.vp; dh.a_rows = (int)h;
     dh.b = g; dh.ldb = p.vc; dh.b_rows = (int)p.mp;
-    dh.k = (int)width; dh.k_per_split = 0;
+    dh.k_per_split = 0;
     dh.ni = p.n_htiles; dh.nj = p.n_ttiles;
     dh.c = acc32; dh.ldc = h; dh.c_rows = (int)p.mp; dh.c_cols = (int)h;
     dh.mode = (p.dh_ksplit > 1) ? kAtomicF32 : (panel == 0 ? kStoreF32 : kAddF32);
-    if (int rc = launch_gemm<E>(dh, p.dh_ksplit, kClassGradHidden, stream)) return rc;
-
+    GemmArgs dw;
+    dw.k_per_split = 0;
+    dw.ni = p.n_htiles; dw.nj = (int)(width / p.tile);
+    dw.c = weight_grad ? static_cast<T*>(grad_weight) + v0 * h : nullptr; dw.ldc = h;
+    dw.c_rows = (int)rows_valid; dw.c_cols = (int)h;
+    dw.mode = kStoreT;
+    if constexpr (E::kHasKMajor) {
+      if (p.kmajor) {
+        // grad_hidden: A = weight rows [v0, v0+K) as stored (K-major), B = G
+        dh.a = weight_t + v0 * h; dh.lda = h; dh.a_rows = (int)h;
+        dh.k = (int)round_up(rows_valid, 64);
+        if (int rc = launch_gemm<E, true, false>(dh, p.dh_ksplit, kClassGradHidden, stream))
+          return rc;
+        if (weight_grad) {
+          // grad_weight: A = hidden as stored, B = G as stored, both K-major (K = token)
+          dw.a = hidden_k; dw.lda = h; dw.a_rows = (int)h;
+          dw.b = g; dw.ldb = p.vc; dw.b_rows = (int)width;
+          dw.k = (int)m64;
+          if (int rc = launch_gemm<E, true, true>(dw, 1, kClassGradWeight, stream)) return rc;
+        }
+        continue;
+      }
+    }
+    dh.a = wt + v0; dh.lda = p.vp; dh.a_rows = (int)h;
+    dh.k = (int)width;
+    if (int rc = launch_gemm<E, false, false>(dh, p.dh_ksplit, kClassGradHidden, stream))
+      return rc;
     if (weight_grad) {
-      GemmArgs dw;
       dw.a = ht; dw.lda = p.mp; dw.a_rows = (int)h;
       dw.b = gt; dw.ldb = p.mp; dw.b_rows = (int)width;
-      dw.k = (int)p.mp; dw.k_per_split = 0;
-      dw.ni = p.n_htiles; dw.nj = (int)(width / p.tile);
-      dw.c = static_cast<T*>(grad_weight) + v0 * h; dw.ldc = h;
-      dw.c_rows = (int)rows_valid; dw.c_cols = (int)h;
-      dw.mode = kStoreT;
-      if (int rc = launch_gemm<E>(dw, 1, kClassGradWeight, stream)) return rc;
+      dw.k = (int)p.mp;
+      if (int rc = launch_gemm<E, false, false>(dw, 1, kClassGradWeight, stream)) return rc;
     }
   }
 
@@ -398,23 +437,19 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
 
 using namespace tlce;
 
-#define TLCE_DISPATCH(plan, dtype, CALL)                                                  \
-  do {                                                                                    \
-    if ((plan).engine == 3) {                                                             \
+#define TLCE_DISPATCH(plan, dtype, CALL)                                                   \
+  do {                                                                                     \
+    if ((plan).engine == 2) {                                                              \
       if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaDirect4Engine<__bf16>; return CALL; } \
-      { using E = MfmaDirect4Engine<_Float16>; return CALL; }                             \
-    }                                                                                     \
-    if ((plan).engine == 2) {                                                             \
-      if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaDirectEngine<__bf16>; return CALL; } \
-      { using E = MfmaDirectEngine<_Float16>; return CALL; }                              \
-    }                                                                                     \
-    if ((plan).engine == 1) {                                                             \
-      if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaEngine<__bf16>; return CALL; }      \
-      { using E = MfmaEngine<_Float16>; return CALL; }                                    \
-    }                                                                                     \
-    if ((dtype) == TLCE_DTYPE_F32) { using E = SimtEngine<float>; return CALL; }          \
-    if ((dtype) == TLCE_DTYPE_BF16) { using E = SimtEngine<__bf16>; return CALL; }        \
-    { using E = SimtEngine<_Float16>; return CALL; }                                      \
+      { using E = MfmaDirect4Engine<_Float16>; return CALL; }                              \
+    }                                                                                      \
+    if ((plan).engine == 1) {                                                              \
+      if ((dtype) == TLCE_DTYPE_BF16) { using E = MfmaEngine<__bf16>; return CALL; }       \
+      { using E = MfmaEngine<_Float16>; return CALL; }                                     \
+    }                                                                                      \
+    if ((dtype) == TLCE_DTYPE_F32) { using E = SimtEngine<float>; return CALL; }           \
+    if ((dtype) == TLCE_DTYPE_BF16) { using E = SimtEngine<__bf16>; return CALL; }         \
+    { using E = SimtEngine<_Float16>; return CALL; }                                       \
   } while (0)
 
 extern "C" int tlce_version(void) { return TLCE_VERSION; }
@@ -490,7 +525,7 @@ extern "C" int64_t tlce_backward_workspace_bytes(int64_t m, int64_t h, int64_t v
   (void)has_bias;
   if (m < 0 || h <= 0 || v <= 0) return -1;
   const Plan p = make_plan(m, h, v, dtype, compute_weight_grad != 0, panel_bytes);
-  return backward_layout(p, h, dtype, compute_weight_grad != 0).total;
+  return backward_layout(p, m, h, dtype, compute_weight_grad != 0).total;
 }
 
 extern "C" int tlce_backward(const void* hidden, const void* weight, const float* bias,
@@ -523,7 +558,7 @@ extern "C" int tlce_backward(const void* hidden, const void* weight, const float
   TLCE_REQUIRE(((uintptr_t)grad_hidden & 15) == 0 && ((uintptr_t)grad_weight & 15) == 0,
                "backward: gradients must be 16-byte aligned");
   const Plan p = make_plan(m, h, v, dtype, grad_weight != nullptr, panel_bytes);
-  const int64_t need = backward_layout(p, h, dtype, grad_weight != nullptr).total;
+  const int64_t need = backward_layout(p, m, h, dtype, grad_weight != nullptr).total;
   TLCE_REQUIRE(workspace_bytes >= need, "backward: workspace too small (%lld < %lld)",
                (long long)workspace_bytes, (long long)need);
   TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0, "backward: workspace must be 256-byte aligned");
