@@ -385,7 +385,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 // with float32 accumulation).  A thread holds runs of 4 consecutive A rows per
 // owned B row, so it reads and writes the output 16 (float32) or 8 (dtype)
 // bytes at a time.  blockIdx.y selects a K split.
-enum { kStoreF32 = 0, kAddF32 = 1, kAtomicF32 = 2, kStoreT = 3 };
+enum { kStoreF32 = 0, kAddF32 = 1, kStoreT = 3 };
 
 struct GemmArgs {
   const void* a;
@@ -399,6 +399,7 @@ struct GemmArgs {
   int ni, nj;       // tiles along A rows / B rows
   void* c;          // [c_rows, ldc]: row = B row, column = A row
   int64_t ldc;
+  int64_t c_split_stride;  // elements between the outputs of consecutive K splits
   int c_rows, c_cols;
   int mode;
 };
@@ -411,14 +412,19 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
   if (logical >= p.ni * p.nj) return;
   int ti, tj;
   grouped_tile(logical, p.ni, p.nj, 4, &ti, &tj);
+  // each K split owns its own output slab: no atomics, reproducible sums; a
+  // split whose K range is empty still writes its (zero) tile
   const int k_begin = blockIdx.y * p.k_per_split;
   const int k_end = min(p.k, k_begin + p.k_per_split);
-  if (k_begin >= k_end) return;
+  p.c = static_cast<char*>(p.c) +
+        (int64_t)blockIdx.y * p.c_split_stride * (p.mode == kStoreT ? sizeof(T) : sizeof(float));
 
   E eng;
   typename E::Acc acc;
   E::zero(acc);
-  if constexpr (E::kHasKMajor) {
+  if (k_begin >= k_end) {
+    // nothing to accumulate
+  } else if constexpr (E::kHasKMajor) {
     const Operand<T> a = {static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows};
     const Operand<T> b = {static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows};
     eng.template mainloop_ex<kAKMajor, kBKMajor>(a, b, k_begin, k_end, acc, smem);
@@ -447,16 +453,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
           store4<T>(static_cast<T*>(p.c) + o, v0, v1, v2, v3);
         } else if (p.mode == kStoreF32) {
           *reinterpret_cast<float4*>(static_cast<float*>(p.c) + o) = make_float4(v0, v1, v2, v3);
-        } else if (p.mode == kAddF32) {
+        } else {
           float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.c) + o);
           float4 old = *dst;
           *dst = make_float4(old.x + v0, old.y + v1, old.z + v2, old.w + v3);
-        } else {
-          float* dst = static_cast<float*>(p.c) + o;
-          atomicAdd(dst, v0);
-          atomicAdd(dst + 1, v1);
-          atomicAdd(dst + 2, v2);
-          atomicAdd(dst + 3, v3);
         }
       } else {
         const float vals[4] = {v0, v1, v2, v3};
@@ -467,10 +467,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
             static_cast<T*>(p.c)[o + e] = from_float<T>(vals[e]);
           } else if (p.mode == kStoreF32) {
             static_cast<float*>(p.c)[o + e] = vals[e];
-          } else if (p.mode == kAddF32) {
-            static_cast<float*>(p.c)[o + e] += vals[e];
           } else {
-            atomicAdd(static_cast<float*>(p.c) + o + e, vals[e]);
+            static_cast<float*>(p.c)[o + e] += vals[e];
           }
         }
       }
@@ -508,18 +506,23 @@ __global__ __launch_bounds__(256) void lce_transpose_pad_kernel(const T* __restr
   }
 }
 
-// grad_hidden[row_idx[r], :] = dtype(acc32[r, :])  (cast_float_to_scalar_kernel,
-// fused_linear_ce_cuda.cu:144-154, fused with the un-compaction scatter).
+// grad_hidden[row_idx[r], :] = dtype(sum over K splits of acc32[s][r, :])
+// (cast_float_to_scalar_kernel, fused_linear_ce_cuda.cu:144-154, fused with the
+// K-split reduction and the un-compaction scatter).
 template <typename T>
 __global__ __launch_bounds__(256) void lce_finalize_grad_hidden_kernel(
-    const float* __restrict__ acc32, const int64_t* __restrict__ row_idx, int m, int h,
-    T* __restrict__ out) {
+    const float* __restrict__ acc32, int n_splits, int64_t split_stride,
+    const int64_t* __restrict__ row_idx, int m, int h, T* __restrict__ out) {
   const int r = blockIdx.x;
   if (r >= m) return;
   const int64_t o = (row_idx != nullptr) ? row_idx[r] : (int64_t)r;
   const float* src = acc32 + (int64_t)r * h;
   T* dst = out + o * h;
-  for (int k = threadIdx.x; k < h; k += 256) dst[k] = from_float<T>(src[k]);
+  for (int k = threadIdx.x; k < h; k += 256) {
+    float sum = src[k];
+    for (int s = 1; s < n_splits; ++s) sum += src[(int64_t)s * split_stride + k];
+    dst[k] = from_float<T>(sum);
+  }
 }
 
 __global__ __launch_bounds__(256) void lce_fill_zero_kernel(uint4* __restrict__ dst16,

@@ -118,22 +118,39 @@ Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_grad,
   p.n_ttiles = (int)(p.mp / p.tile);
   p.n_vtiles = (int)(p.vp / p.tile);
   p.n_htiles = (int)ceil_div(h, p.tile);
-  p.nsplit = (int)std::min<int64_t>(p.n_vtiles,
-                                    std::max<int64_t>(1, ceil_div(kTargetWorkgroups, p.n_ttiles)));
+  // forward: token tiles x vocabulary splits workgroups, at most (and close to)
+  // four whole waves of 256 workgroups
+  p.nsplit = (int)std::min<int64_t>(
+      p.n_vtiles, std::max<int64_t>(1, kTargetWorkgroups / p.n_ttiles));
   if (panel_bytes <= 0) panel_bytes = kDefaultPanelBytes;
   const int64_t col_bytes = p.mp * dtype_bytes(dtype) * ((weight_grad && !p.kmajor) ? 2 : 1);
   int64_t tiles_per_panel = std::max<int64_t>(1, panel_bytes / col_bytes / p.tile);
   tiles_per_panel = std::min<int64_t>(tiles_per_panel, p.n_vtiles);
-  p.n_panels = (int)ceil_div(p.n_vtiles, tiles_per_panel);
-  p.vc = ceil_div(p.n_vtiles, p.n_panels) * p.tile;  // balanced panels
+  // A panel of 16*k vocabulary tiles gives the grad_weight launch (tiles x
+  // n_htiles workgroups) and the logit-gradient launch (tiles x n_ttiles) whole
+  // waves of 256 workgroups at the usual head sizes; the last panel takes the
+  // remainder.  Small problems fall back to equal panels.
+  if (tiles_per_panel >= 16 && tiles_per_panel < p.n_vtiles) {
+    tiles_per_panel = tiles_per_panel / 16 * 16;
+    p.vc = tiles_per_panel * p.tile;
+  } else {
+    p.n_panels = (int)ceil_div(p.n_vtiles, tiles_per_panel);
+    p.vc = ceil_div(p.n_vtiles, p.n_panels) * p.tile;  // balanced panels
+  }
   p.n_panels = (int)ceil_div(p.vp, p.vc);
+  // grad_hidden: n_ttiles x n_htiles tiles per panel.  When that is not close
+  // to whole waves of 256 workgroups, split K (each split accumulates into its
+  // own float32 slab, summed by the final cast) by the smallest factor that
+  // fills at least 90 % of the last wave.
   p.dh_ksplit = 1;
   if (p.engine) {
     const int64_t tiles = (int64_t)p.n_ttiles * p.n_htiles;
-    if (tiles < 256) {
-      const int64_t ksteps = p.vc / p.bk;
-      p.dh_ksplit = (int)std::max<int64_t>(
-          1, std::min<int64_t>(ceil_div(512, tiles), ksteps / 8));
+    const int64_t max_split = std::max<int64_t>(1, std::min<int64_t>(16, p.vc / p.bk / 8));
+    for (int64_t ks = 1; ks <= max_split; ++ks) {
+      const double waves = (double)(tiles * ks) / 256.0;
+      const double fill = waves / (double)ceil_div(tiles * ks, 256);
+      p.dh_ksplit = (int)ks;
+      if (fill >= 0.9 && (waves >= 2.0 || ks == max_split)) break;
     }
   }
   return p;
@@ -162,7 +179,7 @@ BackwardLayout backward_layout(const Plan& p, int64_t m, int64_t h, int dtype, b
   const int64_t es = dtype_bytes(dtype);
   int64_t off = 0;
   l.scale = off; off += align256(p.mp * 4);
-  l.acc32 = off; off += align256(p.mp * h * 4);
+  l.acc32 = off; off += align256(p.mp * h * 4 * p.dh_ksplit);   // one slab per K split
   l.wt = off;    off += p.kmajor ? 0 : align256(h * p.vp * es);
   l.ht = off;
   if (weight_grad) {
@@ -357,9 +374,6 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     if (int rc = fill_zero(ht + m * h, (m64 - m) * h * (int64_t)sizeof(T), stream)) return rc;
     hidden_k = ht;
   }
-  if (p.dh_ksplit > 1) {
-    if (int rc = fill_zero(acc32, p.mp * h * 4, stream)) return rc;
-  }
   if (grad_bias != nullptr) {
     if (int rc = fill_zero(grad_bias, v * 4, stream)) return rc;
   }
@@ -384,12 +398,14 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     dh.k_per_split = 0;
     dh.ni = p.n_htiles; dh.nj = p.n_ttiles;
     dh.c = acc32; dh.ldc = h; dh.c_rows = (int)p.mp; dh.c_cols = (int)h;
-    dh.mode = (p.dh_ksplit > 1) ? kAtomicF32 : (panel == 0 ? kStoreF32 : kAddF32);
+    dh.c_split_stride = p.mp * h;
+    dh.mode = (panel == 0) ? kStoreF32 : kAddF32;
     GemmArgs dw;
     dw.k_per_split = 0;
     dw.ni = p.n_htiles; dw.nj = (int)(width / p.tile);
     dw.c = weight_grad ? static_cast<T*>(grad_weight) + v0 * h : nullptr; dw.ldc = h;
     dw.c_rows = (int)rows_valid; dw.c_cols = (int)h;
+    dw.c_split_stride = 0;
     dw.mode = kStoreT;
     if constexpr (E::kHasKMajor) {
       if (p.kmajor) {
@@ -425,8 +441,8 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
   }
   {
     ScopedTimer timer(kClassOther, stream);
-    lce_finalize_grad_hidden_kernel<T><<<(int)m, 256, 0, stream>>>(acc32, row_idx, (int)m, (int)h,
-                                                                 static_cast<T*>(grad_hidden));
+    lce_finalize_grad_hidden_kernel<T><<<(int)m, 256, 0, stream>>>(
+        acc32, p.dh_ksplit, p.mp * h, row_idx, (int)m, (int)h, static_cast<T*>(grad_hidden));
   }
   TLCE_LAUNCH_CHECK();
   return 0;
