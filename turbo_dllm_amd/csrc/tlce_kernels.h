@@ -69,28 +69,37 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
         for (int j = 0; j < E::kCols; ++j) E::set(acc, j, i, E::get(acc, j, i) + b);
       }
     }
-    // logits -> base-2 scaled, masked entries -> -inf
+    // Only the last vocabulary tile (rows past v) and the tile that holds the
+    // excluded column need per-element masking: a workgroup-uniform branch.
+    const bool edge = (vbase + E::kTile > p.v) ||
+                      (p.exclude >= vbase && p.exclude < vbase + E::kTile);
+    if (kSoftcap || edge) {
+      asm volatile("" ::: "memory");   // keep this a real branch, not per-element selects
+      const int excluded = (int)p.exclude;
 #pragma unroll
-    for (int i = 0; i < E::kRows; ++i) {
-      const int v = vbase + eng.row(i);
-      const bool ok = (v < p.v) && (v != p.exclude);
+      for (int i = 0; i < E::kRows; ++i) {
+        const int v = vbase + eng.row(i);
+        const bool ok = (v < p.v) && (v != excluded);
 #pragma unroll
-      for (int j = 0; j < E::kCols; ++j) {
-        float z = E::get(acc, j, i);
-        if (kSoftcap) z = p.softcap * fast_tanh(z * inv_cap);
-        E::set(acc, j, i, ok ? z * TLCE_LOG2E : -INFINITY);
+        for (int j = 0; j < E::kCols; ++j) {
+          float z = E::get(acc, j, i);
+          if (kSoftcap) z = p.softcap * fast_tanh(z * inv_cap);
+          E::set(acc, j, i, ok ? z : -INFINITY);
+        }
       }
     }
+    // online (max, sum-exp) in the base-2 domain: exp(z - m) = exp2(z*log2e - m2)
 #pragma unroll
     for (int j = 0; j < E::kCols; ++j) {
       float tile_max = -INFINITY;
 #pragma unroll
       for (int i = 0; i < E::kRows; ++i) tile_max = fmaxf(tile_max, E::get(acc, j, i));
-      const float new_max = fmaxf(run_max[j], tile_max);
+      const float new_max = fmaxf(run_max[j], tile_max * TLCE_LOG2E);
       if (new_max > -INFINITY) {
         float s = run_sum[j] * fast_exp2(run_max[j] - new_max);
 #pragma unroll
-        for (int i = 0; i < E::kRows; ++i) s += fast_exp2(E::get(acc, j, i) - new_max);
+        for (int i = 0; i < E::kRows; ++i)
+          s += fast_exp2(fmaf(E::get(acc, j, i), TLCE_LOG2E, -new_max));
         run_sum[j] = s;
         run_max[j] = new_max;
       }
@@ -272,19 +281,25 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   eng.mainloop(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
 
   const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
-  int64_t label[E::kCols];
+  // per owned token column: row of its label inside this tile (-1: none here),
+  // lse in base-2 units, and the loss scale (0 for ignored and padding rows,
+  // which zeroes their whole column of g without a per-element test)
+  int label_row[E::kCols];
   float lse2[E::kCols], scale[E::kCols];
-  bool live[E::kCols];
+  bool label_here = false;
 #pragma unroll
   for (int j = 0; j < E::kCols; ++j) {
     const int r = tt * E::kTile + eng.col(j);
     const int rc = min(r, p.m - 1);
-    label[j] = p.labels[rc];
-    live[j] = (r < p.m) && (label[j] != p.ignore);
+    const int64_t y = p.labels[rc];
+    const bool live = (r < p.m) && (y != p.ignore);
+    const int64_t rel = y - vbase;
+    const bool here = live && rel >= 0 && rel < E::kTile;
+    label_row[j] = here ? (int)rel : -1;
+    label_here |= here;
     lse2[j] = p.lse[rc] * TLCE_LOG2E;
-    scale[j] = live[j] ? p.scale[rc] : 0.0f;
+    scale[j] = live ? p.scale[rc] : 0.0f;
   }
-
   if (kBias) {
 #pragma unroll
     for (int i = 0; i < E::kRows; ++i) {
@@ -293,32 +308,52 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
       for (int j = 0; j < E::kCols; ++j) E::set(acc, j, i, E::get(acc, j, i) + b);
     }
   }
+  // workgroup-uniform: rows past v or the excluded column in this tile;
+  // wave-uniform: some lane of this wave owns a label of this tile (rare)
+  const bool edge = (vbase + E::kTile > p.v) ||
+                    (p.exclude >= vbase && p.exclude < vbase + E::kTile);
+  const bool onehot = __ballot(label_here) != 0ull;
+
+  const int excluded = (int)p.exclude;
+  auto transform = [&](auto edge_tag, auto onehot_tag) {
+    constexpr bool kEdge = decltype(edge_tag)::value;
+    constexpr bool kOnehot = decltype(onehot_tag)::value;
+    asm volatile("" ::: "memory");   // one real branch per variant, no merged selects
 #pragma unroll
-  for (int i = 0; i < E::kRows; ++i) {
-    const int v = vbase + eng.row(i);
-    const bool vok = (v < p.v) && (v != p.exclude);
-    float row_sum = 0.0f;
+    for (int i = 0; i < E::kRows; ++i) {
+      const int row = eng.row(i);
+      const bool vok = !kEdge || ((vbase + row < p.v) && (vbase + row != excluded));
+      float row_sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < E::kCols; ++j) {
-      float z = E::get(acc, j, i);
-      float dcap = 1.0f;
-      if (kSoftcap) {
-        const float t = fast_tanh(z * inv_cap);
-        z = p.softcap * t;
-        dcap = 1.0f - t * t;
+      for (int j = 0; j < E::kCols; ++j) {
+        float z = E::get(acc, j, i);
+        float dcap = 1.0f;
+        if (kSoftcap) {
+          const float t = fast_tanh(z * inv_cap);
+          z = p.softcap * t;
+          dcap = 1.0f - t * t;
+        }
+        float g = fast_exp2(fmaf(z, TLCE_LOG2E, -lse2[j]));
+        if (kOnehot && row == label_row[j]) g -= 1.0f;
+        g *= scale[j];
+        if (kSoftcap) g *= dcap;
+        if (kEdge) g = vok ? g : 0.0f;
+        E::set(acc, j, i, g);
+        row_sum += g;
       }
-      float g = fast_exp2(z * TLCE_LOG2E - lse2[j]);
-      if ((int64_t)v == label[j]) g -= 1.0f;
-      g *= scale[j];
-      if (kSoftcap) g *= dcap;
-      g = (vok && live[j]) ? g : 0.0f;
-      E::set(acc, j, i, g);
-      row_sum += g;
+      if (kBias) {
+        const int v = vbase + row;
+        row_sum = eng.reduce_over_cols(row_sum);
+        if (eng.col_leader() && v < p.v && row_sum != 0.0f) atomicAdd(p.grad_bias + v, row_sum);
+      }
     }
-    if (kBias) {
-      row_sum = eng.reduce_over_cols(row_sum);
-      if (eng.col_leader() && v < p.v && row_sum != 0.0f) atomicAdd(p.grad_bias + v, row_sum);
-    }
+  };
+  if (edge) {
+    transform(std::true_type{}, std::true_type{});
+  } else if (onehot) {
+    transform(std::false_type{}, std::true_type{});
+  } else {
+    transform(std::false_type{}, std::false_type{});
   }
 
   T* g_out = static_cast<T*>(p.g);
