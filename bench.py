@@ -65,6 +65,51 @@ def cpu_baseline(wl, sample_rows: int):
     }
 
 
+def measure_compaction_gather(torch, native, device, n, h, hidden):
+    """Ballot/prefix-sum compaction of a block-diffusion label mask plus the row
+    gather of hidden and labels, timed with HIP events on the launch stream.
+    Algorithmic bytes: 8N labels read twice is not counted, only 8N + 8M + 4MH
+    (labels once, indices, rows read + written)."""
+    gen = torch.Generator().manual_seed(7)
+    half = n // 2
+    blocks = max(half // 32, 1)
+    t = torch.rand(blocks, generator=gen)
+    noisy = (torch.rand(blocks, 32, generator=gen) < t[:, None]).reshape(-1)[:half]
+    keep = torch.cat([torch.zeros(n - noisy.numel(), dtype=torch.bool), noisy])
+    labels = torch.where(keep, torch.randint(0, 1000, (n,), generator=gen),
+                         torch.full((n,), -100)).to(device)
+    for _ in range(3):
+        idx, m = native.compact_rows(labels, -100)
+        native.gather_rows(hidden, idx)
+    torch.cuda.synchronize()
+    reps = 20
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        idx, m = native.compact_rows(labels, -100)
+        native.gather_rows(hidden, idx)
+        native.gather_rows(labels, idx)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / reps
+    nbytes = 8 * n + 8 * m + 4 * m * h
+    # the gather alone (no host read-back of the count inside the timed region)
+    start.record()
+    for _ in range(reps):
+        native.gather_rows(hidden, idx)
+    stop.record()
+    torch.cuda.synchronize()
+    gather_ms = start.elapsed_time(stop) / reps
+    return {
+        "rows": n, "loss_rows": m, "ms": ms, "algorithmic_bytes": nbytes,
+        "GB_per_s": nbytes / ms / 1e6,
+        "gather_only_ms": gather_ms,
+        "gather_only_GB_per_s": 4 * m * h / gather_ms / 1e6,
+        "hbm_peak_GB_per_s": PEAK_HBM_GBS,
+        "note": "compaction includes the host read-back of the row count",
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -72,7 +117,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="block_diffusion_shard_all_rows")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--cpu-rows", type=int, default=256)
+    ap.add_argument("--cpu-rows", type=int, default=2048)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain row copy of the weight matrix (known HBM bytes) "
+                         "so rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -136,6 +184,15 @@ def main() -> int:
                             reduction="mean", **kw)
         torch.cuda.synchronize()
 
+    if args.calibrate_copy:
+        # gather_rows_kernel with identity indices = a plain copy: reads and writes v*h*2 bytes
+        ident = torch.arange(v, device=device)
+        native.gather_rows(weight.detach(), ident)
+        torch.cuda.synchronize()
+
+    # compaction + gather pass on the block-diffusion mask of this shape (HBM-bound)
+    compaction = measure_compaction_gather(torch, native, device, n, h, hidden.detach())
+
     # kernels by symbol: both gradient contractions are launches of lce_gemm_nt_kernel
     contraction_tflop = 2.0 * m * h * v / 1e12          # algorithmic FLOPs of one contraction
     kernels = {
@@ -195,6 +252,7 @@ def main() -> int:
             "flops_per_launch": flops_per_launch,
         },
     }
+    result["compaction_gather"] = compaction
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl, args.cpu_rows)
     print(json.dumps(result), flush=True)

@@ -233,8 +233,9 @@ struct MfmaEngine : MfmaTileLayout<T_> {
 //   K-contiguous: 256 rows x 128 B; 16-byte chunk c of row r in slot
 //                 c ^ ((r >> 1) & 7).
 //   K-major:      64 K rows x 512 B; 16-byte chunk c of K row k in slot
-//                 c ^ (2 * ((k & 3) | (((k >> 3) & 1) << 2))); the even XOR
-//                 keeps 32-byte pairs together for the transposing read.
+//                 c ^ (4 * (k & 3)): the four K rows x 64 bytes that half a
+//                 wave reads at once then fall into four different quarters
+//                 of the banks, and 64-byte runs stay contiguous.
 // ds_read_b64_tr_b16 works on groups of 16 lanes: lane i of a group addresses
 // 4 consecutive elements, and lane l receives element l%4 of the chunks of
 // lanes l/4, 4 + l/4, 8 + l/4, 12 + l/4.  With lane i addressing K row i/4,
@@ -327,7 +328,7 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
 #pragma unroll
       for (int j = 0; j < kLoads; ++j) {
         const int kr = wave * 16 + j * 2 + (lane >> 5);
-        const int swz = 2 * ((kr & 3) | (((kr >> 3) & 1) << 2));
+        const int swz = 4 * (kr & 3);
         const int chunk = min((lane & 31) ^ swz, last_chunk);
         ld.off[j] = (unsigned)((int64_t)kr * x.ld * 2 + chunk * 16);
       }
@@ -355,7 +356,7 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
       const int g = lane >> 4;          // 16-lane group
       const int i = lane & 15;
       const int hi = g >> 1;
-      const int swz = 2 * ((i >> 2) | (hi << 2));
+      const int swz = 4 * (i >> 2);      // = 4 * (K row & 3)
       const int kr = 8 * hi + (i >> 2);  // K row within a 16-wide slice, first half
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
