@@ -138,6 +138,42 @@ int tlce_backward(const void* hidden, const void* weight, const float* bias,
                   int64_t panel_bytes,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- vocabulary shards ---------------------------------------------------
+ * Replace vocab_parallel_ce_forward_local / vocab_parallel_ce_backward_local
+ * (fused_linear_ce.cpp:209-265; fused_vocab_parallel_ce_forward_cuda and
+ * vocab_parallel_ce_stats_kernel, fused_linear_ce_cuda.cu:292-365,1174-1268):
+ * the tensor-parallel form of the loss, where a rank owns the weight rows
+ * [vocab_start, vocab_start + v_local) and labels / exclude_index stay global
+ * ids.  The caller combines the per-row statistics of all shards (one MAX and
+ * one SUM reduction) into the global lse and hands it to the backward.
+ *   forward_local: local_max[m] = max over the shard's non-excluded columns
+ *   (-inf if none), local_sum[m] = sum exp(z - local_max), target_logits[m] =
+ *   logit of the label if this shard owns it and the row is not ignored, else
+ *   0 (-inf if the label is the excluded column and local), valid_count[1].
+ *   Every row gets statistics, ignored ones too, as in the reference.
+ *   backward_local: as tlce_backward with lse = global_lse; grad_hidden [m,h]
+ *   is this shard's partial sum (the caller sums over shards), grad_weight
+ *   [v_local,h] and grad_bias [v_local] are complete.
+ * Workspaces: tlce_forward_workspace_bytes / tlce_backward_workspace_bytes
+ * with v = v_local. */
+int tlce_forward_local(const void* hidden, const void* weight, const float* bias,
+                       const int64_t* labels, int64_t m, int64_t h,
+                       int64_t v_local, int dtype, int64_t vocab_start,
+                       int64_t ignore_index, int64_t exclude_index,
+                       float logit_softcap, float* local_max, float* local_sum,
+                       float* target_logits, float* valid_count,
+                       void* workspace, int64_t workspace_bytes, void* stream);
+
+int tlce_backward_local(const void* hidden, const void* weight, const float* bias,
+                        const int64_t* labels, const float* global_lse,
+                        const float* valid_count, const float* grad_output,
+                        int64_t m, int64_t h, int64_t v_local, int dtype,
+                        int reduction_code, int64_t vocab_start,
+                        int64_t ignore_index, int64_t exclude_index,
+                        float logit_softcap, void* grad_hidden, void* grad_weight,
+                        float* grad_bias, int64_t panel_bytes, void* workspace,
+                        int64_t workspace_bytes, void* stream);
+
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be
  * NULL.  `engine` is 2 for the bf16/f16 MFMA kernels with direct-to-LDS loads

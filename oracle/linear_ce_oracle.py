@@ -22,6 +22,10 @@ What each function follows in the reference (paths relative to its tree):
                            CPU path (tiled_linear_cross_entropy.py:105-149).
   compact_rows             nonzero(labels != ignore) of _compact_valid_loss_rows
                            (dllm_parallel/core/models/backbones/nemotron/model.py:4234-4253).
+  vocab_shard_stats        vocab_parallel_ce_stats_kernel (fused_linear_ce_cuda.cu:292-365):
+                           per-row (max, sum exp, target logit) of one vocabulary shard.
+  combine_vocab_shards     the MAX / SUM reductions over shards and the loss of
+                           dllm_parallel/core/parallel/tensor_parallel/cross_entropy.py:238-252.
 
 Pinning (tests/test_oracle_pins.py): every function above is checked against
 library routines it does not call (torch.nn.functional.cross_entropy, torch
@@ -30,8 +34,11 @@ inputs, against closed forms (uniform logits -> log V, gradient rows summing
 to zero, saturated soft cap), against the committed fixtures under
 tests/golden/, and against the seeded cases of the reference's own test file
 (tests/unit/kernels/test_tiled_linear_cross_entropy.py:61-453), which hold no
-stored vectors and compare to the same library routines.  No function here is
-"parity unpinned".
+stored vectors and compare to the same library routines.  The two shard
+functions are pinned by the identity that the statistics of any split of the
+vocabulary combine to the dense lse / loss of the unsplit head, by brute force
+on a tiny case, and by the special values of the excluded column.  No function
+here is "parity unpinned".
 """
 
 from __future__ import annotations
@@ -136,6 +143,10 @@ def dense_linear_ce_grads(
     rows = torch.nonzero(keep).flatten()
     g[rows, y[rows]] -= 1.0
     g = g * scale[:, None]
+    if exclude_index is not None and exclude_index >= 0:
+        # the excluded column gets no gradient even on a row whose label it is
+        # (ce_grad_logits_kernel skips it before the onehot, fused_linear_ce_cuda.cu:270-283)
+        g[:, exclude_index] = 0.0
     if squashed is not None:
         g = g * (1.0 - squashed * squashed)
     if round_grad_logits is not None:
@@ -218,3 +229,58 @@ def relative_max_error(actual: torch.Tensor, expected: torch.Tensor) -> float:
     if denom == 0.0:
         return float(a.abs().max())
     return float((a - e).abs().max()) / denom
+
+
+def vocab_shard_stats(
+    hidden: torch.Tensor,
+    weight_shard: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    vocab_start: int,
+    bias: Optional[torch.Tensor] = None,
+    ignore_index: int = -100,
+    exclude_index: int = -1,
+    logit_softcap: float = 0.0,
+    dtype: torch.dtype = torch.float64,
+):
+    """(local_max, local_sum, target_logits, valid_count) of the weight rows
+    [vocab_start, vocab_start + V_local); labels and exclude_index are global ids."""
+    h = hidden.reshape(-1, hidden.shape[-1]).to(dtype)
+    z = h @ weight_shard.to(dtype).t()
+    if bias is not None:
+        z = z + bias.to(dtype)
+    if logit_softcap and logit_softcap > 0:
+        z = torch.tanh(z / logit_softcap) * logit_softcap
+    v_local = weight_shard.shape[0]
+    y = labels.reshape(-1).to(torch.long)
+    valid = y != ignore_index
+    local_exclude = exclude_index - vocab_start
+    masked = z.clone()
+    if 0 <= local_exclude < v_local:
+        masked[:, local_exclude] = -float("inf")
+    local_max = masked.max(dim=1).values
+    shifted = masked - torch.where(torch.isinf(local_max), torch.zeros_like(local_max),
+                                   local_max)[:, None]
+    local_sum = torch.exp(shifted).sum(dim=1)
+    local_sum = torch.where(torch.isinf(local_max), torch.zeros_like(local_sum), local_sum)
+    y_local = y - vocab_start
+    here = valid & (y_local >= 0) & (y_local < v_local)
+    picked = z.gather(1, y_local.clamp(0, v_local - 1)[:, None])[:, 0]
+    target = torch.where(here, picked, torch.zeros_like(picked))
+    target = torch.where(here & (y == exclude_index),
+                         torch.full_like(target, -float("inf")), target)
+    valid_count = valid.sum().to(dtype).reshape(1)
+    return local_max, local_sum, target, valid_count
+
+
+def combine_vocab_shards(stats, labels: torch.Tensor, *, ignore_index: int = -100):
+    """Global (losses, lse) from the per-shard statistics: MAX over the maxima,
+    SUM of the rescaled sums and of the target logits (every label lives in
+    exactly one shard), loss = lse - target on rows that are not ignored."""
+    global_max = torch.stack([s[0] for s in stats]).max(dim=0).values
+    global_sum = sum(s[1] * torch.exp(s[0] - global_max) for s in stats)
+    target = sum(s[2] for s in stats)
+    lse = global_max + torch.log(global_sum)
+    valid = labels.reshape(-1) != ignore_index
+    losses = torch.where(valid, lse - target, torch.zeros_like(lse))
+    return losses, lse

@@ -387,3 +387,35 @@ def test_scaled_benchmark_configurations(gpu_device, name):
         wl.weight.shape[0])
     check_against_oracle(gpu_device, wl.hidden, wl.weight, wl.labels,
                          logit_softcap=wl.logit_softcap, odtype=torch.float32)
+
+
+def test_label_on_the_excluded_column(gpu_device):
+    """A row labelled with the excluded column: the native path gives loss = lse
+    (target logit 0, fused_linear_ce_cuda.cu:199-219) and no gradient on that
+    column (:270-283); every other row is unaffected."""
+    say("label == exclude, bias, bf16")
+    gen = torch.Generator().manual_seed(77)
+    n, h, v, exclude = 150, 128, 1536, 1023
+    hidden = torch.randn(n, h, generator=gen).bfloat16()
+    weight = (torch.randn(v, h, generator=gen) * 0.2).bfloat16()
+    bias = torch.randn(v, generator=gen).bfloat16()
+    labels = torch.randint(0, v, (n,), generator=gen)
+    labels[labels == exclude] = 0
+    labels[3] = exclude
+    labels[5] = -100
+    loss, dh, dw, db = run_api(gpu_device, hidden, weight, labels, bias=bias,
+                               grad_out=torch.ones(n), reduction="none", exclude_index=exclude,
+                               dtype=torch.bfloat16, weight_layout="vocab_first")
+    ref, lse = oracle.dense_linear_ce(hidden, weight, labels, bias=bias, reduction="none",
+                                      exclude_index=exclude, return_lse=True)
+    others = torch.ones(n, dtype=torch.bool)
+    others[3] = False
+    torch.testing.assert_close(loss[others].double(), ref[others].double(), rtol=LOSS_RTOL,
+                               atol=1e-5)
+    torch.testing.assert_close(loss[3].double(), lse[3].double(), rtol=LOSS_RTOL, atol=1e-5)
+    rdh, rdw, rdb = oracle.dense_linear_ce_grads(hidden, weight, labels, torch.ones(n), bias=bias,
+                                                 reduction="none", exclude_index=exclude)
+    assert oracle.relative_max_error(dh, rdh) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(dw, rdw) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(db, rdb) <= GRAD_REL_MAX
+    assert torch.count_nonzero(dw[exclude]) == 0 and float(db[exclude]) == 0.0

@@ -184,3 +184,80 @@ def test_compaction_oracle_matches_nonzero_and_loop():
             assert got.tolist() == oracle.compact_rows_loop(labels)
     assert oracle.compact_rows(np.full(10, -100)).size == 0
     np.testing.assert_array_equal(oracle.compact_rows(np.arange(10)), np.arange(10))
+
+
+@pytest.mark.parametrize("splits", [(0, 13), (0, 5, 13), (0, 1, 6, 7, 13)])
+@pytest.mark.parametrize("softcap,exclude", [(0.0, -1), (3.0, -1), (0.0, 6), (2.5, 0)])
+def test_vocab_shard_statistics_combine_to_the_dense_loss(splits, softcap, exclude):
+    """Any split of the vocabulary must combine to F.cross_entropy over the whole
+    head (a library routine neither shard function calls).  A shard that holds
+    only the excluded column (the [6,7) shard with exclude 6) has max -inf, sum 0."""
+    torch.manual_seed(11)
+    n, h, v = 9, 7, 13
+    hidden = torch.randn(n, h, dtype=torch.float64)
+    weight = torch.randn(v, h, dtype=torch.float64)
+    bias = torch.randn(v, dtype=torch.float64)
+    labels = torch.randint(0, v, (n,))
+    labels[labels == exclude] = (exclude + 1) % v
+    labels[2] = -100
+    z = hidden @ weight.t() + bias
+    if softcap:
+        z = torch.tanh(z / softcap) * softcap
+    if exclude >= 0:
+        z[:, exclude] = -float("inf")
+    expect = F.cross_entropy(z, labels, ignore_index=-100, reduction="none")
+    stats = [
+        oracle.vocab_shard_stats(hidden, weight[a:b], labels, vocab_start=a, bias=bias[a:b],
+                                 exclude_index=exclude, logit_softcap=softcap)
+        for a, b in zip(splits[:-1], splits[1:])
+    ]
+    losses, lse = oracle.combine_vocab_shards(stats, labels)
+    torch.testing.assert_close(losses, expect, rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(lse, torch.logsumexp(z, dim=1), rtol=1e-12, atol=1e-12)
+    for s in stats:
+        assert float(s[3]) == n - 1          # every shard counts every valid row
+    if exclude == 6 and (6, 7) in list(zip(splits[:-1], splits[1:])):
+        lonely = stats[list(zip(splits[:-1], splits[1:])).index((6, 7))]
+        assert torch.isinf(lonely[0]).all() and (lonely[0] < 0).all()
+        assert torch.count_nonzero(lonely[1]) == 0
+
+
+def test_vocab_shard_statistics_brute_force_and_excluded_target():
+    torch.manual_seed(12)
+    n, h, v0, vl = 4, 3, 5, 6
+    hidden = torch.randn(n, h, dtype=torch.float64)
+    shard = torch.randn(vl, h, dtype=torch.float64)
+    labels = torch.tensor([5, 7, 20, -100])      # first, inside (== exclude), other shard, ignored
+    mx, sm, tg, cnt = oracle.vocab_shard_stats(hidden, shard, labels, vocab_start=v0,
+                                               exclude_index=7)
+    for r in range(n):
+        zs = [sum(float(hidden[r, k]) * float(shard[c, k]) for k in range(h)) for c in range(vl)]
+        kept = [z for c, z in enumerate(zs) if v0 + c != 7]
+        assert math.isclose(float(mx[r]), max(kept), rel_tol=1e-12)
+        assert math.isclose(float(sm[r]), sum(math.exp(z - max(kept)) for z in kept), rel_tol=1e-12)
+    assert math.isclose(float(tg[0]), sum(float(hidden[0, k]) * float(shard[0, k]) for k in range(h)),
+                        rel_tol=1e-12)
+    assert float(tg[1]) == -math.inf             # label is the excluded column and local
+    assert float(tg[2]) == 0.0 and float(tg[3]) == 0.0
+    assert float(cnt) == 3.0
+
+
+def test_label_on_the_excluded_column_gets_no_gradient_there():
+    """Degenerate input the reference defines by construction: the excluded
+    column is skipped before the onehot term (fused_linear_ce_cuda.cu:270-283),
+    so a row labelled with it has gradient softmax(z) on the other columns and
+    0 on the excluded one -- brute force on a 1 x 3 case."""
+    hidden = torch.tensor([[1.0, -2.0]], dtype=torch.float64)
+    weight = torch.tensor([[0.5, 0.25], [-1.0, 0.5], [2.0, 1.0]], dtype=torch.float64)
+    labels = torch.tensor([1])
+    dh, dw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, None, reduction="sum",
+                                             exclude_index=1)
+    z = [0.5 - 0.5, -1.0 - 1.0, 2.0 - 2.0]
+    p0 = math.exp(z[0]) / (math.exp(z[0]) + math.exp(z[2]))
+    g = [p0, 0.0, 1.0 - p0]
+    for c in range(3):
+        for k in range(2):
+            assert math.isclose(float(dw[c, k]), g[c] * float(hidden[0, k]), abs_tol=1e-12)
+    for k in range(2):
+        assert math.isclose(float(dh[0, k]), sum(g[c] * float(weight[c, k]) for c in range(3)),
+                            abs_tol=1e-12)

@@ -59,6 +59,27 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_forward_local": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p,             # hidden weight bias labels
+            c_int64, c_int64, c_int64, c_int, c_int64,          # m h v_local dtype vocab_start
+            c_int64, c_int64, c_float,                          # ignore exclude softcap
+            c_void_p, c_void_p, c_void_p, c_void_p,             # local_max local_sum target count
+            c_void_p, c_int64, c_void_p,                        # workspace bytes stream
+        ],
+    ),
+    "tlce_backward_local": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p,             # hidden weight bias labels
+            c_void_p, c_void_p, c_void_p,                       # global_lse valid_count grad_output
+            c_int64, c_int64, c_int64, c_int,                   # m h v_local dtype
+            c_int, c_int64, c_int64, c_int64, c_float,          # reduction start ignore exclude cap
+            c_void_p, c_void_p, c_void_p,                       # grad_hidden grad_weight grad_bias
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
     "tlce_profile_begin": (c_int, []),
     "tlce_profile_end": (c_int, [c_void_p, c_void_p, c_int]),
     "tlce_query_plan": (

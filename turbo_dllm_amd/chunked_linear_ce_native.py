@@ -344,3 +344,127 @@ def backward_frozen_weight(
         logit_softcap=logit_softcap, weight_dim_first=weight_dim_first,
         compute_weight_grad=False, row_idx=row_idx, n_out=n_out,
     )
+
+
+# ------------------------------------------------------------ vocabulary shards --
+def vocab_parallel_forward_local(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    labels: torch.Tensor,
+    *,
+    vocab_start: int,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Softmax statistics of one vocabulary shard, without logits storage.
+
+    Same call and results as the reference shim
+    (chunked_linear_ce_native.py:185-216): ``weight`` holds the rows
+    ``[vocab_start, vocab_start + V_local)`` of the head, ``labels`` and
+    ``exclude_index`` are global ids.  Returns ``(local_max, local_sum,
+    target_logits, valid_count)``, float32, ``[N]`` each and ``[1]``.
+    """
+    device = _require_device(hidden, weight, bias, labels)
+    if hidden.dim() != 2:
+        raise RuntimeError("vocab-parallel hidden must be [N, D]")
+    if weight.dim() != 2:
+        raise RuntimeError("vocab-parallel weight must be [V_local, D]")
+    if weight.shape[1] != hidden.shape[1]:
+        raise RuntimeError("vocab-parallel head width mismatch")
+    if weight.dtype != hidden.dtype:
+        raise RuntimeError("native linear CE expects hidden and weight of one dtype")
+    hidden = hidden.contiguous()
+    weight = weight.contiguous()
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v_local = weight.shape[0]
+    if labels.numel() != m:
+        raise RuntimeError("vocab-parallel label count mismatch")
+    bias32 = None if bias is None else bias.to(torch.float32).contiguous()
+    lib = _lib.library()
+    code = _dtype_code(hidden)
+    with torch.cuda.device(device):
+        local_max = torch.empty(m, dtype=torch.float32, device=device)
+        local_sum = torch.empty(m, dtype=torch.float32, device=device)
+        target_logits = torch.empty(m, dtype=torch.float32, device=device)
+        valid_count = torch.empty(1, dtype=torch.float32, device=device)
+        ws = _workspace(lib.tlce_forward_workspace_bytes(m, h, v_local, code), device)
+        _lib.check(
+            lib.tlce_forward_local(
+                _ptr(hidden), _ptr(weight), _ptr(bias32), _ptr(labels),
+                m, h, v_local, code, int(vocab_start),
+                int(ignore_index), int(exclude_index), float(logit_softcap),
+                _ptr(local_max), _ptr(local_sum), _ptr(target_logits), valid_count.data_ptr(),
+                ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_forward_local",
+        )
+    return local_max, local_sum, target_logits, valid_count
+
+
+def vocab_parallel_backward_local(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    labels: torch.Tensor,
+    global_lse: torch.Tensor,
+    valid_count: torch.Tensor,
+    grad_output: torch.Tensor,
+    *,
+    reduction: str,
+    vocab_start: int,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """One vocabulary shard's exact gradient contributions
+    (reference shim, chunked_linear_ce_native.py:219-256): ``grad_hidden`` is
+    this shard's partial sum, ``grad_weight`` / ``grad_bias`` cover the shard."""
+    device = _require_device(hidden, weight, bias, labels, global_lse, valid_count, grad_output)
+    hidden = hidden.contiguous()
+    weight = weight.contiguous()
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v_local = weight.shape[0]
+    code = _dtype_code(hidden)
+    reduction_code = _reduction_code(reduction)
+    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
+    expected = m if reduction_code == _lib.REDUCTION_NONE else 1
+    if grad_output.numel() != expected:
+        raise RuntimeError(
+            f"grad_output has {grad_output.numel()} elements, expected {expected}"
+        )
+    global_lse = global_lse.reshape(-1).to(torch.float32).contiguous()
+    bias32 = None if bias is None else bias.to(torch.float32).contiguous()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        grad_hidden = torch.empty((m, h), dtype=hidden.dtype, device=device)
+        grad_weight = torch.empty((v_local, h), dtype=weight.dtype, device=device)
+        grad_bias32 = (
+            torch.empty(v_local, dtype=torch.float32, device=device) if bias is not None else None
+        )
+        ws = _workspace(
+            lib.tlce_backward_workspace_bytes(
+                m, h, v_local, code, 1, int(bias is not None), PANEL_BYTES
+            ),
+            device,
+        )
+        _lib.check(
+            lib.tlce_backward_local(
+                _ptr(hidden), _ptr(weight), _ptr(bias32), _ptr(labels),
+                _ptr(global_lse), valid_count.data_ptr(), _ptr(grad_output),
+                m, h, v_local, code,
+                reduction_code, int(vocab_start), int(ignore_index), int(exclude_index),
+                float(logit_softcap),
+                _ptr(grad_hidden), _ptr(grad_weight), _ptr(grad_bias32),
+                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_backward_local",
+        )
+    if grad_bias32 is None:
+        grad_bias = torch.empty(0, dtype=torch.float32, device=device)
+    else:
+        grad_bias = grad_bias32.to(bias.dtype)
+    return grad_hidden, grad_weight, grad_bias

@@ -152,6 +152,14 @@ struct CombineArgs {
   float* losses;
   float* lse;
   float* valid_count;
+  // vocabulary-shard mode (local_max != null): labels and exclude are global
+  // ids, the weight holds rows [label_offset, label_offset + v); the kernel
+  // writes the shard's softmax statistics instead of lse and loss
+  // (vocab_parallel_ce_stats_kernel, fused_linear_ce_cuda.cu:292-365)
+  int64_t label_offset;
+  float* local_max;
+  float* local_sum;
+  float* target_logits;
 };
 
 template <typename T>
@@ -170,9 +178,11 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
   sum = wave_sum(sum);
   const float lse = (mx + log2f(sum)) * TLCE_LN2;
 
-  const int64_t y = p.labels[r];
-  const bool valid = (y != p.ignore);
-  const bool has_target = valid && y >= 0 && y < p.v && y != p.exclude;
+  const int64_t label = p.labels[r];
+  const bool valid = (label != p.ignore);
+  const int64_t y = label - p.label_offset;   // row of the label in this weight
+  const bool here = valid && y >= 0 && y < p.v;
+  const bool has_target = here && label != p.exclude;
   float target = 0.0f;
   if (has_target) {
     const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
@@ -185,9 +195,16 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
     target = dot;
   }
   if (lane == 0) {
-    p.lse[r] = lse;
-    const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r;
-    p.losses[o] = valid ? (lse - target) : 0.0f;
+    if (p.local_max != nullptr) {
+      // the partials are in base-2 units: max2 = max * log2(e), sum = sum exp(z - max)
+      p.local_max[r] = mx * TLCE_LN2;
+      p.local_sum[r] = (mx > -INFINITY) ? sum : 0.0f;
+      p.target_logits[r] = (here && label == p.exclude) ? -INFINITY : target;
+    } else {
+      p.lse[r] = lse;
+      const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r;
+      p.losses[o] = valid ? (lse - target) : 0.0f;
+    }
     if (valid) atomicAdd(p.valid_count, 1.0f);
   }
 }
@@ -239,6 +256,7 @@ struct GradLogitsArgs {
   int m, h, v;
   int64_t ignore, exclude;
   float softcap;
+  int64_t label_offset;  // global id of weight row 0 (vocabulary shards), else 0
   int v0;             // first vocabulary row of the panel
   int n_ttiles, n_ptiles;
   void* g;            // [mp, ldg]
@@ -293,7 +311,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
     const int rc = min(r, p.m - 1);
     const int64_t y = p.labels[rc];
     const bool live = (r < p.m) && (y != p.ignore);
-    const int64_t rel = y - vbase;
+    const int64_t rel = y - p.label_offset - vbase;
     const bool here = live && rel >= 0 && rel < E::kTile;
     label_row[j] = here ? (int)rel : -1;
     label_here |= here;

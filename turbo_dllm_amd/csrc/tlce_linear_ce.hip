@@ -296,17 +296,25 @@ int fill_zero(void* dst, int64_t bytes, hipStream_t stream) {
 }
 
 // ----------------------------------------------------------------- forward --
+// Outputs of the vocabulary-shard forward (all null for the full-vocabulary one).
+struct ShardStats {
+  int64_t vocab_start = 0;
+  float* local_max = nullptr;
+  float* local_sum = nullptr;
+  float* target_logits = nullptr;
+};
+
 template <class E>
 int forward_impl(const Plan& p, const void* hidden, const void* weight, const float* bias,
                  const int64_t* labels, const int64_t* row_idx, int64_t m, int64_t h, int64_t v,
                  int64_t ignore, int64_t exclude, float softcap, float* losses, float* lse,
-                 float* valid_count, char* ws, hipStream_t stream) {
+                 float* valid_count, const ShardStats& shard, char* ws, hipStream_t stream) {
   using T = typename E::T;
   const ForwardLayout l = forward_layout(p);
   ForwardArgs fa;
   fa.hidden = hidden; fa.weight = weight; fa.bias = bias;
   fa.m = (int)m; fa.h = (int)h; fa.v = (int)v;
-  fa.exclude = exclude; fa.softcap = softcap;
+  fa.exclude = exclude - shard.vocab_start; fa.softcap = softcap;
   fa.n_ttiles = p.n_ttiles; fa.n_vtiles = p.n_vtiles; fa.nsplit = p.nsplit;
   fa.part_max = reinterpret_cast<float*>(ws + l.part_max);
   fa.part_sum = reinterpret_cast<float*>(ws + l.part_sum);
@@ -321,6 +329,9 @@ int forward_impl(const Plan& p, const void* hidden, const void* weight, const fl
   ca.part_max = fa.part_max; ca.part_sum = fa.part_sum;
   ca.part_ld = fa.part_ld; ca.nsplit = p.nsplit;
   ca.losses = losses; ca.lse = lse; ca.valid_count = valid_count;
+  ca.label_offset = shard.vocab_start;
+  ca.local_max = shard.local_max; ca.local_sum = shard.local_sum;
+  ca.target_logits = shard.target_logits;
   {
     ScopedTimer timer(kClassCombine, stream);
     lce_combine_loss_kernel<T><<<(int)ceil_div(m, 4), 256, 0, stream>>>(ca);
@@ -330,13 +341,14 @@ int forward_impl(const Plan& p, const void* hidden, const void* weight, const fl
 }
 
 // ---------------------------------------------------------------- backward --
+// vocab_start: global id of weight row 0 (labels and exclude are global ids)
 template <class E>
 int backward_impl(const Plan& p, const void* hidden, const void* weight, const float* bias,
                   const int64_t* labels, const int64_t* row_idx, const float* lse,
                   const float* valid_count, const float* grad_output, int64_t m, int64_t n_out,
                   int64_t h, int64_t v, int dtype, int reduction, int64_t ignore, int64_t exclude,
-                  float softcap, void* grad_hidden, void* grad_weight, float* grad_bias, char* ws,
-                  hipStream_t stream) {
+                  float softcap, int64_t vocab_start, void* grad_hidden, void* grad_weight,
+                  float* grad_bias, char* ws, hipStream_t stream) {
   using T = typename E::T;
   const bool weight_grad = grad_weight != nullptr;
   const BackwardLayout l = backward_layout(p, m, h, dtype, weight_grad);
@@ -386,7 +398,8 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     ga.hidden = hidden; ga.weight = weight; ga.bias = bias; ga.labels = labels;
     ga.lse = lse; ga.scale = scale;
     ga.m = (int)m; ga.h = (int)h; ga.v = (int)v;
-    ga.ignore = ignore; ga.exclude = exclude; ga.softcap = softcap;
+    ga.ignore = ignore; ga.exclude = exclude - vocab_start; ga.softcap = softcap;
+    ga.label_offset = vocab_start;
     ga.v0 = (int)v0;
     ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
     ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
@@ -505,25 +518,27 @@ extern "C" int64_t tlce_forward_workspace_bytes(int64_t m, int64_t h, int64_t v,
   return forward_layout(make_plan(m, h, v, dtype, false, 0)).total;
 }
 
-extern "C" int tlce_forward(const void* hidden, const void* weight, const float* bias,
-                            const int64_t* labels, const int64_t* row_idx, int64_t m,
-                            int64_t n_out, int64_t h, int64_t v, int dtype, int64_t ignore_index,
-                            int64_t exclude_index, float logit_softcap, float* losses, float* lse,
-                            float* valid_count, void* workspace, int64_t workspace_bytes,
-                            void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
+namespace {
+
+int forward_entry(const void* hidden, const void* weight, const float* bias,
+                  const int64_t* labels, const int64_t* row_idx, int64_t m, int64_t n_out,
+                  int64_t h, int64_t v, int dtype, int64_t ignore_index, int64_t exclude_index,
+                  float logit_softcap, float* losses, float* lse, float* valid_count,
+                  const ShardStats& shard, void* workspace, int64_t workspace_bytes,
+                  hipStream_t stream) {
+  const bool local = shard.local_max != nullptr;
   if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
   TLCE_REQUIRE(valid_count != nullptr, "forward: valid_count is null");
   TLCE_REQUIRE(n_out >= m, "forward: n_out=%lld < m=%lld", (long long)n_out, (long long)m);
   TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
                "forward: n_out != m without row_idx");
   if (int rc = fill_zero(valid_count, 4, stream)) return rc;
-  if (row_idx != nullptr || m == 0) {
+  if (!local && (row_idx != nullptr || m == 0)) {
     TLCE_REQUIRE(losses != nullptr || n_out == 0, "forward: losses is null");
     if (int rc = fill_zero(losses, n_out * 4, stream)) return rc;
   }
   if (m == 0) return 0;
-  TLCE_REQUIRE(labels && losses && lse && workspace, "forward: null pointer");
+  TLCE_REQUIRE(labels && workspace && (local || (losses && lse)), "forward: null pointer");
   const Plan p = make_plan(m, h, v, dtype, false, 0);
   TLCE_REQUIRE(workspace_bytes >= forward_layout(p).total,
                "forward: workspace too small (%lld < %lld)", (long long)workspace_bytes,
@@ -531,8 +546,43 @@ extern "C" int tlce_forward(const void* hidden, const void* weight, const float*
   TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0, "forward: workspace must be 256-byte aligned");
   TLCE_DISPATCH(p, dtype,
                 forward_impl<E>(p, hidden, weight, bias, labels, row_idx, m, h, v, ignore_index,
-                                exclude_index, logit_softcap, losses, lse, valid_count,
+                                exclude_index, logit_softcap, losses, lse, valid_count, shard,
                                 static_cast<char*>(workspace), stream));
+}
+
+}  // namespace
+
+extern "C" int tlce_forward(const void* hidden, const void* weight, const float* bias,
+                            const int64_t* labels, const int64_t* row_idx, int64_t m,
+                            int64_t n_out, int64_t h, int64_t v, int dtype, int64_t ignore_index,
+                            int64_t exclude_index, float logit_softcap, float* losses, float* lse,
+                            float* valid_count, void* workspace, int64_t workspace_bytes,
+                            void* stream) {
+  return forward_entry(hidden, weight, bias, labels, row_idx, m, n_out, h, v, dtype, ignore_index,
+                       exclude_index, logit_softcap, losses, lse, valid_count, ShardStats{},
+                       workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlce_forward_local(const void* hidden, const void* weight, const float* bias,
+                                  const int64_t* labels, int64_t m, int64_t h, int64_t v_local,
+                                  int dtype, int64_t vocab_start, int64_t ignore_index,
+                                  int64_t exclude_index, float logit_softcap, float* local_max,
+                                  float* local_sum, float* target_logits, float* valid_count,
+                                  void* workspace, int64_t workspace_bytes, void* stream) {
+  TLCE_REQUIRE(m == 0 || (local_max && local_sum && target_logits),
+               "forward_local: null output pointer");
+  if (m == 0) {
+    TLCE_REQUIRE(valid_count != nullptr, "forward_local: valid_count is null");
+    return fill_zero(valid_count, 4, static_cast<hipStream_t>(stream));
+  }
+  ShardStats shard;
+  shard.vocab_start = vocab_start;
+  shard.local_max = local_max;
+  shard.local_sum = local_sum;
+  shard.target_logits = target_logits;
+  return forward_entry(hidden, weight, bias, labels, nullptr, m, m, h, v_local, dtype,
+                       ignore_index, exclude_index, logit_softcap, nullptr, nullptr, valid_count,
+                       shard, workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int64_t tlce_backward_workspace_bytes(int64_t m, int64_t h, int64_t v, int dtype,
@@ -544,15 +594,15 @@ extern "C" int64_t tlce_backward_workspace_bytes(int64_t m, int64_t h, int64_t v
   return backward_layout(p, m, h, dtype, compute_weight_grad != 0).total;
 }
 
-extern "C" int tlce_backward(const void* hidden, const void* weight, const float* bias,
-                             const int64_t* labels, const int64_t* row_idx, const float* lse,
-                             const float* valid_count, const float* grad_output, int64_t m,
-                             int64_t n_out, int64_t h, int64_t v, int dtype, int reduction_code,
-                             int64_t ignore_index, int64_t exclude_index, float logit_softcap,
-                             void* grad_hidden, void* grad_weight, float* grad_bias,
-                             int64_t panel_bytes, void* workspace, int64_t workspace_bytes,
-                             void* stream_) {
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
+namespace {
+
+int backward_entry(const void* hidden, const void* weight, const float* bias,
+                   const int64_t* labels, const int64_t* row_idx, const float* lse,
+                   const float* valid_count, const float* grad_output, int64_t m, int64_t n_out,
+                   int64_t h, int64_t v, int dtype, int reduction_code, int64_t vocab_start,
+                   int64_t ignore_index, int64_t exclude_index, float logit_softcap,
+                   void* grad_hidden, void* grad_weight, float* grad_bias, int64_t panel_bytes,
+                   void* workspace, int64_t workspace_bytes, hipStream_t stream) {
   if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
   TLCE_REQUIRE(reduction_code >= TLCE_REDUCTION_NONE && reduction_code <= TLCE_REDUCTION_MEAN,
                "backward: bad reduction code %d", reduction_code);
@@ -581,9 +631,40 @@ extern "C" int tlce_backward(const void* hidden, const void* weight, const float
   TLCE_DISPATCH(p, dtype,
                 backward_impl<E>(p, hidden, weight, bias, labels, row_idx, lse, valid_count,
                                  grad_output, m, n_out, h, v, dtype, reduction_code, ignore_index,
-                                 exclude_index, logit_softcap, grad_hidden, grad_weight,
-                                 (bias != nullptr) ? grad_bias : nullptr,
+                                 exclude_index, logit_softcap, vocab_start, grad_hidden,
+                                 grad_weight, (bias != nullptr) ? grad_bias : nullptr,
                                  static_cast<char*>(workspace), stream));
+}
+
+}  // namespace
+
+extern "C" int tlce_backward(const void* hidden, const void* weight, const float* bias,
+                             const int64_t* labels, const int64_t* row_idx, const float* lse,
+                             const float* valid_count, const float* grad_output, int64_t m,
+                             int64_t n_out, int64_t h, int64_t v, int dtype, int reduction_code,
+                             int64_t ignore_index, int64_t exclude_index, float logit_softcap,
+                             void* grad_hidden, void* grad_weight, float* grad_bias,
+                             int64_t panel_bytes, void* workspace, int64_t workspace_bytes,
+                             void* stream) {
+  return backward_entry(hidden, weight, bias, labels, row_idx, lse, valid_count, grad_output, m,
+                        n_out, h, v, dtype, reduction_code, 0, ignore_index, exclude_index,
+                        logit_softcap, grad_hidden, grad_weight, grad_bias, panel_bytes, workspace,
+                        workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlce_backward_local(const void* hidden, const void* weight, const float* bias,
+                                   const int64_t* labels, const float* global_lse,
+                                   const float* valid_count, const float* grad_output, int64_t m,
+                                   int64_t h, int64_t v_local, int dtype, int reduction_code,
+                                   int64_t vocab_start, int64_t ignore_index,
+                                   int64_t exclude_index, float logit_softcap, void* grad_hidden,
+                                   void* grad_weight, float* grad_bias, int64_t panel_bytes,
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
+  return backward_entry(hidden, weight, bias, labels, nullptr, global_lse, valid_count,
+                        grad_output, m, m, h, v_local, dtype, reduction_code, vocab_start,
+                        ignore_index, exclude_index, logit_softcap, grad_hidden, grad_weight,
+                        grad_bias, panel_bytes, workspace, workspace_bytes,
+                        static_cast<hipStream_t>(stream));
 }
 
 extern "C" int tlce_profile_begin(void) {
