@@ -174,6 +174,22 @@ int tlce_backward_local(const void* hidden, const void* weight, const float* bia
                         float* grad_bias, int64_t panel_bytes, void* workspace,
                         int64_t workspace_bytes, void* stream);
 
+/* ---- streaming soft embedding ---------------------------------------------
+ * Replaces streaming_soft_embedding(_from_shards)
+ * (dllm_parallel/core/kernels/streaming_soft_embedding.py:60-148):
+ *   out[r] = embedding_scale * softmax(cap(hidden[r] . weight^T)) . weight
+ * forward-only, without a logits buffer: the forward tile loop yields lse, the
+ * probability panels (rounded to `dtype`, as the reference rounds them before
+ * its second matmul) are contracted with the weight rows in float32.
+ *   hidden [m,h], weight [v,h], out [m,h], all `dtype`. */
+int64_t tlce_soft_embedding_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                            int dtype, int64_t panel_bytes);
+
+int tlce_soft_embedding(const void* hidden, const void* weight, int64_t m,
+                        int64_t h, int64_t v, int dtype, float logit_softcap,
+                        float embedding_scale, void* out, int64_t panel_bytes,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be
  * NULL.  `engine` is 2 for the bf16/f16 MFMA kernels with direct-to-LDS loads

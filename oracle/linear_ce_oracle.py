@@ -24,6 +24,8 @@ What each function follows in the reference (paths relative to its tree):
                            (dllm_parallel/core/models/backbones/nemotron/model.py:4234-4253).
   vocab_shard_stats        vocab_parallel_ce_stats_kernel (fused_linear_ce_cuda.cu:292-365):
                            per-row (max, sum exp, target logit) of one vocabulary shard.
+  dense_soft_embedding     softmax(cap(h W^T)) W * scale, the value that
+                           dllm_parallel/core/kernels/streaming_soft_embedding.py:60-148 streams.
   combine_vocab_shards     the MAX / SUM reductions over shards and the loss of
                            dllm_parallel/core/parallel/tensor_parallel/cross_entropy.py:238-252.
 
@@ -284,3 +286,15 @@ def combine_vocab_shards(stats, labels: torch.Tensor, *, ignore_index: int = -10
     valid = labels.reshape(-1) != ignore_index
     losses = torch.where(valid, lse - target, torch.zeros_like(lse))
     return losses, lse
+
+
+def dense_soft_embedding(hidden, weight, *, logit_softcap=None, embedding_scale=1.0,
+                         dtype=torch.float64):
+    """embedding_scale * softmax(cap(hidden @ weight.T)) @ weight, shaped like hidden."""
+    z = hidden.reshape(-1, hidden.shape[-1]).to(dtype) @ weight.to(dtype).t()
+    if logit_softcap:
+        z = logit_softcap * torch.tanh(z / logit_softcap)
+    z = z - z.max(dim=-1, keepdim=True).values
+    e = torch.exp(z)
+    p = e / e.sum(dim=-1, keepdim=True)
+    return (embedding_scale * (p @ weight.to(dtype))).reshape(hidden.shape)

@@ -261,3 +261,24 @@ def test_label_on_the_excluded_column_gets_no_gradient_there():
     for k in range(2):
         assert math.isclose(float(dh[0, k]), sum(g[c] * float(weight[c, k]) for c in range(3)),
                             abs_tol=1e-12)
+
+
+def test_soft_embedding_oracle_brute_force_and_limits():
+    torch.manual_seed(21)
+    hidden = torch.randn(3, 4, dtype=torch.float64)
+    weight = torch.randn(5, 4, dtype=torch.float64)
+    got = oracle.dense_soft_embedding(hidden, weight, logit_softcap=1.5, embedding_scale=2.0)
+    for r in range(3):
+        z = [1.5 * math.tanh(sum(float(hidden[r, k]) * float(weight[c, k]) for k in range(4)) / 1.5)
+             for c in range(5)]
+        total = sum(math.exp(x) for x in z)
+        for k in range(4):
+            expect = 2.0 * sum(math.exp(z[c]) / total * float(weight[c, k]) for c in range(5))
+            assert math.isclose(float(got[r, k]), expect, rel_tol=1e-12, abs_tol=1e-12)
+    # library routine, no cap
+    lib = torch.softmax(hidden @ weight.t(), dim=-1) @ weight
+    torch.testing.assert_close(oracle.dense_soft_embedding(hidden, weight), lib, rtol=1e-12,
+                               atol=1e-12)
+    # zero hidden -> uniform softmax -> mean of the weight rows
+    mean = oracle.dense_soft_embedding(torch.zeros(1, 4, dtype=torch.float64), weight)
+    torch.testing.assert_close(mean[0], weight.mean(dim=0), rtol=1e-12, atol=1e-12)

@@ -1,0 +1,88 @@
+"""Streaming soft embedding: argument checks and the host path on the CPU, the
+device path against dense float64 softmax(h W^T) W on the GPU."""
+
+import pytest
+import torch
+
+import linear_ce_oracle as oracle
+
+from turbo_dllm_amd.streaming_soft_embedding import (
+    streaming_soft_embedding,
+    streaming_soft_embedding_from_shards,
+)
+
+
+def dense(hidden, weight, softcap=None, scale=1.0):
+    return oracle.dense_soft_embedding(hidden, weight, logit_softcap=softcap, embedding_scale=scale)
+
+
+def rel_max(a, b):
+    return float((a.double() - b.double()).abs().max() / b.double().abs().max())
+
+
+def test_argument_checks():
+    h = torch.randn(3, 8)
+    w = torch.randn(11, 8)
+    kw = dict(row_chunk_size=2, vocab_chunk_size=4)
+    with pytest.raises(ValueError, match="at least two dimensions"):
+        streaming_soft_embedding(torch.randn(8), w, **kw)
+    with pytest.raises(ValueError, match="chunk sizes must be positive"):
+        streaming_soft_embedding(h, w, row_chunk_size=0, vocab_chunk_size=4)
+    with pytest.raises(ValueError, match="at least one vocabulary weight shard"):
+        streaming_soft_embedding_from_shards(h, (), **kw)
+    with pytest.raises(ValueError, match="two-dimensional"):
+        streaming_soft_embedding(h, torch.randn(8), **kw)
+    with pytest.raises(ValueError, match="does not match hidden"):
+        streaming_soft_embedding(h, torch.randn(11, 7), **kw)
+    with pytest.raises(ValueError, match="logit_softcap must be positive"):
+        streaming_soft_embedding(h, w, logit_softcap=0.0, **kw)
+    with pytest.raises(RuntimeError, match="tensor-parallel"):
+        streaming_soft_embedding(h, w, tensor_parallel_size=2, **kw)
+
+
+@pytest.mark.parametrize("softcap,scale", [(None, 1.0), (2.0, 3.0)])
+def test_host_path_matches_dense(softcap, scale):
+    torch.manual_seed(0)
+    h = torch.randn(2, 5, 8)
+    w = torch.randn(13, 8)
+    got = streaming_soft_embedding(h, w, row_chunk_size=3, vocab_chunk_size=4,
+                                   logit_softcap=softcap, embedding_scale=scale)
+    assert got.shape == h.shape and got.dtype == h.dtype and not got.requires_grad
+    assert rel_max(got, dense(h, w, softcap, scale)) < 1e-5
+    shards = streaming_soft_embedding_from_shards(h, (w[:6], w[6:]), row_chunk_size=4,
+                                                  vocab_chunk_size=5, logit_softcap=softcap,
+                                                  embedding_scale=scale)
+    assert rel_max(shards, got) < 1e-6
+    empty = streaming_soft_embedding(torch.zeros(0, 8), w, row_chunk_size=3, vocab_chunk_size=4)
+    assert empty.shape == (0, 8)
+
+
+GPU_CASES = [
+    ("f32_generic", torch.float32, (37, 33), 301, None, 1.0, 2e-5),
+    ("bf16_staged_h72", torch.bfloat16, (61, 72), 1025, None, 1.0, 2e-2),
+    ("bf16_direct", torch.bfloat16, (3, 100, 256), 2304, None, 1.0, 2e-2),
+    ("bf16_direct_softcap_scale", torch.bfloat16, (129, 128), 1536, 5.0, 16.0, 2e-2),
+    ("f16_direct", torch.float16, (70, 64), 1000, None, 0.5, 2e-2),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", GPU_CASES, ids=[c[0] for c in GPU_CASES])
+def test_device_path_matches_dense(gpu_device, case):
+    name, dtype, shape, v, softcap, scale, tol = case
+    print("[case]", name, flush=True)
+    gen = torch.Generator().manual_seed(len(name))
+    h = torch.randn(*shape, generator=gen).to(dtype)
+    w = (torch.randn(v, shape[-1], generator=gen) * (3.0 / shape[-1] ** 0.5)).to(dtype)
+    got = streaming_soft_embedding(h.to(gpu_device), w.to(gpu_device), row_chunk_size=64,
+                                   vocab_chunk_size=256, logit_softcap=softcap,
+                                   embedding_scale=scale)
+    torch.cuda.synchronize()
+    assert got.shape == h.shape and got.dtype == dtype
+    err = rel_max(got.cpu(), dense(h, w, softcap, scale))
+    print("[case] rel max err", f"{err:.2e}", flush=True)
+    assert err <= tol
+    two = streaming_soft_embedding_from_shards(
+        h.to(gpu_device), (w[: v // 2].to(gpu_device), w[v // 2:].to(gpu_device)),
+        row_chunk_size=64, vocab_chunk_size=256, logit_softcap=softcap, embedding_scale=scale)
+    assert torch.equal(two, got)

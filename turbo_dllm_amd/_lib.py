@@ -80,6 +80,17 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_soft_embedding_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int, c_int64]
+    ),
+    "tlce_soft_embedding": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int,   # hidden weight m h v dtype
+            c_float, c_float, c_void_p,                             # softcap scale out
+            c_int64, c_void_p, c_int64, c_void_p,                   # panel_bytes workspace bytes stream
+        ],
+    ),
     "tlce_profile_begin": (c_int, []),
     "tlce_profile_end": (c_int, [c_void_p, c_void_p, c_int]),
     "tlce_query_plan": (

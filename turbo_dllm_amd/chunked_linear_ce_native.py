@@ -468,3 +468,40 @@ def vocab_parallel_backward_local(
     else:
         grad_bias = grad_bias32.to(bias.dtype)
     return grad_hidden, grad_weight, grad_bias
+
+
+# --------------------------------------------------------------- soft embedding --
+def soft_embedding(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    *,
+    logit_softcap: float,
+    embedding_scale: float,
+) -> torch.Tensor:
+    """``embedding_scale * softmax(cap(hidden @ weight.T)) @ weight`` for
+    flattened ``hidden`` [N, H] and ``weight`` [V, H], without a logits buffer."""
+    device = _require_device(hidden, weight)
+    if hidden.dim() != 2 or weight.dim() != 2 or weight.shape[1] != hidden.shape[1]:
+        raise RuntimeError("soft embedding expects hidden [N, H] and weight [V, H]")
+    if weight.dtype != hidden.dtype:
+        raise RuntimeError("native linear CE expects hidden and weight of one dtype")
+    hidden = hidden.contiguous()
+    weight = weight.contiguous()
+    m, h = hidden.shape
+    v = weight.shape[0]
+    code = _dtype_code(hidden)
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        out = torch.empty((m, h), dtype=hidden.dtype, device=device)
+        if m == 0:
+            return out
+        ws = _workspace(lib.tlce_soft_embedding_workspace_bytes(m, h, v, code, PANEL_BYTES), device)
+        _lib.check(
+            lib.tlce_soft_embedding(
+                _ptr(hidden), _ptr(weight), m, h, v, code,
+                float(logit_softcap), float(embedding_scale), _ptr(out),
+                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_soft_embedding",
+        )
+    return out

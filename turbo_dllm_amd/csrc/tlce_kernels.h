@@ -178,6 +178,10 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
   sum = wave_sum(sum);
   const float lse = (mx + log2f(sum)) * TLCE_LN2;
 
+  if (p.labels == nullptr) {   // statistics only (soft embedding): no targets, no loss
+    if (lane == 0) p.lse[r] = lse;
+    return;
+  }
   const int64_t label = p.labels[r];
   const bool valid = (label != p.ignore);
   const int64_t y = label - p.label_offset;   // row of the label in this weight
@@ -220,6 +224,7 @@ struct ScaleArgs {
   int m, mp;
   int reduction;
   int64_t ignore;
+  float constant;   // labels == null: every real row gets this scale
   float* scale;
 };
 
@@ -227,7 +232,9 @@ __global__ __launch_bounds__(256) void lce_token_scale_kernel(ScaleArgs p) {
   const int r = blockIdx.x * 256 + threadIdx.x;
   if (r >= p.mp) return;
   float s = 0.0f;
-  if (r < p.m && p.labels[r] != p.ignore) {
+  if (p.labels == nullptr) {
+    s = (r < p.m) ? p.constant : 0.0f;
+  } else if (r < p.m && p.labels[r] != p.ignore) {
     if (p.reduction == TLCE_REDUCTION_NONE) {
       s = p.grad_output[(p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r];
     } else if (p.reduction == TLCE_REDUCTION_SUM) {
@@ -257,6 +264,7 @@ struct GradLogitsArgs {
   int64_t ignore, exclude;
   float softcap;
   int64_t label_offset;  // global id of weight row 0 (vocabulary shards), else 0
+  int probabilities;     // 1: g = softmax * scale (labels may be null; no onehot, no cap')
   int v0;             // first vocabulary row of the panel
   int n_ttiles, n_ptiles;
   void* g;            // [mp, ldg]
@@ -309,8 +317,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   for (int j = 0; j < E::kCols; ++j) {
     const int r = tt * E::kTile + eng.col(j);
     const int rc = min(r, p.m - 1);
-    const int64_t y = p.labels[rc];
-    const bool live = (r < p.m) && (y != p.ignore);
+    const int64_t y = p.probabilities ? p.label_offset - 1 : p.labels[rc];   // never in a tile
+    const bool live = (r < p.m) && (p.probabilities || y != p.ignore);
     const int64_t rel = y - p.label_offset - vbase;
     const bool here = live && rel >= 0 && rel < E::kTile;
     label_row[j] = here ? (int)rel : -1;
@@ -354,7 +362,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
         float g = fast_exp2(fmaf(z, TLCE_LOG2E, -lse2[j]));
         if (kOnehot && row == label_row[j]) g -= 1.0f;
         g *= scale[j];
-        if (kSoftcap) g *= dcap;
+        if (kSoftcap && !p.probabilities) g *= dcap;
         if (kEdge) g = vok ? g : 0.0f;
         E::set(acc, j, i, g);
         row_sum += g;

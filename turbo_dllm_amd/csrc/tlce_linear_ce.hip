@@ -348,7 +348,10 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
                   const float* valid_count, const float* grad_output, int64_t m, int64_t n_out,
                   int64_t h, int64_t v, int dtype, int reduction, int64_t ignore, int64_t exclude,
                   float softcap, int64_t vocab_start, void* grad_hidden, void* grad_weight,
-                  float* grad_bias, char* ws, hipStream_t stream) {
+                  float* grad_bias, char* ws, hipStream_t stream,
+                  float probabilities_scale = 0.0f) {
+  // labels == null: the "gradient" panel holds softmax * probabilities_scale, so
+  // grad_hidden becomes the probability-weighted sum of weight rows
   using T = typename E::T;
   const bool weight_grad = grad_weight != nullptr;
   const BackwardLayout l = backward_layout(p, m, h, dtype, weight_grad);
@@ -362,7 +365,7 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
   ScaleArgs sa;
   sa.labels = labels; sa.row_idx = row_idx; sa.grad_output = grad_output;
   sa.valid_count = valid_count; sa.m = (int)m; sa.mp = (int)p.mp; sa.reduction = reduction;
-  sa.ignore = ignore; sa.scale = scale;
+  sa.ignore = ignore; sa.scale = scale; sa.constant = probabilities_scale;
   {
     ScopedTimer timer(kClassOther, stream);
     lce_token_scale_kernel<<<(int)ceil_div(p.mp, 256), 256, 0, stream>>>(sa);
@@ -400,6 +403,7 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     ga.m = (int)m; ga.h = (int)h; ga.v = (int)v;
     ga.ignore = ignore; ga.exclude = exclude - vocab_start; ga.softcap = softcap;
     ga.label_offset = vocab_start;
+    ga.probabilities = (labels == nullptr) ? 1 : 0;
     ga.v0 = (int)v0;
     ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
     ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
@@ -665,6 +669,70 @@ extern "C" int tlce_backward_local(const void* hidden, const void* weight, const
                         ignore_index, exclude_index, logit_softcap, grad_hidden, grad_weight,
                         grad_bias, panel_bytes, workspace, workspace_bytes,
                         static_cast<hipStream_t>(stream));
+}
+
+// ---------------------------------------------------------- soft embedding --
+namespace {
+
+struct SoftEmbeddingLayout {
+  int64_t forward_ws, lse, backward_ws, total;
+};
+
+SoftEmbeddingLayout soft_embedding_layout(const Plan& fp, const Plan& bp, int64_t m, int64_t h,
+                                          int dtype) {
+  SoftEmbeddingLayout l;
+  l.forward_ws = 0;
+  l.lse = round_up(forward_layout(fp).total, 256);
+  l.backward_ws = l.lse + round_up(m * 4, 256);
+  l.total = l.backward_ws + backward_layout(bp, m, h, dtype, false).total;
+  return l;
+}
+
+template <class E>
+int soft_embedding_impl(const Plan& fp, const Plan& bp, const SoftEmbeddingLayout& l,
+                        const void* hidden, const void* weight, int64_t m, int64_t h, int64_t v,
+                        int dtype, float softcap, float scale, void* out, char* ws,
+                        hipStream_t stream) {
+  float* lse = reinterpret_cast<float*>(ws + l.lse);
+  if (int rc = forward_impl<E>(fp, hidden, weight, nullptr, nullptr, nullptr, m, h, v, 0, -1,
+                               softcap, nullptr, lse, nullptr, ShardStats{}, ws + l.forward_ws,
+                               stream))
+    return rc;
+  return backward_impl<E>(bp, hidden, weight, nullptr, nullptr, nullptr, lse, nullptr, nullptr, m,
+                          m, h, v, dtype, TLCE_REDUCTION_SUM, 0, -1, softcap, 0, out, nullptr,
+                          nullptr, ws + l.backward_ws, stream, scale);
+}
+
+}  // namespace
+
+extern "C" int64_t tlce_soft_embedding_workspace_bytes(int64_t m, int64_t h, int64_t v, int dtype,
+                                                       int64_t panel_bytes) {
+  if (m < 0 || h <= 0 || v <= 0) return -1;
+  const Plan fp = make_plan(m, h, v, dtype, false, 0);
+  const Plan bp = make_plan(m, h, v, dtype, false, panel_bytes);
+  return soft_embedding_layout(fp, bp, m, h, dtype).total;
+}
+
+extern "C" int tlce_soft_embedding(const void* hidden, const void* weight, int64_t m, int64_t h,
+                                   int64_t v, int dtype, float logit_softcap,
+                                   float embedding_scale, void* out, int64_t panel_bytes,
+                                   void* workspace, int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  if (m == 0) return 0;
+  TLCE_REQUIRE(out != nullptr && workspace != nullptr, "soft_embedding: null pointer");
+  TLCE_REQUIRE(((uintptr_t)out & 15) == 0, "soft_embedding: out must be 16-byte aligned");
+  const Plan fp = make_plan(m, h, v, dtype, false, 0);
+  const Plan bp = make_plan(m, h, v, dtype, false, panel_bytes);
+  const SoftEmbeddingLayout l = soft_embedding_layout(fp, bp, m, h, dtype);
+  TLCE_REQUIRE(workspace_bytes >= l.total, "soft_embedding: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)l.total);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+               "soft_embedding: workspace must be 256-byte aligned");
+  TLCE_DISPATCH(fp, dtype,
+                soft_embedding_impl<E>(fp, bp, l, hidden, weight, m, h, v, dtype, logit_softcap,
+                                       embedding_scale, out, static_cast<char*>(workspace),
+                                       stream));
 }
 
 extern "C" int tlce_profile_begin(void) {
