@@ -130,8 +130,8 @@ def measured_traffic(workload, kernel):
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="block_diffusion_shard_all_rows")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--cpu-rows", type=int, default=2048)
@@ -176,14 +176,18 @@ def main() -> int:
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(args.steps):
+    # the timed region: exactly `steps` steps between two synchronisations; the
+    # events between steps only yield the per-step spread (median) afterwards
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+    marks[0].record()
+    for i in range(args.steps):
         loss = step()
-    stop.record()
+        marks[i + 1].record()
     torch.cuda.synchronize()
-    ms_per_step = start.elapsed_time(stop) / args.steps
-    loss_value = float(loss)
+    ms_per_step = marks[0].elapsed_time(marks[-1]) / args.steps
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    ms_median = per_step[len(per_step) // 2] if per_step else float("nan")
+    loss_value = float(loss.detach())
 
     # per-kernel-class durations of one forward + backward (HIP events on the launch stream)
     with torch.no_grad():
@@ -254,6 +258,10 @@ def main() -> int:
         "tflops_executed_8MHV": executed_tflops,
         "frac_of_bf16_peak_useful": useful_tflops / PEAK_BF16_TFLOPS,
         "mfma_util_executed": executed_tflops / PEAK_BF16_TFLOPS,
+        "ms_per_step_median": ms_median,
+        "forward_only_ms": round(prof.ms["forward_stats"] + prof.ms["combine_loss"], 3),
+        "backward_only_ms": round(sum(x for k, x in prof.ms.items()
+                                      if k not in ("forward_stats", "combine_loss")), 3),
         "kernel_ms": {k: round(x, 3) for k, x in prof.ms.items()},
         "kernel_launches": prof.launches,
         "roofline": {
