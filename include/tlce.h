@@ -190,6 +190,39 @@ int tlce_soft_embedding(const void* hidden, const void* weight, int64_t m,
                         float embedding_scale, void* out, int64_t panel_bytes,
                         void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- frozen-head forward KL -------------------------------------------------
+ * Replaces dflash_frozen_kl_forward / dflash_frozen_kl_backward
+ * (fused_linear_ce.cpp:267-330; fused_linear_ce_cuda.cu:367-480,1270-1509):
+ *   losses[r] = sum_v p_t (log p_t - log p_d),  p_x = softmax(cap(hidden_x[r] . weight_x^T))
+ * for a draft and a teacher head over one vocabulary; only the draft hidden
+ * states get a gradient,
+ *   grad_hidden = ((p_d - p_t) * grad_output[r] * cap'(z_d)) . draft_weight,
+ * with the logit gradient rounded to `dtype` before the contraction, like the
+ * reference.  No logits buffer: the teacher probabilities cross memory in the
+ * same bounded vocabulary panels as the cross-entropy backward (rounded to
+ * `dtype`; the loss is accumulated as the generalised KL sum t log(t/q) - t + q,
+ * which is insensitive to that rounding to first order).
+ *   draft_hidden [m,h_draft], draft_weight [v,h_draft], teacher_hidden
+ *   [m,h_teacher], teacher_weight [v,h_teacher], all `dtype`; losses,
+ *   draft_lse, teacher_lse, grad_output: float32 [m]; grad_hidden [m,h_draft]. */
+int64_t tlce_kl_workspace_bytes(int64_t m, int64_t h_draft, int64_t h_teacher,
+                                int64_t v, int dtype, int64_t panel_bytes);
+
+int tlce_kl_forward(const void* draft_hidden, const void* draft_weight,
+                    const void* teacher_hidden, const void* teacher_weight,
+                    int64_t m, int64_t h_draft, int64_t h_teacher, int64_t v,
+                    int dtype, float logit_softcap, float* losses,
+                    float* draft_lse, float* teacher_lse, int64_t panel_bytes,
+                    void* workspace, int64_t workspace_bytes, void* stream);
+
+int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
+                     const void* teacher_hidden, const void* teacher_weight,
+                     const float* draft_lse, const float* teacher_lse,
+                     const float* grad_output, int64_t m, int64_t h_draft,
+                     int64_t h_teacher, int64_t v, int dtype, float logit_softcap,
+                     void* grad_hidden, int64_t panel_bytes, void* workspace,
+                     int64_t workspace_bytes, void* stream);
+
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be
  * NULL.  `engine` is 2 for the bf16/f16 MFMA kernels with direct-to-LDS loads

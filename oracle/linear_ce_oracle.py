@@ -26,6 +26,11 @@ What each function follows in the reference (paths relative to its tree):
                            per-row (max, sum exp, target logit) of one vocabulary shard.
   dense_soft_embedding     softmax(cap(h W^T)) W * scale, the value that
                            dllm_parallel/core/kernels/streaming_soft_embedding.py:60-148 streams.
+  dense_frozen_kl(_grad)   per-token KL(teacher || draft) of two heads and its
+                           gradient for the draft hidden states
+                           (dflash_kl_forward_kernel / dflash_kl_grad_logits_kernel,
+                           fused_linear_ce_cuda.cu:367-480; dense form in
+                           dllm_parallel/core/kernels/dflash_kl.py:108-121).
   combine_vocab_shards     the MAX / SUM reductions over shards and the loss of
                            dllm_parallel/core/parallel/tensor_parallel/cross_entropy.py:238-252.
 
@@ -298,3 +303,35 @@ def dense_soft_embedding(hidden, weight, *, logit_softcap=None, embedding_scale=
     e = torch.exp(z)
     p = e / e.sum(dim=-1, keepdim=True)
     return (embedding_scale * (p @ weight.to(dtype))).reshape(hidden.shape)
+
+
+def _kl_parts(draft_hidden, draft_weight, teacher_hidden, teacher_weight, logit_softcap, dtype):
+    zd = draft_hidden.to(dtype) @ draft_weight.to(dtype).t()
+    zt = teacher_hidden.to(dtype) @ teacher_weight.to(dtype).t()
+    dcap = torch.ones_like(zd)
+    if logit_softcap:
+        td = torch.tanh(zd / logit_softcap)
+        dcap = 1.0 - td * td
+        zd = logit_softcap * td
+        zt = logit_softcap * torch.tanh(zt / logit_softcap)
+    log_q = zd - torch.logsumexp(zd, dim=-1, keepdim=True)
+    log_p = zt - torch.logsumexp(zt, dim=-1, keepdim=True)
+    return log_q, log_p, dcap
+
+
+def dense_frozen_kl(draft_hidden, draft_weight, teacher_hidden, teacher_weight, *,
+                    logit_softcap=None, dtype=torch.float64):
+    """losses[r] = sum_v p_t (log p_t - log p_d)."""
+    log_q, log_p, _ = _kl_parts(draft_hidden, draft_weight, teacher_hidden, teacher_weight,
+                                logit_softcap, dtype)
+    return (torch.exp(log_p) * (log_p - log_q)).sum(dim=-1)
+
+
+def dense_frozen_kl_grad(draft_hidden, draft_weight, teacher_hidden, teacher_weight, grad_output,
+                         *, logit_softcap=None, dtype=torch.float64):
+    """d sum_r(grad_output[r] * losses[r]) / d draft_hidden
+    = ((p_d - p_t) * grad_output[r] * cap'(z_d)) @ draft_weight."""
+    log_q, log_p, dcap = _kl_parts(draft_hidden, draft_weight, teacher_hidden, teacher_weight,
+                                   logit_softcap, dtype)
+    g = (torch.exp(log_q) - torch.exp(log_p)) * grad_output.to(dtype)[:, None] * dcap
+    return g @ draft_weight.to(dtype)

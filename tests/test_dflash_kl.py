@@ -1,0 +1,100 @@
+"""Frozen-head forward KL: argument checks and the host path on the CPU (the
+reference's own host cases), the device path against the float64 oracle."""
+
+import pytest
+import torch
+
+import linear_ce_oracle as oracle
+from turbo_dllm_amd.dflash_kl import frozen_linear_kl
+
+
+def test_argument_checks():
+    a, w = torch.randn(4, 8), torch.randn(11, 8)
+    with pytest.raises(ValueError, match=r"\[tokens, hidden\]"):
+        frozen_linear_kl(torch.randn(8), w, a, w)
+    with pytest.raises(ValueError, match="token counts differ"):
+        frozen_linear_kl(a, w, torch.randn(5, 8), w)
+    with pytest.raises(ValueError, match=r"\[vocabulary, hidden\]"):
+        frozen_linear_kl(a, torch.randn(8), a, w)
+    with pytest.raises(ValueError, match="vocabularies differ"):
+        frozen_linear_kl(a, w, a, torch.randn(12, 8))
+    with pytest.raises(ValueError, match="draft head width"):
+        frozen_linear_kl(a, torch.randn(11, 7), a, w)
+    with pytest.raises(ValueError, match="teacher head width"):
+        frozen_linear_kl(a, w, a, torch.randn(11, 7))
+    with pytest.raises(ValueError, match="must be positive"):
+        frozen_linear_kl(a, w, a, w, logit_softcap=0.0)
+
+
+@pytest.mark.parametrize("seed,shapes,softcap", [(17, (7, 5, 6, 11), None),
+                                                 (23, (5, 7, 9, 13), 2.5)])
+def test_host_path_reference_cases(seed, shapes, softcap):
+    """tests/unit/kernels/test_dflash_kl.py:13-76 of the reference."""
+    n, hd, ht, v = shapes
+    torch.manual_seed(seed)
+    dh = torch.randn(n, hd, requires_grad=True)
+    th, dw, tw = torch.randn(n, ht), torch.randn(v, hd), torch.randn(v, ht)
+    scale = torch.randn(n)
+    got = frozen_linear_kl(dh, dw, th, tw, logit_softcap=softcap)
+    grad = torch.autograd.grad((got * scale).sum(), dh)[0]
+    ref = oracle.dense_frozen_kl(dh.detach(), dw, th, tw, logit_softcap=softcap)
+    ref_grad = oracle.dense_frozen_kl_grad(dh.detach(), dw, th, tw, scale, logit_softcap=softcap)
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.double(), ref, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(grad.double(), ref_grad, rtol=1e-4, atol=1e-6)
+
+
+GPU_CASES = [
+    # name, dtype, N, H_draft, H_teacher, V, softcap, weight std, loss tol, grad tol
+    ("ref_bf16_seed31", torch.bfloat16, 7, 32, 48, 257, None, 1.0, 2e-2, 4e-2),
+    ("ref_bf16_softcap_seed37", torch.bfloat16, 7, 32, 48, 257, 3.0, 1.0, 2e-2, 4e-2),
+    ("f32_generic", torch.float32, 37, 33, 20, 301, None, 0.3, 2e-5, 2e-5),
+    ("bf16_direct", torch.bfloat16, 300, 256, 128, 2304, None, 0.08, 2e-2, 2e-2),
+    ("bf16_direct_softcap", torch.bfloat16, 129, 128, 192, 1536, 5.0, 0.2, 2e-2, 2e-2),
+    ("bf16_mixed_engines", torch.bfloat16, 70, 128, 72, 1000, None, 0.15, 2e-2, 2e-2),
+    ("f16_direct_two_panels", torch.float16, 520, 64, 64, 1024, None, 0.2, 2e-2, 2e-2),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", GPU_CASES, ids=[c[0] for c in GPU_CASES])
+def test_device_path_matches_oracle(gpu_device, case, monkeypatch):
+    name, dtype, n, hd, ht, v, softcap, std, loss_tol, grad_tol = case
+    print("[case]", name, flush=True)
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    if "two_panels" in name:
+        monkeypatch.setattr(native, "PANEL_BYTES", 768 * 512 * 2)   # 512 columns per panel
+    gen = torch.Generator().manual_seed({"ref_bf16_seed31": 31, "ref_bf16_softcap_seed37": 37}
+                                        .get(name, len(name)))
+    dh = torch.randn(n, hd, generator=gen).to(dtype)
+    th = torch.randn(n, ht, generator=gen).to(dtype)
+    dw = (torch.randn(v, hd, generator=gen) * std).to(dtype)
+    tw = (torch.randn(v, ht, generator=gen) * std).to(dtype)
+    scale = torch.randn(n, generator=gen)
+    x = dh.to(gpu_device).requires_grad_(True)
+    got = frozen_linear_kl(x, dw.to(gpu_device), th.to(gpu_device), tw.to(gpu_device),
+                           logit_softcap=softcap)
+    (got * scale.to(gpu_device)).sum().backward()
+    torch.cuda.synchronize()
+    ref = oracle.dense_frozen_kl(dh, dw, th, tw, logit_softcap=softcap)
+    ref_grad = oracle.dense_frozen_kl_grad(dh, dw, th, tw, scale, logit_softcap=softcap)
+    assert got.dtype == torch.float32 and got.shape == (n,)
+    assert x.grad.dtype == dtype and x.grad.shape == (n, hd)
+    print("[case] loss max abs err", float((got.cpu().double() - ref).abs().max()),
+          "ref max", float(ref.max()), "grad rel max err",
+          oracle.relative_max_error(x.grad.cpu(), ref_grad), flush=True)
+    torch.testing.assert_close(got.cpu().double(), ref, rtol=loss_tol, atol=loss_tol)
+    assert oracle.relative_max_error(x.grad.cpu(), ref_grad) <= grad_tol
+
+
+@pytest.mark.gpu
+def test_same_head_gives_zero(gpu_device):
+    gen = torch.Generator().manual_seed(9)
+    h = torch.randn(200, 128, generator=gen).bfloat16().to(gpu_device)
+    w = (torch.randn(1536, 128, generator=gen) * 0.2).bfloat16().to(gpu_device)
+    x = h.clone().requires_grad_(True)
+    got = frozen_linear_kl(x, w, h, w)
+    got.sum().backward()
+    torch.cuda.synchronize()
+    assert float(got.abs().max()) < 2e-3
+    assert float(x.grad.float().abs().max()) < 2e-2 * float(w.float().abs().max())

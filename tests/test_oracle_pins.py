@@ -282,3 +282,31 @@ def test_soft_embedding_oracle_brute_force_and_limits():
     # zero hidden -> uniform softmax -> mean of the weight rows
     mean = oracle.dense_soft_embedding(torch.zeros(1, 4, dtype=torch.float64), weight)
     torch.testing.assert_close(mean[0], weight.mean(dim=0), rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("softcap", [None, 2.5])
+def test_frozen_kl_oracle_matches_library_kl_div_and_autograd(softcap):
+    """The reference's own host cases (tests/unit/kernels/test_dflash_kl.py:13-76,
+    seeds 17 and 23) against F.kl_div / autograd, which the oracle does not call."""
+    torch.manual_seed(17 if softcap is None else 23)
+    dh = torch.randn(7, 5, dtype=torch.float64, requires_grad=True)
+    th = torch.randn(7, 6, dtype=torch.float64)
+    dw = torch.randn(11, 5, dtype=torch.float64)
+    tw = torch.randn(11, 6, dtype=torch.float64)
+    scale = torch.randn(7, dtype=torch.float64)
+    zd, zt = F.linear(dh, dw), F.linear(th, tw)
+    if softcap:
+        zd, zt = softcap * torch.tanh(zd / softcap), softcap * torch.tanh(zt / softcap)
+    expect = F.kl_div(F.log_softmax(zd, dim=-1), F.softmax(zt, dim=-1), reduction="none").sum(-1)
+    grad = torch.autograd.grad((expect * scale).sum(), dh)[0]
+    got = oracle.dense_frozen_kl(dh.detach(), dw, th, tw, logit_softcap=softcap)
+    torch.testing.assert_close(got, expect.detach(), rtol=1e-12, atol=1e-12)
+    got_grad = oracle.dense_frozen_kl_grad(dh.detach(), dw, th, tw, scale, logit_softcap=softcap)
+    torch.testing.assert_close(got_grad, grad, rtol=1e-10, atol=1e-12)
+    # same head on both sides: zero divergence, zero gradient
+    same = oracle.dense_frozen_kl(dh.detach(), dw, dh.detach(), dw, logit_softcap=softcap)
+    assert float(same.abs().max()) < 1e-12
+    zero = oracle.dense_frozen_kl_grad(dh.detach(), dw, dh.detach(), dw, scale,
+                                       logit_softcap=softcap)
+    assert float(zero.abs().max()) < 1e-12
+    assert bool((got >= 0).all())

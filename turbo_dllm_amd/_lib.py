@@ -91,6 +91,28 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,                   # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_kl_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int64, c_int, c_int64]
+    ),
+    "tlce_kl_forward": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p,             # draft h/w, teacher h/w
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m h_draft h_teacher v dtype
+            c_float, c_void_p, c_void_p, c_void_p,              # softcap losses draft_lse teacher_lse
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
+    "tlce_kl_backward": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p,             # draft h/w, teacher h/w
+            c_void_p, c_void_p, c_void_p,                       # draft_lse teacher_lse grad_output
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m h_draft h_teacher v dtype
+            c_float, c_void_p,                                  # softcap grad_hidden
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
     "tlce_profile_begin": (c_int, []),
     "tlce_profile_end": (c_int, [c_void_p, c_void_p, c_int]),
     "tlce_query_plan": (

@@ -505,3 +505,95 @@ def soft_embedding(
             "tlce_soft_embedding",
         )
     return out
+
+
+# -------------------------------------------------------------- frozen-head KL --
+def _kl_operands(draft_hidden, draft_weight, teacher_hidden, teacher_weight):
+    device = _require_device(draft_hidden, draft_weight, teacher_hidden, teacher_weight)
+    tensors = [t.contiguous() for t in (draft_hidden, draft_weight, teacher_hidden,
+                                        teacher_weight)]
+    dh, dw, th, tw = tensors
+    if dh.dim() != 2 or th.dim() != 2 or dw.dim() != 2 or tw.dim() != 2:
+        raise RuntimeError("DFlash KL expects [tokens, hidden] states and [vocabulary, hidden] heads")
+    if dh.shape[0] != th.shape[0] or dw.shape[0] != tw.shape[0]:
+        raise RuntimeError("DFlash KL draft and teacher shapes differ")
+    if dw.shape[1] != dh.shape[1] or tw.shape[1] != th.shape[1]:
+        raise RuntimeError("DFlash KL head width is incompatible")
+    if any(t.dtype != dh.dtype for t in tensors):
+        raise RuntimeError("DFlash KL tensors must use one dtype")
+    return device, dh, dw, th, tw
+
+
+def dflash_kl_forward(
+    draft_hidden: torch.Tensor,
+    draft_weight: torch.Tensor,
+    teacher_hidden: torch.Tensor,
+    teacher_weight: torch.Tensor,
+    logit_softcap: float,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(losses, draft_lse, teacher_lse)``, float32 [N]: per-token forward KL
+    of the teacher head against the draft head without a logits buffer
+    (reference shim, chunked_linear_ce_native.py:259-283)."""
+    device, dh, dw, th, tw = _kl_operands(draft_hidden, draft_weight, teacher_hidden,
+                                          teacher_weight)
+    m, hd = dh.shape
+    ht, v = th.shape[1], dw.shape[0]
+    code = _dtype_code(dh)
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        losses = torch.empty(m, dtype=torch.float32, device=device)
+        draft_lse = torch.empty(m, dtype=torch.float32, device=device)
+        teacher_lse = torch.empty(m, dtype=torch.float32, device=device)
+        if m == 0:
+            return losses, draft_lse, teacher_lse
+        ws = _workspace(lib.tlce_kl_workspace_bytes(m, hd, ht, v, code, PANEL_BYTES), device)
+        _lib.check(
+            lib.tlce_kl_forward(
+                _ptr(dh), _ptr(dw), _ptr(th), _ptr(tw), m, hd, ht, v, code,
+                float(logit_softcap), _ptr(losses), _ptr(draft_lse), _ptr(teacher_lse),
+                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_kl_forward",
+        )
+    return losses, draft_lse, teacher_lse
+
+
+def dflash_kl_backward(
+    draft_hidden: torch.Tensor,
+    draft_weight: torch.Tensor,
+    teacher_hidden: torch.Tensor,
+    teacher_weight: torch.Tensor,
+    draft_lse: torch.Tensor,
+    teacher_lse: torch.Tensor,
+    grad_output: torch.Tensor,
+    logit_softcap: float,
+) -> torch.Tensor:
+    """Gradient of the per-token KL with respect to the draft hidden states
+    (reference shim, chunked_linear_ce_native.py:286-316)."""
+    device, dh, dw, th, tw = _kl_operands(draft_hidden, draft_weight, teacher_hidden,
+                                          teacher_weight)
+    _require_device(draft_lse, teacher_lse, grad_output)
+    m, hd = dh.shape
+    ht, v = th.shape[1], dw.shape[0]
+    code = _dtype_code(dh)
+    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
+    if grad_output.numel() != m:
+        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected {m}")
+    draft_lse = draft_lse.reshape(-1).to(torch.float32).contiguous()
+    teacher_lse = teacher_lse.reshape(-1).to(torch.float32).contiguous()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        grad_hidden = torch.empty((m, hd), dtype=dh.dtype, device=device)
+        if m == 0:
+            return grad_hidden
+        ws = _workspace(lib.tlce_kl_workspace_bytes(m, hd, ht, v, code, PANEL_BYTES), device)
+        _lib.check(
+            lib.tlce_kl_backward(
+                _ptr(dh), _ptr(dw), _ptr(th), _ptr(tw),
+                _ptr(draft_lse), _ptr(teacher_lse), _ptr(grad_output),
+                m, hd, ht, v, code, float(logit_softcap), _ptr(grad_hidden),
+                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_kl_backward",
+        )
+    return grad_hidden

@@ -99,6 +99,12 @@ struct MfmaTileLayout {
     return v;
   }
   __device__ __forceinline__ bool col_leader() const { return (lane & 31) == 0; }
+  // Sum over the lanes of this wave that hold the same tile column (lanes l and
+  // l ^ 32 hold different rows of it); other waves keep their own sums.
+  __device__ __forceinline__ float reduce_over_rows_in_wave(float v) const {
+    return v + __shfl_xor(v, 32, 64);
+  }
+  __device__ __forceinline__ bool row_leader() const { return lane < 32; }
 };
 
 // Register-staged engine: global -> VGPR -> LDS, two 64-wide K stages.  Takes

@@ -43,6 +43,9 @@ struct SimtEngine {
   // A wave is 64 lanes = the 64 tile columns of one 16-row band.
   __device__ __forceinline__ float reduce_over_cols(float v) const { return wave_sum(v); }
   __device__ __forceinline__ bool col_leader() const { return (tid & 63) == 0; }
+  // every lane of a wave owns a different tile column
+  __device__ __forceinline__ float reduce_over_rows_in_wave(float v) const { return v; }
+  __device__ __forceinline__ bool row_leader() const { return true; }
 
   __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
                                            int a_rows, const T* __restrict__ B, int64_t ldb,

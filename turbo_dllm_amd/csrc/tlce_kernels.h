@@ -233,7 +233,8 @@ __global__ __launch_bounds__(256) void lce_token_scale_kernel(ScaleArgs p) {
   if (r >= p.mp) return;
   float s = 0.0f;
   if (p.labels == nullptr) {
-    s = (r < p.m) ? p.constant : 0.0f;
+    // no labels: every real row gets grad_output[r] (per-row objectives) or the constant
+    s = (r < p.m) ? (p.grad_output != nullptr ? p.grad_output[r] : p.constant) : 0.0f;
   } else if (r < p.m && p.labels[r] != p.ignore) {
     if (p.reduction == TLCE_REDUCTION_NONE) {
       s = p.grad_output[(p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r];
@@ -430,6 +431,160 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 #pragma unroll
       for (int i = 0; i < E::kRows; ++i)
         gt_out[(int64_t)(prow + eng.row(i)) * p.ldgt + r] = from_float<T>(E::get(acc, j, i));
+    }
+  }
+}
+
+// Forward KL(teacher || draft) of two frozen heads, one vocabulary panel at a
+// time (dflash_kl_forward_kernel / dflash_kl_grad_logits_kernel,
+// fused_linear_ce_cuda.cu:367-480).  The panel holds the teacher probabilities
+// t = softmax(cap(z_teacher)) rounded to the input dtype (written by
+// lce_grad_logits_panel_kernel in its probabilities mode).  This kernel
+// recomputes the draft logits tile and, with lp = cap(z_draft) - lse_draft:
+//   mode kKlLoss: losses[token] += sum_v ( t * (log t - lp) - t )
+//                 (the generalised KL; the caller adds 1 per row = sum_v q.
+//                 It equals sum_v p_t (log p_t - log p_d) to first order in the
+//                 rounding of t, where the plain sum would be off by sum_v dt)
+//   mode kKlGrad: panel[token, v] = (exp(lp) - t) * scale[token] * cap'(z_draft)
+//                 in place, rounded to the input dtype: the logit gradient that
+//                 feeds the grad-hidden contraction.
+enum { kKlLoss = 0, kKlGrad = 1 };
+
+struct KlPanelArgs {
+  const void* hidden;   // draft hidden [m, h]
+  const void* weight;   // draft head [v, h]
+  const float* lse;     // draft lse [m]
+  const float* scale;   // kKlGrad: grad_output per row, 0 on padding rows [mp]
+  int m, h, v;
+  float softcap;
+  int v0;               // first vocabulary row of the panel
+  int n_ttiles, n_ptiles;
+  void* panel;          // [mp, ld] teacher probabilities in, logit gradients out
+  int64_t ld;
+  float* losses;        // kKlLoss: [m], accumulated with atomics
+  int mode;
+};
+
+template <class E, bool kSoftcap>
+__global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p) {
+  extern __shared__ __align__(16) char smem[];
+  using T = typename E::T;
+  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
+  if (logical >= p.n_ttiles * p.n_ptiles) return;
+  int tt, pv;
+  grouped_tile(logical, p.n_ttiles, p.n_ptiles, 4, &tt, &pv);
+
+  E eng;
+  typename E::Acc acc;
+  E::zero(acc);
+  const int vbase = p.v0 + pv * E::kTile;
+  eng.mainloop(static_cast<const T*>(p.weight), p.h, vbase, p.v, static_cast<const T*>(p.hidden),
+               p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+
+  const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
+  const bool grad = p.mode == kKlGrad;
+  float lse2[E::kCols], scale[E::kCols], partial[E::kCols];
+  bool live[E::kCols];
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    const int r = tt * E::kTile + eng.col(j);
+    const int rc = min(r, p.m - 1);
+    live[j] = r < p.m;
+    lse2[j] = p.lse[rc] * TLCE_LOG2E;
+    scale[j] = (grad && live[j]) ? p.scale[rc] : 0.0f;
+    partial[j] = 0.0f;
+  }
+  T* panel = static_cast<T*>(p.panel);
+  const int prow = pv * E::kTile;   // first panel column of this tile
+  constexpr bool kCanStage = E::kHasKMajor && sizeof(T) == 2;
+
+  // one group of 4 consecutive vocabulary rows of owned column j: t[] in,
+  // gradient out (kKlGrad) or the loss partial updated (kKlLoss)
+  auto process = [&](int j, int i4, const float (&t)[4], float (&g)[4]) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int row = eng.row(i4 + u);
+      const bool vok = vbase + row < p.v;
+      float z = E::get(acc, j, i4 + u);
+      float dcap = 1.0f;
+      if (kSoftcap) {
+        const float th = fast_tanh(z * inv_cap);
+        z = p.softcap * th;
+        dcap = 1.0f - th * th;
+      }
+      const float lp2 = fmaf(z, TLCE_LOG2E, -lse2[j]);   // log2 of the draft probability
+      if (grad) {
+        const float v = (fast_exp2(lp2) - t[u]) * scale[j] * dcap;
+        g[u] = vok ? v : 0.0f;
+      } else {
+        const float tv = t[u];
+        const float term = tv * ((fast_log2(tv) - lp2) * TLCE_LN2) - tv;
+        if (vok && tv > 0.0f) partial[j] += term;
+      }
+    }
+  };
+
+  if constexpr (kCanStage) {
+    // the tile of the panel goes through LDS in whole 512-byte token rows
+    // (16-byte chunk c of token t in slot c ^ (t & 31)), both ways
+#pragma unroll 4
+    for (int it = 0; it < (E::kTile * 32) / E::kThreads; ++it) {
+      const int c = it * E::kThreads + threadIdx.x;
+      const int tok = c >> 5;
+      const int ch = c & 31;
+      *reinterpret_cast<uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)) =
+          *reinterpret_cast<const uint4*>(panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow +
+                                          ch * 8);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      const int tok = eng.col(j);
+#pragma unroll
+      for (int i4 = 0; i4 < E::kRows; i4 += 4) {
+        const int vq = eng.row(i4) >> 2;
+        T* cell = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
+                                       (vq & 1) * 8);
+        typedef T v4_t __attribute__((ext_vector_type(4)));
+        const v4_t tv = *reinterpret_cast<const v4_t*>(cell);
+        const float t[4] = {to_float<T>(tv[0]), to_float<T>(tv[1]), to_float<T>(tv[2]),
+                            to_float<T>(tv[3])};
+        float g[4];
+        process(j, i4, t, g);
+        if (grad) store4<T>(cell, g[0], g[1], g[2], g[3]);
+      }
+    }
+    if (grad) {
+      __syncthreads();
+#pragma unroll 4
+      for (int it = 0; it < (E::kTile * 32) / E::kThreads; ++it) {
+        const int c = it * E::kThreads + threadIdx.x;
+        const int tok = c >> 5;
+        const int ch = c & 31;
+        *reinterpret_cast<uint4*>(panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 8) =
+            *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      T* cell0 = panel + ((int64_t)tt * E::kTile + eng.col(j)) * p.ld + prow;
+#pragma unroll
+      for (int i4 = 0; i4 < E::kRows; i4 += 4) {
+        T* cell = cell0 + eng.row(i4);
+        const float t[4] = {to_float<T>(cell[0]), to_float<T>(cell[1]), to_float<T>(cell[2]),
+                            to_float<T>(cell[3])};
+        float g[4];
+        process(j, i4, t, g);
+        if (grad) store4<T>(cell, g[0], g[1], g[2], g[3]);
+      }
+    }
+  }
+  if (!grad) {
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      const float total = eng.reduce_over_rows_in_wave(partial[j]);
+      if (eng.row_leader() && live[j]) atomicAdd(p.losses + tt * E::kTile + eng.col(j), total);
     }
   }
 }

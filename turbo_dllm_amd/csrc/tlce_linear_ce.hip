@@ -94,14 +94,17 @@ struct Plan {
   int dh_ksplit;
 };
 
+int engine_class(int64_t h, int dtype) {
+  if (dtype == TLCE_DTYPE_F32 || (h % 8) != 0) return 0;
+  return (h % 64) == 0 ? 2 : 1;
+}
+
 Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_grad,
-               int64_t panel_bytes) {
+               int64_t panel_bytes, int max_engine = 2) {
   Plan p;
   // 2: four-wave direct-to-LDS MFMA (h % 64 == 0), 1: register-staged MFMA
   // (h % 8 == 0), 0: generic float32-FMA tiles
-  if (dtype == TLCE_DTYPE_F32 || (h % 8) != 0) p.engine = 0;
-  else if ((h % 64) == 0) p.engine = 2;
-  else p.engine = 1;
+  p.engine = std::min(engine_class(h, dtype), max_engine);
   if (const char* forced = getenv("TLCE_FORCE_ENGINE")) {
     const int e = atoi(forced);           // debugging aid: only to a less demanding engine
     if (e >= 0 && e < p.engine) p.engine = e;
@@ -341,36 +344,23 @@ int forward_impl(const Plan& p, const void* hidden, const void* weight, const fl
 }
 
 // ---------------------------------------------------------------- backward --
-// vocab_start: global id of weight row 0 (labels and exclude are global ids)
-template <class E>
-int backward_impl(const Plan& p, const void* hidden, const void* weight, const float* bias,
-                  const int64_t* labels, const int64_t* row_idx, const float* lse,
-                  const float* valid_count, const float* grad_output, int64_t m, int64_t n_out,
-                  int64_t h, int64_t v, int dtype, int reduction, int64_t ignore, int64_t exclude,
-                  float softcap, int64_t vocab_start, void* grad_hidden, void* grad_weight,
-                  float* grad_bias, char* ws, hipStream_t stream,
-                  float probabilities_scale = 0.0f) {
-  // labels == null: the "gradient" panel holds softmax * probabilities_scale, so
-  // grad_hidden becomes the probability-weighted sum of weight rows
+// The panel loop shared by every objective whose gradient is G . weight (and
+// G^T . hidden): `produce(v0, width, g, gt)` fills the panel of rounded logit
+// gradients for the vocabulary rows [v0, v0 + width); the loop contracts it
+// into the float32 grad_hidden slabs and, when grad_weight != null, into the
+// panel's rows of grad_weight, then casts / un-compacts grad_hidden.
+template <class E, class Producer>
+int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidden,
+                       const void* weight, const int64_t* row_idx, int64_t m, int64_t n_out,
+                       int64_t h, int64_t v, int dtype, void* grad_hidden, void* grad_weight,
+                       char* ws, hipStream_t stream, Producer&& produce) {
   using T = typename E::T;
   const bool weight_grad = grad_weight != nullptr;
-  const BackwardLayout l = backward_layout(p, m, h, dtype, weight_grad);
-  float* scale = reinterpret_cast<float*>(ws + l.scale);
   float* acc32 = reinterpret_cast<float*>(ws + l.acc32);
   T* wt = reinterpret_cast<T*>(ws + l.wt);
   T* ht = reinterpret_cast<T*>(ws + l.ht);
   T* g = reinterpret_cast<T*>(ws + l.g);
   T* gt = (weight_grad && !p.kmajor) ? reinterpret_cast<T*>(ws + l.gt) : nullptr;
-
-  ScaleArgs sa;
-  sa.labels = labels; sa.row_idx = row_idx; sa.grad_output = grad_output;
-  sa.valid_count = valid_count; sa.m = (int)m; sa.mp = (int)p.mp; sa.reduction = reduction;
-  sa.ignore = ignore; sa.scale = scale; sa.constant = probabilities_scale;
-  {
-    ScopedTimer timer(kClassOther, stream);
-    lce_token_scale_kernel<<<(int)ceil_div(p.mp, 256), 256, 0, stream>>>(sa);
-  }
-  TLCE_LAUNCH_CHECK();
 
   const T* hidden_t = static_cast<const T*>(hidden);
   const T* weight_t = static_cast<const T*>(weight);
@@ -389,26 +379,12 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     if (int rc = fill_zero(ht + m * h, (m64 - m) * h * (int64_t)sizeof(T), stream)) return rc;
     hidden_k = ht;
   }
-  if (grad_bias != nullptr) {
-    if (int rc = fill_zero(grad_bias, v * 4, stream)) return rc;
-  }
 
   for (int panel = 0; panel < p.n_panels; ++panel) {
     const int64_t v0 = (int64_t)panel * p.vc;
     const int64_t width = std::min<int64_t>(p.vc, p.vp - v0);   // multiple of tile
     const int64_t rows_valid = std::min<int64_t>(p.vc, v - v0);  // real vocabulary rows
-    GradLogitsArgs ga;
-    ga.hidden = hidden; ga.weight = weight; ga.bias = bias; ga.labels = labels;
-    ga.lse = lse; ga.scale = scale;
-    ga.m = (int)m; ga.h = (int)h; ga.v = (int)v;
-    ga.ignore = ignore; ga.exclude = exclude - vocab_start; ga.softcap = softcap;
-    ga.label_offset = vocab_start;
-    ga.probabilities = (labels == nullptr) ? 1 : 0;
-    ga.v0 = (int)v0;
-    ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
-    ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
-    ga.grad_bias = (bias != nullptr) ? grad_bias : nullptr;
-    if (int rc = launch_grad_logits<E>(ga, stream)) return rc;
+    if (int rc = produce(v0, width, g, gt)) return rc;
 
     GemmArgs dh;
     dh.b = g; dh.ldb = p.vc; dh.b_rows = (int)p.mp;
@@ -463,6 +439,177 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
   }
   TLCE_LAUNCH_CHECK();
   return 0;
+}
+
+int launch_token_scale(const ScaleArgs& sa, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_token_scale_kernel<<<(int)ceil_div(sa.mp, 256), 256, 0, stream>>>(sa);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+// vocab_start: global id of weight row 0 (labels and exclude are global ids).
+// labels == null: the "gradient" panel holds softmax * probabilities_scale, so
+// grad_hidden becomes the probability-weighted sum of weight rows.
+template <class E>
+int backward_impl(const Plan& p, const void* hidden, const void* weight, const float* bias,
+                  const int64_t* labels, const int64_t* row_idx, const float* lse,
+                  const float* valid_count, const float* grad_output, int64_t m, int64_t n_out,
+                  int64_t h, int64_t v, int dtype, int reduction, int64_t ignore, int64_t exclude,
+                  float softcap, int64_t vocab_start, void* grad_hidden, void* grad_weight,
+                  float* grad_bias, char* ws, hipStream_t stream,
+                  float probabilities_scale = 0.0f) {
+  const BackwardLayout l = backward_layout(p, m, h, dtype, grad_weight != nullptr);
+  float* scale = reinterpret_cast<float*>(ws + l.scale);
+  ScaleArgs sa;
+  sa.labels = labels; sa.row_idx = row_idx; sa.grad_output = grad_output;
+  sa.valid_count = valid_count; sa.m = (int)m; sa.mp = (int)p.mp; sa.reduction = reduction;
+  sa.ignore = ignore; sa.scale = scale; sa.constant = probabilities_scale;
+  if (int rc = launch_token_scale(sa, stream)) return rc;
+  if (grad_bias != nullptr) {
+    if (int rc = fill_zero(grad_bias, v * 4, stream)) return rc;
+  }
+  auto produce = [&](int64_t v0, int64_t width, void* g, void* gt) -> int {
+    GradLogitsArgs ga;
+    ga.hidden = hidden; ga.weight = weight; ga.bias = bias; ga.labels = labels;
+    ga.lse = lse; ga.scale = scale;
+    ga.m = (int)m; ga.h = (int)h; ga.v = (int)v;
+    ga.ignore = ignore; ga.exclude = exclude - vocab_start; ga.softcap = softcap;
+    ga.label_offset = vocab_start;
+    ga.probabilities = (labels == nullptr) ? 1 : 0;
+    ga.v0 = (int)v0;
+    ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
+    ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
+    ga.grad_bias = (bias != nullptr) ? grad_bias : nullptr;
+    return launch_grad_logits<E>(ga, stream);
+  };
+  return panel_contractions<E>(p, l, hidden, weight, row_idx, m, n_out, h, v, dtype, grad_hidden,
+                               grad_weight, ws, stream, produce);
+}
+
+// -------------------------------------------------------------- frozen KL ----
+// KL(teacher || draft) of two frozen heads over one vocabulary
+// (fused_dflash_kl_forward_cuda / _backward_cuda, fused_linear_ce_cuda.cu:1270-1509).
+// Both heads run on one engine class (the less demanding of the two hidden sizes).
+struct KlLayout {
+  int64_t stats, ones, backward, total;   // backward: BackwardLayout of the draft head
+};
+
+KlLayout kl_layout(const Plan& pd, const Plan& pt, int64_t m, int64_t hd, int dtype) {
+  KlLayout l;
+  l.stats = 0;
+  int64_t off = std::max(forward_layout(pd).total, forward_layout(pt).total);
+  l.ones = off;      off += align256(pd.mp * 4);
+  l.backward = off;  off += backward_layout(pd, m, hd, dtype, false).total;
+  l.total = off;
+  return l;
+}
+
+template <class E, bool kSoftcap>
+int launch_kl_panel_variant(const KlPanelArgs& a, hipStream_t stream) {
+  static int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap>, E::kSmemBytes);
+  if (rc) return rc;
+  const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
+  ScopedTimer timer(kClassGradLogits, stream);
+  lce_kl_panel_kernel<E, kSoftcap><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+template <class E>
+int launch_kl_panel(const KlPanelArgs& a, hipStream_t stream) {
+  if (a.softcap > 0.0f) return launch_kl_panel_variant<E, true>(a, stream);
+  return launch_kl_panel_variant<E, false>(a, stream);
+}
+
+// Teacher probabilities of the panel [v0, v0 + width), then the draft pass over it.
+template <class E>
+int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
+             const void* teacher_hidden, const void* teacher_weight, const float* draft_lse,
+             const float* teacher_lse, const float* ones, const float* scale, int64_t m,
+             int64_t hd, int64_t ht, int64_t v, float softcap, int64_t v0, int64_t width,
+             void* g, float* losses, int mode, hipStream_t stream) {
+  GradLogitsArgs ga;
+  ga.hidden = teacher_hidden; ga.weight = teacher_weight; ga.bias = nullptr;
+  ga.labels = nullptr; ga.lse = teacher_lse; ga.scale = ones;
+  ga.m = (int)m; ga.h = (int)ht; ga.v = (int)v;
+  ga.ignore = 0; ga.exclude = -1; ga.softcap = softcap;
+  ga.label_offset = 0; ga.probabilities = 1;
+  ga.v0 = (int)v0;
+  ga.n_ttiles = pd.n_ttiles; ga.n_ptiles = (int)(width / pd.tile);
+  ga.g = g; ga.ldg = pd.vc; ga.gt = nullptr; ga.ldgt = 0;
+  ga.grad_bias = nullptr;
+  if (int rc = launch_grad_logits<E>(ga, stream)) return rc;
+  KlPanelArgs ka;
+  ka.hidden = draft_hidden; ka.weight = draft_weight; ka.lse = draft_lse; ka.scale = scale;
+  ka.m = (int)m; ka.h = (int)hd; ka.v = (int)v; ka.softcap = softcap;
+  ka.v0 = (int)v0; ka.n_ttiles = pd.n_ttiles; ka.n_ptiles = (int)(width / pd.tile);
+  ka.panel = g; ka.ld = pd.vc; ka.losses = losses; ka.mode = mode;
+  return launch_kl_panel<E>(ka, stream);
+}
+
+template <class E>
+int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const void* draft_hidden,
+                    const void* draft_weight, const void* teacher_hidden,
+                    const void* teacher_weight, int64_t m, int64_t hd, int64_t ht, int64_t v,
+                    int dtype, float softcap, float* losses, float* draft_lse, float* teacher_lse,
+                    char* ws, hipStream_t stream) {
+  if (int rc = forward_impl<E>(pd, draft_hidden, draft_weight, nullptr, nullptr, nullptr, m, hd,
+                               v, 0, -1, softcap, nullptr, draft_lse, nullptr, ShardStats{},
+                               ws + l.stats, stream))
+    return rc;
+  if (int rc = forward_impl<E>(pt, teacher_hidden, teacher_weight, nullptr, nullptr, nullptr, m,
+                               ht, v, 0, -1, softcap, nullptr, teacher_lse, nullptr, ShardStats{},
+                               ws + l.stats, stream))
+    return rc;
+  float* ones = reinterpret_cast<float*>(ws + l.ones);
+  ScaleArgs sa;
+  sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = nullptr; sa.valid_count = nullptr;
+  sa.m = (int)m; sa.mp = (int)pd.mp; sa.reduction = TLCE_REDUCTION_SUM; sa.ignore = 0;
+  sa.scale = ones; sa.constant = 1.0f;
+  if (int rc = launch_token_scale(sa, stream)) return rc;
+  // losses start at sum_v q = 1 per row (the generalised KL's constant term)
+  ScaleArgs init = sa;
+  init.mp = (int)m;
+  init.scale = losses;
+  if (int rc = launch_token_scale(init, stream)) return rc;
+  const BackwardLayout bl = backward_layout(pd, m, hd, dtype, false);
+  void* g = ws + l.backward + bl.g;
+  for (int panel = 0; panel < pd.n_panels; ++panel) {
+    const int64_t v0 = (int64_t)panel * pd.vc;
+    const int64_t width = std::min<int64_t>(pd.vc, pd.vp - v0);
+    if (int rc = kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight,
+                             draft_lse, teacher_lse, ones, nullptr, m, hd, ht, v, softcap, v0,
+                             width, g, losses, kKlLoss, stream))
+      return rc;
+  }
+  return 0;
+}
+
+template <class E>
+int kl_backward_impl(const Plan& pd, const KlLayout& l, const void* draft_hidden,
+                     const void* draft_weight, const void* teacher_hidden,
+                     const void* teacher_weight, const float* draft_lse, const float* teacher_lse,
+                     const float* grad_output, int64_t m, int64_t hd, int64_t ht, int64_t v,
+                     int dtype, float softcap, void* grad_hidden, char* ws, hipStream_t stream) {
+  float* ones = reinterpret_cast<float*>(ws + l.ones);
+  char* bws = ws + l.backward;
+  const BackwardLayout bl = backward_layout(pd, m, hd, dtype, false);
+  float* scale = reinterpret_cast<float*>(bws + bl.scale);
+  ScaleArgs sa;
+  sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = nullptr; sa.valid_count = nullptr;
+  sa.m = (int)m; sa.mp = (int)pd.mp; sa.reduction = TLCE_REDUCTION_NONE; sa.ignore = 0;
+  sa.scale = ones; sa.constant = 1.0f;
+  if (int rc = launch_token_scale(sa, stream)) return rc;
+  sa.grad_output = grad_output; sa.scale = scale;   // scale[r] = grad_output[r]
+  if (int rc = launch_token_scale(sa, stream)) return rc;
+  auto produce = [&](int64_t v0, int64_t width, void* g, void*) -> int {
+    return kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight, draft_lse,
+                       teacher_lse, ones, scale, m, hd, ht, v, softcap, v0, width, g, nullptr,
+                       kKlGrad, stream);
+  };
+  return panel_contractions<E>(pd, bl, draft_hidden, draft_weight, nullptr, m, m, hd, v, dtype,
+                               grad_hidden, nullptr, bws, stream, produce);
 }
 
 }  // namespace
@@ -733,6 +880,91 @@ extern "C" int tlce_soft_embedding(const void* hidden, const void* weight, int64
                 soft_embedding_impl<E>(fp, bp, l, hidden, weight, m, h, v, dtype, logit_softcap,
                                        embedding_scale, out, static_cast<char*>(workspace),
                                        stream));
+}
+
+// ---------------------------------------------------------------- frozen KL --
+namespace {
+
+struct KlPlans {
+  Plan draft, teacher;
+  KlLayout layout;
+};
+
+KlPlans kl_plans(int64_t m, int64_t hd, int64_t ht, int64_t v, int dtype, int64_t panel_bytes) {
+  KlPlans k;
+  const int engine = std::min(engine_class(hd, dtype), engine_class(ht, dtype));
+  k.draft = make_plan(m, hd, v, dtype, false, panel_bytes, engine);
+  k.teacher = make_plan(m, ht, v, dtype, false, panel_bytes, engine);
+  // one engine class for both heads (TLCE_FORCE_ENGINE may have lowered either)
+  const int common = std::min(k.draft.engine, k.teacher.engine);
+  if (k.draft.engine != common) k.draft = make_plan(m, hd, v, dtype, false, panel_bytes, common);
+  if (k.teacher.engine != common) k.teacher = make_plan(m, ht, v, dtype, false, panel_bytes, common);
+  k.layout = kl_layout(k.draft, k.teacher, m, hd, dtype);
+  return k;
+}
+
+int kl_validate(const void* draft_hidden, const void* draft_weight, const void* teacher_hidden,
+                const void* teacher_weight, int64_t m, int64_t hd, int64_t ht, int64_t v,
+                int dtype) {
+  if (int rc = validate_common(draft_hidden, draft_weight, m, hd, v, dtype)) return rc;
+  return validate_common(teacher_hidden, teacher_weight, m, ht, v, dtype);
+}
+
+}  // namespace
+
+extern "C" int64_t tlce_kl_workspace_bytes(int64_t m, int64_t h_draft, int64_t h_teacher,
+                                           int64_t v, int dtype, int64_t panel_bytes) {
+  if (m < 0 || h_draft <= 0 || h_teacher <= 0 || v <= 0) return -1;
+  return kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes).layout.total;
+}
+
+extern "C" int tlce_kl_forward(const void* draft_hidden, const void* draft_weight,
+                               const void* teacher_hidden, const void* teacher_weight, int64_t m,
+                               int64_t h_draft, int64_t h_teacher, int64_t v, int dtype,
+                               float logit_softcap, float* losses, float* draft_lse,
+                               float* teacher_lse, int64_t panel_bytes, void* workspace,
+                               int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = kl_validate(draft_hidden, draft_weight, teacher_hidden, teacher_weight, m,
+                           h_draft, h_teacher, v, dtype))
+    return rc;
+  if (m == 0) return 0;
+  TLCE_REQUIRE(losses && draft_lse && teacher_lse && workspace, "kl_forward: null pointer");
+  const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes);
+  TLCE_REQUIRE(workspace_bytes >= k.layout.total, "kl_forward: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)k.layout.total);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0, "kl_forward: workspace must be 256-byte aligned");
+  TLCE_DISPATCH(k.draft, dtype,
+                kl_forward_impl<E>(k.draft, k.teacher, k.layout, draft_hidden, draft_weight,
+                                   teacher_hidden, teacher_weight, m, h_draft, h_teacher, v, dtype,
+                                   logit_softcap, losses, draft_lse, teacher_lse,
+                                   static_cast<char*>(workspace), stream));
+}
+
+extern "C" int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
+                                const void* teacher_hidden, const void* teacher_weight,
+                                const float* draft_lse, const float* teacher_lse,
+                                const float* grad_output, int64_t m, int64_t h_draft,
+                                int64_t h_teacher, int64_t v, int dtype, float logit_softcap,
+                                void* grad_hidden, int64_t panel_bytes, void* workspace,
+                                int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = kl_validate(draft_hidden, draft_weight, teacher_hidden, teacher_weight, m,
+                           h_draft, h_teacher, v, dtype))
+    return rc;
+  if (m == 0) return 0;
+  TLCE_REQUIRE(draft_lse && teacher_lse && grad_output && grad_hidden && workspace,
+               "kl_backward: null pointer");
+  TLCE_REQUIRE(((uintptr_t)grad_hidden & 15) == 0, "kl_backward: grad_hidden must be 16-byte aligned");
+  const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes);
+  TLCE_REQUIRE(workspace_bytes >= k.layout.total, "kl_backward: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)k.layout.total);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0, "kl_backward: workspace must be 256-byte aligned");
+  TLCE_DISPATCH(k.draft, dtype,
+                kl_backward_impl<E>(k.draft, k.layout, draft_hidden, draft_weight, teacher_hidden,
+                                    teacher_weight, draft_lse, teacher_lse, grad_output, m,
+                                    h_draft, h_teacher, v, dtype, logit_softcap, grad_hidden,
+                                    static_cast<char*>(workspace), stream));
 }
 
 extern "C" int tlce_profile_begin(void) {

@@ -1,0 +1,88 @@
+"""Per-token forward KL between two frozen LM heads without a logits buffer.
+
+Same entry point and checks as the reference module
+(dllm_parallel/core/kernels/dflash_kl.py:74-121): ``frozen_linear_kl`` returns
+``KL(softmax(teacher logits) || softmax(draft logits))`` per token, float32,
+and differentiates with respect to the draft hidden states only.  Device
+tensors run in the HIP library; host tensors take the dense torch expression.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+
+class _FrozenLinearKL(torch.autograd.Function):
+    """Autograd node around the library's KL forward / backward entry points."""
+
+    @staticmethod
+    def forward(ctx, draft_hidden, draft_weight, teacher_hidden, teacher_weight, logit_softcap):
+        from . import chunked_linear_ce_native as native
+
+        operands = tuple(t.contiguous() for t in (draft_hidden, draft_weight, teacher_hidden,
+                                                  teacher_weight))
+        losses, draft_lse, teacher_lse = native.dflash_kl_forward(*operands, float(logit_softcap))
+        ctx.save_for_backward(*operands, draft_lse, teacher_lse)
+        ctx.logit_softcap = float(logit_softcap)
+        return losses
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        from . import chunked_linear_ce_native as native
+
+        *operands, draft_lse, teacher_lse = ctx.saved_tensors
+        grad_hidden = native.dflash_kl_backward(*operands, draft_lse, teacher_lse,
+                                                grad_output.contiguous(), ctx.logit_softcap)
+        return grad_hidden, None, None, None, None
+
+
+def _check(draft_hidden, draft_weight, teacher_hidden, teacher_weight, logit_softcap):
+    # messages of the reference, dflash_kl.py:84-99
+    if draft_hidden.ndim != 2 or teacher_hidden.ndim != 2:
+        raise ValueError("DFlash KL hidden states must be [tokens, hidden]")
+    if draft_hidden.shape[0] != teacher_hidden.shape[0]:
+        raise ValueError("DFlash KL draft and teacher token counts differ")
+    if draft_weight.ndim != 2 or teacher_weight.ndim != 2:
+        raise ValueError("DFlash KL head weights must be [vocabulary, hidden]")
+    if draft_weight.shape[0] != teacher_weight.shape[0]:
+        raise ValueError("DFlash KL draft and teacher vocabularies differ")
+    if draft_weight.shape[1] != draft_hidden.shape[1]:
+        raise ValueError("DFlash KL draft head width is incompatible")
+    if teacher_weight.shape[1] != teacher_hidden.shape[1]:
+        raise ValueError("DFlash KL teacher head width is incompatible")
+    if logit_softcap is not None and logit_softcap <= 0.0:
+        raise ValueError("DFlash KL logit_softcap must be positive")
+
+
+def frozen_linear_kl(
+    draft_hidden: torch.Tensor,
+    draft_weight: torch.Tensor,
+    teacher_hidden: torch.Tensor,
+    teacher_weight: torch.Tensor,
+    *,
+    logit_softcap: float | None = None,
+) -> torch.Tensor:
+    """Per-token forward KL, float32 [tokens]."""
+    _check(draft_hidden, draft_weight, teacher_hidden, teacher_weight, logit_softcap)
+    cap = 0.0 if logit_softcap is None else float(logit_softcap)
+    others = (draft_weight, teacher_hidden, teacher_weight)
+    if draft_hidden.is_cuda:
+        if not all(t.is_cuda for t in others):
+            raise ValueError("DFlash KL tensors must be on one CUDA device")
+        if not all(t.dtype == draft_hidden.dtype for t in others):
+            raise ValueError("DFlash KL tensors must use one dtype")
+        return _FrozenLinearKL.apply(draft_hidden, draft_weight, teacher_hidden, teacher_weight,
+                                     cap)
+    if any(t.is_cuda for t in others):
+        raise ValueError("DFlash KL tensors must be on one device")
+    draft = F.linear(draft_hidden, draft_weight)
+    teacher = F.linear(teacher_hidden, teacher_weight)
+    if cap > 0.0:
+        draft, teacher = (cap * torch.tanh(z / cap) for z in (draft, teacher))
+    log_q = F.log_softmax(draft, dim=-1, dtype=torch.float32)
+    p = F.softmax(teacher, dim=-1, dtype=torch.float32)
+    return F.kl_div(log_q, p, reduction="none").sum(dim=-1)
+
+
+__all__ = ["frozen_linear_kl"]
