@@ -127,8 +127,79 @@ def measured_traffic(workload, kernel):
     return MEASURED_TRAFFIC_BYTES.get(workload, {}).get(kernel)
 
 
+def bench_next_objective(args) -> int:
+    """The objectives built on the same kernels: frozen-head forward KL
+    (forward + backward) and the streaming soft embedding (forward only)."""
+    import torch
+
+    from turbo_dllm_amd import _lib
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    from turbo_dllm_amd.dflash_kl import frozen_linear_kl
+    from turbo_dllm_amd.streaming_soft_embedding import streaming_soft_embedding
+
+    device = torch.device("cuda:0")
+    native.verify_device(0)
+    gen = torch.Generator().manual_seed(args.seed)
+    m = args.rows
+
+    def randn(rows, cols, std):
+        return (torch.randn(rows, cols, generator=gen) * std).bfloat16().to(device)
+
+    if args.objective == "kl":
+        h, v = 4096, 151936
+        draft_w, teacher_w = randn(v, h, 0.02), randn(v, h, 0.02)
+        draft_h = randn(m, h, 1.0).requires_grad_(True)
+        teacher_h = randn(m, h, 1.0)
+
+        def step():
+            draft_h.grad = None
+            frozen_linear_kl(draft_h, draft_w, teacher_h, teacher_w).sum().backward()
+
+        contractions, name = 7, "frozen-head KL fwd+bwd"   # 4 forward + 3 backward
+        shape = f"M={m}, H_draft=H_teacher={h}, V={v}"
+    else:
+        h, v = 3840, 262144
+        weight, hidden = randn(v, h, 0.02), randn(m, h, 1.0)
+
+        def step():
+            streaming_soft_embedding(hidden, weight, row_chunk_size=1024, vocab_chunk_size=8192,
+                                     logit_softcap=30.0)
+
+        contractions, name = 3, "streaming soft embedding fwd"
+        shape = f"M={m}, H={h}, V={v}, softcap=30"
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / args.steps
+    with _lib.kernel_profile() as prof:
+        step()
+    torch.cuda.synchronize()
+    executed = contractions * 2.0 * m * h * v / 1e12 / (ms / 1e3)
+    print(json.dumps({
+        "metric": f"{name} tokens/s", "value": m / (ms / 1e3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.objective}: {shape}, seed={args.seed}"},
+        "contractions_executed": contractions, "tflops_executed": executed,
+        "mfma_util_executed": executed / PEAK_BF16_TFLOPS,
+        "kernel_ms": {k: round(x, 3) for k, x in prof.ms.items()},
+        "kernel_launches": prof.launches,
+    }), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--objective", choices=("ce", "kl", "soft_embedding"), default="ce",
+                    help="ce: the headline fused linear cross-entropy (default); kl / "
+                         "soft_embedding: the objectives built on the same kernels")
+    ap.add_argument("--rows", type=int, default=8192, help="rows for --objective kl / soft_embedding")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
@@ -154,6 +225,8 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
+    if args.objective != "ce":
+        return bench_next_objective(args)
     device = torch.device("cuda:0")
     native.verify_device(0)
 
