@@ -13,6 +13,7 @@
 #include <stdlib.h>
 
 #include <algorithm>
+#include <atomic>
 #include <vector>
 
 #include "tlce_common.h"
@@ -195,11 +196,23 @@ BackwardLayout backward_layout(const Plan& p, int64_t m, int64_t h, int dtype, b
   return l;
 }
 
+// Kernels with more than 64 KiB of dynamic LDS need the limit raised once per
+// kernel and device; `done` is the calling site's per-device record.
+constexpr int kMaxDevices = 64;
+struct LdsOptIn {
+  std::atomic<bool> done[kMaxDevices] = {};
+};
+
 template <typename K>
-int enable_large_lds(K kernel, int bytes) {
+int enable_large_lds(K kernel, int bytes, LdsOptIn& state) {
   if (bytes <= 64 * 1024) return 0;
+  int device = 0;
+  TLCE_HIP(hipGetDevice(&device));
+  const bool tracked = device >= 0 && device < kMaxDevices;
+  if (tracked && state.done[device].load(std::memory_order_acquire)) return 0;
   TLCE_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  if (tracked) state.done[device].store(true, std::memory_order_release);
   return 0;
 }
 
@@ -220,8 +233,9 @@ int validate_common(const void* hidden, const void* weight, int64_t m, int64_t h
 // ---------------------------------------------------------------- launches --
 template <class E, bool kSoftcap, bool kBias>
 int launch_forward_variant(const Plan& p, const ForwardArgs& a, hipStream_t stream) {
-  static int rc = enable_large_lds(lce_forward_stats_kernel<E, kSoftcap, kBias>, E::kSmemBytes);
-  if (rc) return rc;
+  static LdsOptIn lds;
+  if (int rc = enable_large_lds(lce_forward_stats_kernel<E, kSoftcap, kBias>, E::kSmemBytes, lds))
+    return rc;
   const int grid = xcd_grid((int64_t)p.n_ttiles * p.nsplit);
   ScopedTimer timer(kClassForwardStats, stream);
   lce_forward_stats_kernel<E, kSoftcap, kBias><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
@@ -240,9 +254,10 @@ int launch_forward(const Plan& p, const ForwardArgs& a, hipStream_t stream) {
 
 template <class E, bool kSoftcap, bool kBias>
 int launch_grad_logits_variant(const GradLogitsArgs& a, hipStream_t stream) {
-  static int rc =
-      enable_large_lds(lce_grad_logits_panel_kernel<E, kSoftcap, kBias>, E::kSmemBytes);
-  if (rc) return rc;
+  static LdsOptIn lds;
+  if (int rc = enable_large_lds(lce_grad_logits_panel_kernel<E, kSoftcap, kBias>, E::kSmemBytes,
+                                lds))
+    return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
   ScopedTimer timer(kClassGradLogits, stream);
   lce_grad_logits_panel_kernel<E, kSoftcap, kBias>
@@ -262,8 +277,9 @@ int launch_grad_logits(const GradLogitsArgs& a, hipStream_t stream) {
 
 template <class E, bool kAKMajor, bool kBKMajor>
 int launch_gemm(GemmArgs a, int ksplit, int cls, hipStream_t stream) {
-  static int rc = enable_large_lds(lce_gemm_nt_kernel<E, kAKMajor, kBKMajor>, E::kSmemBytes);
-  if (rc) return rc;
+  static LdsOptIn lds;
+  if (int rc = enable_large_lds(lce_gemm_nt_kernel<E, kAKMajor, kBKMajor>, E::kSmemBytes, lds))
+    return rc;
   const int ksteps = a.k / E::kBK;
   a.k_per_split = (int)ceil_div(ksteps, ksplit) * E::kBK;
   dim3 grid(xcd_grid((int64_t)a.ni * a.nj), ksplit, 1);
@@ -507,8 +523,8 @@ KlLayout kl_layout(const Plan& pd, const Plan& pt, int64_t m, int64_t hd, int dt
 
 template <class E, bool kSoftcap>
 int launch_kl_panel_variant(const KlPanelArgs& a, hipStream_t stream) {
-  static int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap>, E::kSmemBytes);
-  if (rc) return rc;
+  static LdsOptIn lds;
+  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap>, E::kSmemBytes, lds)) return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
   ScopedTimer timer(kClassGradLogits, stream);
   lce_kl_panel_kernel<E, kSoftcap><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
