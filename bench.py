@@ -155,7 +155,7 @@ def bench_next_objective(args) -> int:
             draft_h.grad = None
             frozen_linear_kl(draft_h, draft_w, teacher_h, teacher_w).sum().backward()
 
-        contractions, name = 7, "frozen-head KL fwd+bwd"   # 4 forward + 3 backward
+        contractions, name = 6, "frozen-head KL fwd+bwd"   # 3 forward + 3 backward
         shape = f"M={m}, H_draft=H_teacher={h}, V={v}"
     else:
         h, v = 3840, 262144

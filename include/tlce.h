@@ -201,7 +201,10 @@ int tlce_soft_embedding(const void* hidden, const void* weight, int64_t m,
  * reference.  No logits buffer: the teacher probabilities cross memory in the
  * same bounded vocabulary panels as the cross-entropy backward (rounded to
  * `dtype`; the loss is accumulated as the generalised KL sum t log(t/q) - t + q,
- * which is insensitive to that rounding to first order).
+ * which is insensitive to that rounding to first order).  Forward: one
+ * statistics pass over the teacher head, then per panel the teacher
+ * probabilities and one pass over the draft head that yields both the loss
+ * terms and the draft's softmax statistics.
  *   draft_hidden [m,h_draft], draft_weight [v,h_draft], teacher_hidden
  *   [m,h_teacher], teacher_weight [v,h_teacher], all `dtype`; losses,
  *   draft_lse, teacher_lse, grad_output: float32 [m]; grad_hidden [m,h_draft]. */

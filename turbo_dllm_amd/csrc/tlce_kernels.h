@@ -441,10 +441,14 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 // t = softmax(cap(z_teacher)) rounded to the input dtype (written by
 // lce_grad_logits_panel_kernel in its probabilities mode).  This kernel
 // recomputes the draft logits tile and, with lp = cap(z_draft) - lse_draft:
-//   mode kKlLoss: losses[token] += sum_v ( t * (log t - lp) - t )
-//                 (the generalised KL; the caller adds 1 per row = sum_v q.
-//                 It equals sum_v p_t (log p_t - log p_d) to first order in the
-//                 rounding of t, where the plain sum would be off by sum_v dt)
+//   mode kKlLoss: losses[token] += sum_v ( t * (log t - cap(z_draft)) - t ),
+//                 tsum[token] += sum_v t, and the tile's (max, sum exp) of the
+//                 draft logits go to the forward partial arrays, so that no
+//                 separate statistics pass over the draft head is needed.  The
+//                 caller finishes with loss = losses + tsum * lse_draft + 1: the
+//                 generalised KL sum_v t log(t/q) - t + q, which equals
+//                 sum_v p_t (log p_t - log p_d) to first order in the rounding
+//                 of t (the plain sum would be off by sum_v dt).  lse is not read.
 //   mode kKlGrad: panel[token, v] = (exp(lp) - t) * scale[token] * cap'(z_draft)
 //                 in place, rounded to the input dtype: the logit gradient that
 //                 feeds the grad-hidden contraction.
@@ -462,6 +466,10 @@ struct KlPanelArgs {
   void* panel;          // [mp, ld] teacher probabilities in, logit gradients out
   int64_t ld;
   float* losses;        // kKlLoss: [m], accumulated with atomics
+  float* tsum;          // kKlLoss: [m], accumulated with atomics
+  float* part_max;      // kKlLoss: [n vocabulary tiles, part_ld] base-2 tile maxima
+  float* part_sum;      //          and sums of exp2(z2 - max2), as the forward writes them
+  int part_ld;
   int mode;
 };
 
@@ -483,16 +491,36 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
 
   const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
   const bool grad = p.mode == kKlGrad;
-  float lse2[E::kCols], scale[E::kCols], partial[E::kCols];
+  float lse2[E::kCols], scale[E::kCols], partial[E::kCols], tsum[E::kCols];
+  float tile_max[E::kCols], tile_sum[E::kCols];
   bool live[E::kCols];
 #pragma unroll
   for (int j = 0; j < E::kCols; ++j) {
     const int r = tt * E::kTile + eng.col(j);
     const int rc = min(r, p.m - 1);
     live[j] = r < p.m;
-    lse2[j] = p.lse[rc] * TLCE_LOG2E;
+    lse2[j] = grad ? p.lse[rc] * TLCE_LOG2E : 0.0f;
     scale[j] = (grad && live[j]) ? p.scale[rc] : 0.0f;
     partial[j] = 0.0f;
+    tsum[j] = 0.0f;
+    tile_max[j] = -INFINITY;
+    tile_sum[j] = 0.0f;
+  }
+  if (!grad) {
+    // maxima of the capped draft logits per owned column (base-2 units) for the
+    // tile's softmax partial; the capped values replace the raw accumulators
+#pragma unroll
+    for (int i = 0; i < E::kRows; ++i) {
+      const bool vok = vbase + eng.row(i) < p.v;
+#pragma unroll
+      for (int j = 0; j < E::kCols; ++j) {
+        float z = E::get(acc, j, i);
+        if (kSoftcap) z = p.softcap * fast_tanh(z * inv_cap);
+        z = vok ? z * TLCE_LOG2E : -INFINITY;
+        E::set(acc, j, i, z);
+        tile_max[j] = fmaxf(tile_max[j], z);
+      }
+    }
   }
   T* panel = static_cast<T*>(p.panel);
   const int prow = pv * E::kTile;   // first panel column of this tile
@@ -506,20 +534,24 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
       const int row = eng.row(i4 + u);
       const bool vok = vbase + row < p.v;
       float z = E::get(acc, j, i4 + u);
-      float dcap = 1.0f;
-      if (kSoftcap) {
-        const float th = fast_tanh(z * inv_cap);
-        z = p.softcap * th;
-        dcap = 1.0f - th * th;
-      }
-      const float lp2 = fmaf(z, TLCE_LOG2E, -lse2[j]);   // log2 of the draft probability
       if (grad) {
+        float dcap = 1.0f;
+        if (kSoftcap) {
+          const float th = fast_tanh(z * inv_cap);
+          z = p.softcap * th;
+          dcap = 1.0f - th * th;
+        }
+        const float lp2 = fmaf(z, TLCE_LOG2E, -lse2[j]);   // log2 of the draft probability
         const float v = (fast_exp2(lp2) - t[u]) * scale[j] * dcap;
         g[u] = vok ? v : 0.0f;
       } else {
+        // z already is the capped draft logit in base-2 units (-inf past the vocabulary)
         const float tv = t[u];
-        const float term = tv * ((fast_log2(tv) - lp2) * TLCE_LN2) - tv;
-        if (vok && tv > 0.0f) partial[j] += term;
+        if (vok) tile_sum[j] += fast_exp2(z - tile_max[j]);
+        if (vok && tv > 0.0f) {
+          partial[j] += tv * ((fast_log2(tv) - z) * TLCE_LN2) - tv;
+          tsum[j] += tv;
+        }
       }
     }
   };
@@ -584,9 +616,47 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
 #pragma unroll
     for (int j = 0; j < E::kCols; ++j) {
       const float total = eng.reduce_over_rows_in_wave(partial[j]);
-      if (eng.row_leader() && live[j]) atomicAdd(p.losses + tt * E::kTile + eng.col(j), total);
+      const float total_t = eng.reduce_over_rows_in_wave(tsum[j]);
+      if (eng.row_leader() && live[j]) {
+        atomicAdd(p.losses + tt * E::kTile + eng.col(j), total);
+        atomicAdd(p.tsum + tt * E::kTile + eng.col(j), total_t);
+      }
+    }
+    // merge the kShare threads that hold the same token column and publish the
+    // tile's partial, as the forward kernel does per vocabulary split
+    __syncthreads();
+    float* sh_max = reinterpret_cast<float*>(smem);
+    float* sh_sum = sh_max + E::kShare * E::kTile;
+    const int slot = eng.share_slot();
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      sh_max[slot * E::kTile + eng.col(j)] = tile_max[j];
+      sh_sum[slot * E::kTile + eng.col(j)] = tile_sum[j];
+    }
+    __syncthreads();
+    const int tile_index = vbase / E::kTile;
+    for (int c = threadIdx.x; c < E::kTile; c += E::kThreads) {
+      float mx = -INFINITY;
+#pragma unroll
+      for (int sl = 0; sl < E::kShare; ++sl) mx = fmaxf(mx, sh_max[sl * E::kTile + c]);
+      float sum = 0.0f;
+      if (mx > -INFINITY) {
+#pragma unroll
+        for (int sl = 0; sl < E::kShare; ++sl)
+          sum += sh_sum[sl * E::kTile + c] * fast_exp2(sh_max[sl * E::kTile + c] - mx);
+      }
+      const int64_t o = (int64_t)tile_index * p.part_ld + tt * E::kTile + c;
+      p.part_max[o] = mx;
+      p.part_sum[o] = sum;
     }
   }
+}
+
+// losses[r] = losses[r] + tsum[r] * lse_draft[r] + 1  (see lce_kl_panel_kernel)
+__global__ __launch_bounds__(256) void lce_kl_finish_kernel(float* losses, const float* tsum,
+                                                            const float* lse, int m) {
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r < m) losses[r] = losses[r] + tsum[r] * lse[r] + 1.0f;
 }
 
 // C[j][i] (op)= sum_k A[i][k] * B[j][k]  - the two gradient contractions, with

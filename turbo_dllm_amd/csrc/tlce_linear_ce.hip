@@ -508,14 +508,19 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
 // (fused_dflash_kl_forward_cuda / _backward_cuda, fused_linear_ce_cuda.cu:1270-1509).
 // Both heads run on one engine class (the less demanding of the two hidden sizes).
 struct KlLayout {
-  int64_t stats, ones, backward, total;   // backward: BackwardLayout of the draft head
+  // stats: the teacher's forward partials, then the draft's per-tile partials
+  // (part_max, part_sum: n_vtiles x mp float32 each); backward: BackwardLayout
+  // of the draft head
+  int64_t stats, tile_part, ones, tsum, backward, total;
 };
 
 KlLayout kl_layout(const Plan& pd, const Plan& pt, int64_t m, int64_t hd, int dtype) {
   KlLayout l;
   l.stats = 0;
-  int64_t off = std::max(forward_layout(pd).total, forward_layout(pt).total);
+  l.tile_part = align256((int64_t)pd.n_vtiles * pd.mp * 4);
+  int64_t off = std::max(2 * l.tile_part, forward_layout(pt).total);
   l.ones = off;      off += align256(pd.mp * 4);
+  l.tsum = off;      off += align256(pd.mp * 4);
   l.backward = off;  off += backward_layout(pd, m, hd, dtype, false).total;
   l.total = off;
   return l;
@@ -544,7 +549,8 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
              const void* teacher_hidden, const void* teacher_weight, const float* draft_lse,
              const float* teacher_lse, const float* ones, const float* scale, int64_t m,
              int64_t hd, int64_t ht, int64_t v, float softcap, int64_t v0, int64_t width,
-             void* g, float* losses, int mode, hipStream_t stream) {
+             void* g, float* losses, float* tsum, float* part_max, float* part_sum, int mode,
+             hipStream_t stream) {
   GradLogitsArgs ga;
   ga.hidden = teacher_hidden; ga.weight = teacher_weight; ga.bias = nullptr;
   ga.labels = nullptr; ga.lse = teacher_lse; ga.scale = ones;
@@ -560,7 +566,8 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
   ka.hidden = draft_hidden; ka.weight = draft_weight; ka.lse = draft_lse; ka.scale = scale;
   ka.m = (int)m; ka.h = (int)hd; ka.v = (int)v; ka.softcap = softcap;
   ka.v0 = (int)v0; ka.n_ttiles = pd.n_ttiles; ka.n_ptiles = (int)(width / pd.tile);
-  ka.panel = g; ka.ld = pd.vc; ka.losses = losses; ka.mode = mode;
+  ka.panel = g; ka.ld = pd.vc; ka.losses = losses; ka.tsum = tsum;
+  ka.part_max = part_max; ka.part_sum = part_sum; ka.part_ld = (int)pd.mp; ka.mode = mode;
   return launch_kl_panel<E>(ka, stream);
 }
 
@@ -570,35 +577,51 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
                     const void* teacher_weight, int64_t m, int64_t hd, int64_t ht, int64_t v,
                     int dtype, float softcap, float* losses, float* draft_lse, float* teacher_lse,
                     char* ws, hipStream_t stream) {
-  if (int rc = forward_impl<E>(pd, draft_hidden, draft_weight, nullptr, nullptr, nullptr, m, hd,
-                               v, 0, -1, softcap, nullptr, draft_lse, nullptr, ShardStats{},
-                               ws + l.stats, stream))
-    return rc;
+  using T = typename E::T;
+  // teacher statistics first: its probabilities need the teacher lse
   if (int rc = forward_impl<E>(pt, teacher_hidden, teacher_weight, nullptr, nullptr, nullptr, m,
                                ht, v, 0, -1, softcap, nullptr, teacher_lse, nullptr, ShardStats{},
                                ws + l.stats, stream))
     return rc;
   float* ones = reinterpret_cast<float*>(ws + l.ones);
+  float* tsum = reinterpret_cast<float*>(ws + l.tsum);
+  float* part_max = reinterpret_cast<float*>(ws + l.stats);
+  float* part_sum = reinterpret_cast<float*>(ws + l.stats + l.tile_part);
   ScaleArgs sa;
   sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = nullptr; sa.valid_count = nullptr;
   sa.m = (int)m; sa.mp = (int)pd.mp; sa.reduction = TLCE_REDUCTION_SUM; sa.ignore = 0;
   sa.scale = ones; sa.constant = 1.0f;
   if (int rc = launch_token_scale(sa, stream)) return rc;
-  // losses start at sum_v q = 1 per row (the generalised KL's constant term)
-  ScaleArgs init = sa;
-  init.mp = (int)m;
-  init.scale = losses;
-  if (int rc = launch_token_scale(init, stream)) return rc;
+  if (int rc = fill_zero(tsum, pd.mp * 4, stream)) return rc;
+  if (int rc = fill_zero(losses, m * 4, stream)) return rc;
+  // one pass over the draft head per panel: loss terms and the draft's per-tile
+  // softmax partials (the teacher partials above are dead by now)
   const BackwardLayout bl = backward_layout(pd, m, hd, dtype, false);
   void* g = ws + l.backward + bl.g;
   for (int panel = 0; panel < pd.n_panels; ++panel) {
     const int64_t v0 = (int64_t)panel * pd.vc;
     const int64_t width = std::min<int64_t>(pd.vc, pd.vp - v0);
     if (int rc = kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight,
-                             draft_lse, teacher_lse, ones, nullptr, m, hd, ht, v, softcap, v0,
-                             width, g, losses, kKlLoss, stream))
+                             nullptr, teacher_lse, ones, nullptr, m, hd, ht, v, softcap, v0,
+                             width, g, losses, tsum, part_max, part_sum, kKlLoss, stream))
       return rc;
   }
+  CombineArgs ca;
+  ca.hidden = draft_hidden; ca.weight = draft_weight; ca.bias = nullptr; ca.labels = nullptr;
+  ca.row_idx = nullptr;
+  ca.m = (int)m; ca.h = (int)hd; ca.v = (int)v;
+  ca.ignore = 0; ca.exclude = -1; ca.softcap = softcap;
+  ca.part_max = part_max; ca.part_sum = part_sum;
+  ca.part_ld = (int)pd.mp; ca.nsplit = pd.n_vtiles;
+  ca.losses = nullptr; ca.lse = draft_lse; ca.valid_count = nullptr;
+  ca.label_offset = 0; ca.local_max = nullptr; ca.local_sum = nullptr; ca.target_logits = nullptr;
+  {
+    ScopedTimer timer(kClassCombine, stream);
+    lce_combine_loss_kernel<T><<<(int)ceil_div(m, 4), 256, 0, stream>>>(ca);
+    lce_kl_finish_kernel<<<(int)ceil_div(m, 256), 256, 0, stream>>>(losses, tsum, draft_lse,
+                                                                    (int)m);
+  }
+  TLCE_LAUNCH_CHECK();
   return 0;
 }
 
@@ -622,7 +645,7 @@ int kl_backward_impl(const Plan& pd, const KlLayout& l, const void* draft_hidden
   auto produce = [&](int64_t v0, int64_t width, void* g, void*) -> int {
     return kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight, draft_lse,
                        teacher_lse, ones, scale, m, hd, ht, v, softcap, v0, width, g, nullptr,
-                       kKlGrad, stream);
+                       nullptr, nullptr, nullptr, kKlGrad, stream);
   };
   return panel_contractions<E>(pd, bl, draft_hidden, draft_weight, nullptr, m, m, hd, v, dtype,
                                grad_hidden, nullptr, bws, stream, produce);
