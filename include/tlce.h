@@ -226,6 +226,47 @@ int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
                      void* grad_hidden, int64_t panel_bytes, void* workspace,
                      int64_t workspace_bytes, void* stream);
 
+/* ---- frozen-head cross entropy with exact top-k ---------------------------
+ * Replaces dflash_ce_topk_forward / dflash_ce_topk_backward
+ * (fused_linear_ce.cpp:332-354; fused_linear_ce_cuda.cu:482-599,1511-1773;
+ * torch form in dllm_parallel/core/kernels/dflash_linear_topk.py:100-225):
+ *   z = cap(output_multiplier * hidden . weight^T),  losses = lse(z) - z[label],
+ *   probabilities = exp(-losses), top_values / top_ids = the top_k largest z of
+ *   every row, sorted descending (ties towards the smaller id), lse [m].
+ * The logits cross memory once, in float32, in vocabulary panels bounded by
+ * `panel_bytes`; a per-row scan folds each panel into the running softmax
+ * statistics and the running top-k list.  top_k <= 256.
+ * Backward (hidden only; the head is frozen):
+ *   grad_hidden = (softmax(z) * ce_scale[r] * dz/draw) . weight
+ *                 - ce_scale[r] * dz/draw[label] * weight[label]
+ *                 + sum_j grad_top_values[r,j] * dz/draw[id_j] * weight[id_j]
+ * with ce_scale = grad_loss - grad_probability * probability (the caller forms
+ * it) and grad_top_values optional (NULL: no such term).
+ *   hidden [m,h], weight [v,h] (`dtype`), labels [m] int64 in [0, v);
+ *   float32: losses, probabilities, lse, ce_scale [m], top_values and
+ *   grad_top_values [m,top_k]; top_ids int64 [m,top_k]; grad_hidden [m,h]. */
+int64_t tlce_ce_topk_forward_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                             int dtype, int64_t panel_bytes);
+int64_t tlce_ce_topk_backward_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                              int dtype, int64_t panel_bytes);
+
+int tlce_ce_topk_forward(const void* hidden, const void* weight,
+                         const int64_t* labels, int64_t m, int64_t h, int64_t v,
+                         int dtype, int top_k, float output_multiplier,
+                         float logit_softcap, float* losses, float* probabilities,
+                         float* top_values, int64_t* top_ids, float* lse,
+                         int64_t panel_bytes, void* workspace,
+                         int64_t workspace_bytes, void* stream);
+
+int tlce_ce_topk_backward(const void* hidden, const void* weight,
+                          const int64_t* labels, const float* lse,
+                          const int64_t* top_ids, const float* ce_scale,
+                          const float* grad_top_values, int64_t m, int64_t h,
+                          int64_t v, int dtype, int top_k, float output_multiplier,
+                          float logit_softcap, void* grad_hidden,
+                          int64_t panel_bytes, void* workspace,
+                          int64_t workspace_bytes, void* stream);
+
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be
  * NULL.  `engine` is 2 for the bf16/f16 MFMA kernels with direct-to-LDS loads

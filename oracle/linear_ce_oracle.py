@@ -31,6 +31,9 @@ What each function follows in the reference (paths relative to its tree):
                            (dflash_kl_forward_kernel / dflash_kl_grad_logits_kernel,
                            fused_linear_ce_cuda.cu:367-480; dense form in
                            dllm_parallel/core/kernels/dflash_kl.py:108-121).
+  dense_ce_topk(_grad)     frozen-head CE with the label's probability and the exact
+                           top-k logits, and its gradient for hidden
+                           (dllm_parallel/core/kernels/dflash_linear_topk.py:100-225).
   combine_vocab_shards     the MAX / SUM reductions over shards and the loss of
                            dllm_parallel/core/parallel/tensor_parallel/cross_entropy.py:238-252.
 
@@ -335,3 +338,38 @@ def dense_frozen_kl_grad(draft_hidden, draft_weight, teacher_hidden, teacher_wei
                                    logit_softcap, dtype)
     g = (torch.exp(log_q) - torch.exp(log_p)) * grad_output.to(dtype)[:, None] * dcap
     return g @ draft_weight.to(dtype)
+
+
+def _topk_logits(hidden, weight, output_multiplier, logit_softcap, dtype):
+    raw = hidden.to(dtype) @ weight.to(dtype).t() * output_multiplier
+    if logit_softcap:
+        th = torch.tanh(raw / logit_softcap)
+        return logit_softcap * th, output_multiplier * (1.0 - th * th)
+    return raw, torch.full_like(raw, output_multiplier)
+
+
+def dense_ce_topk(hidden, weight, labels, top_k, *, output_multiplier=1.0, logit_softcap=None,
+                  dtype=torch.float64):
+    """(loss, probability, top_values, top_ids, lse); the top-k sorted descending,
+    equal values in ascending id order."""
+    z, _ = _topk_logits(hidden, weight, output_multiplier, logit_softcap, dtype)
+    lse = torch.logsumexp(z, dim=-1)
+    loss = lse - z.gather(1, labels.reshape(-1, 1).to(torch.long))[:, 0]
+    order = torch.sort(z, dim=-1, descending=True, stable=True).indices[:, :top_k]
+    return loss, torch.exp(-loss), z.gather(1, order), order, lse
+
+
+def dense_ce_topk_grad(hidden, weight, labels, top_ids, grad_loss, grad_probability,
+                       grad_top_values, *, output_multiplier=1.0, logit_softcap=None,
+                       dtype=torch.float64):
+    """d(sum grad_loss*loss + grad_probability*probability + grad_top_values*top_values)/d hidden."""
+    z, dz = _topk_logits(hidden, weight, output_multiplier, logit_softcap, dtype)
+    lse = torch.logsumexp(z, dim=-1)
+    y = labels.reshape(-1, 1).to(torch.long)
+    prob = torch.exp(z.gather(1, y)[:, 0] - lse)
+    ce_scale = grad_loss.to(dtype) - grad_probability.to(dtype) * prob
+    g = torch.exp(z - lse[:, None]) * ce_scale[:, None]
+    g.scatter_add_(1, y, -ce_scale[:, None])
+    if grad_top_values is not None:
+        g.scatter_add_(1, top_ids.to(torch.long), grad_top_values.to(dtype))
+    return (g * dz) @ weight.to(dtype)

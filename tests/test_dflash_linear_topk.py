@@ -1,0 +1,123 @@
+"""Frozen-head CE with exact top-k: argument checks and the dense path on the
+CPU, the device path against the float64 oracle."""
+
+import pytest
+import torch
+
+import linear_ce_oracle as oracle
+from turbo_dllm_amd.dflash_linear_topk import frozen_linear_ce_topk
+
+
+def test_argument_checks():
+    h, w, y = torch.randn(4, 8), torch.randn(11, 8), torch.randint(0, 11, (4,))
+    with pytest.raises(ValueError, match=r"expects \[N,D\], \[V,D\], and \[N\]"):
+        frozen_linear_ce_topk(h, w, y[None], top_k=2)
+    with pytest.raises(ValueError, match="dimensions are incompatible"):
+        frozen_linear_ce_topk(h, torch.randn(11, 7), y, top_k=2)
+    with pytest.raises(ValueError, match="frozen weight"):
+        frozen_linear_ce_topk(h, w.clone().requires_grad_(True), y, top_k=2)
+    with pytest.raises(ValueError, match="vocabulary range"):
+        frozen_linear_ce_topk(h, w, y, top_k=12)
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        frozen_linear_ce_topk(h, w, torch.full((4,), 11), top_k=2)
+    with pytest.raises(ValueError, match="must be positive"):
+        frozen_linear_ce_topk(h, w, y, top_k=2, logit_softcap=0.0)
+
+
+@pytest.mark.parametrize("softcap,mult", [(None, 1.0), (3.0, 0.5)])
+def test_dense_path_matches_oracle(softcap, mult):
+    torch.manual_seed(5)
+    n, h, v, k = 9, 6, 23, 5
+    hidden = torch.randn(n, h, requires_grad=True)
+    weight = torch.randn(v, h)
+    labels = torch.randint(0, v, (n,))
+    loss, prob, vals, ids = frozen_linear_ce_topk(hidden, weight, labels, top_k=k,
+                                                  output_multiplier=mult, logit_softcap=softcap)
+    gl, gp, gv = torch.randn(n), torch.randn(n), torch.randn(n, k)
+    ((gl * loss).sum() + (gp * prob).sum() + (gv * vals).sum()).backward()
+    r_loss, r_prob, r_vals, r_ids, _ = oracle.dense_ce_topk(
+        hidden.detach(), weight, labels, k, output_multiplier=mult, logit_softcap=softcap)
+    torch.testing.assert_close(loss.double(), r_loss, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(prob.double(), r_prob, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(vals.double(), r_vals, rtol=1e-5, atol=1e-5)
+    assert torch.equal(ids, r_ids)
+    r_grad = oracle.dense_ce_topk_grad(hidden.detach(), weight, labels, ids, gl, gp, gv,
+                                       output_multiplier=mult, logit_softcap=softcap)
+    torch.testing.assert_close(hidden.grad.double(), r_grad, rtol=1e-4, atol=1e-5)
+
+
+GPU_CASES = [
+    # name, dtype, N, H, V, k, softcap, multiplier, weight std, panel bytes
+    ("bf16_staged_h72", torch.bfloat16, 61, 72, 1025, 4, None, 1.0, 0.3, 0),
+    ("bf16_direct", torch.bfloat16, 300, 256, 2304, 8, None, 1.0, 0.1, 0),
+    ("bf16_direct_softcap_mult", torch.bfloat16, 129, 128, 1536, 16, 5.0, 0.6, 0.3, 0),
+    ("f16_three_panels_k1", torch.float16, 520, 64, 1024, 1, None, 1.0, 0.3, 768 * 512 * 4),
+    ("bf16_wide_chunks_k33", torch.bfloat16, 40, 64, 40000, 33, None, 2.0, 0.2, 0),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", GPU_CASES, ids=[c[0] for c in GPU_CASES])
+def test_device_path_matches_oracle(gpu_device, case, monkeypatch):
+    name, dtype, n, h, v, k, softcap, mult, std, panel_bytes = case
+    print("[case]", name, flush=True)
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    if panel_bytes:
+        monkeypatch.setattr(native, "PANEL_BYTES", panel_bytes)
+    gen = torch.Generator().manual_seed(len(name) + k)
+    hidden = torch.randn(n, h, generator=gen).to(dtype)
+    weight = (torch.randn(v, h, generator=gen) * std).to(dtype)
+    labels = torch.randint(0, v, (n,), generator=gen)
+    gl, gp, gv = (torch.randn(n, generator=gen), torch.randn(n, generator=gen),
+                  torch.randn(n, k, generator=gen))
+    x = hidden.to(gpu_device).requires_grad_(True)
+    loss, prob, vals, ids = frozen_linear_ce_topk(x, weight.to(gpu_device), labels.to(gpu_device),
+                                                  top_k=k, output_multiplier=mult,
+                                                  logit_softcap=softcap)
+    ((gl.to(gpu_device) * loss).sum() + (gp.to(gpu_device) * prob).sum()
+     + (gv.to(gpu_device) * vals).sum()).backward()
+    torch.cuda.synchronize()
+    r_loss, r_prob, r_vals, r_ids, _ = oracle.dense_ce_topk(
+        hidden, weight, labels, k, output_multiplier=mult, logit_softcap=softcap)
+    z = oracle._topk_logits(hidden, weight, mult, softcap, torch.float64)[0]
+    loss, prob, vals, ids = (t.detach().cpu() for t in (loss, prob, vals, ids))
+    torch.testing.assert_close(loss.double(), r_loss, rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(prob.double(), r_prob, rtol=2e-3, atol=1e-4)
+    # the values are the row's k largest logits in descending order, and the ids name them;
+    # ids may differ from the oracle's only where float32 rounding reorders near-equal logits
+    torch.testing.assert_close(vals.double(), r_vals, rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(z.gather(1, ids), vals.double(), rtol=1e-3, atol=1e-3)
+    assert bool((vals[:, :-1] >= vals[:, 1:]).all()) if k > 1 else True
+    assert ids.dtype == torch.long and bool(((ids >= 0) & (ids < v)).all())
+    assert all(len(set(row)) == k for row in ids.tolist())
+    agree = float((ids == r_ids).double().mean())
+    print("[case] ids agreeing with the oracle", agree, flush=True)
+    assert agree > 0.97
+    r_grad = oracle.dense_ce_topk_grad(hidden, weight, labels, ids, gl, gp, gv,
+                                       output_multiplier=mult, logit_softcap=softcap)
+    err = oracle.relative_max_error(x.grad.cpu(), r_grad)
+    print("[case] grad rel max err", f"{err:.2e}", flush=True)
+    assert err <= 2e-2
+
+
+@pytest.mark.gpu
+def test_only_loss_gradient_matches_cross_entropy_backward(gpu_device):
+    """With gradients for the loss alone the result equals the frozen-weight
+    cross-entropy backward of the main path."""
+    from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+    gen = torch.Generator().manual_seed(3)
+    n, h, v = 260, 128, 2048
+    hidden = torch.randn(n, h, generator=gen).bfloat16().to(gpu_device)
+    weight = (torch.randn(v, h, generator=gen) * 0.2).bfloat16().to(gpu_device)
+    labels = torch.randint(0, v, (n,), generator=gen).to(gpu_device)
+    a = hidden.clone().requires_grad_(True)
+    loss, _, _, _ = frozen_linear_ce_topk(a, weight, labels, top_k=3)
+    loss.sum().backward()
+    b = hidden.clone().requires_grad_(True)
+    ref = tiled_linear_cross_entropy(b, weight, labels, reduction="sum", dtype=torch.bfloat16,
+                                     weight_layout="vocab_first")
+    ref.backward()
+    torch.cuda.synchronize()
+    torch.testing.assert_close(loss.sum(), ref, rtol=1e-4, atol=1e-2)
+    denom = float(b.grad.float().abs().max())
+    assert float((a.grad.float() - b.grad.float()).abs().max()) <= 1e-2 * denom

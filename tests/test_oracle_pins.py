@@ -310,3 +310,38 @@ def test_frozen_kl_oracle_matches_library_kl_div_and_autograd(softcap):
                                        logit_softcap=softcap)
     assert float(zero.abs().max()) < 1e-12
     assert bool((got >= 0).all())
+
+
+@pytest.mark.parametrize("softcap,mult", [(None, 1.0), (2.0, 0.7)])
+def test_ce_topk_oracle_matches_library_topk_and_autograd(softcap, mult):
+    torch.manual_seed(41)
+    n, h, v, k = 6, 5, 17, 4
+    hidden = torch.randn(n, h, dtype=torch.float64, requires_grad=True)
+    weight = torch.randn(v, h, dtype=torch.float64)
+    labels = torch.randint(0, v, (n,))
+    z = hidden @ weight.t() * mult
+    if softcap:
+        z = softcap * torch.tanh(z / softcap)
+    loss = F.cross_entropy(z, labels, reduction="none")
+    values, ids = z.topk(k, dim=-1)
+    gl, gp, gv = torch.randn(n).double(), torch.randn(n).double(), torch.randn(n, k).double()
+    objective = (gl * loss).sum() + (gp * torch.exp(-loss)).sum() + (gv * values).sum()
+    grad = torch.autograd.grad(objective, hidden)[0]
+    o_loss, o_prob, o_vals, o_ids, o_lse = oracle.dense_ce_topk(
+        hidden.detach(), weight, labels, k, output_multiplier=mult, logit_softcap=softcap)
+    torch.testing.assert_close(o_loss, loss.detach(), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(o_prob, torch.exp(-loss).detach(), rtol=1e-12, atol=1e-12)
+    torch.testing.assert_close(o_vals, values.detach(), rtol=0, atol=0)
+    assert torch.equal(o_ids, ids)
+    torch.testing.assert_close(o_lse, torch.logsumexp(z, dim=-1).detach(), rtol=1e-12, atol=1e-12)
+    o_grad = oracle.dense_ce_topk_grad(hidden.detach(), weight, labels, ids, gl, gp, gv,
+                                       output_multiplier=mult, logit_softcap=softcap)
+    torch.testing.assert_close(o_grad, grad, rtol=1e-10, atol=1e-12)
+
+
+def test_ce_topk_oracle_orders_ties_by_id():
+    hidden = torch.tensor([[1.0, 0.0]], dtype=torch.float64)
+    weight = torch.tensor([[2.0, 0.0], [3.0, 1.0], [2.0, 5.0], [3.0, -1.0], [1.0, 0.0]],
+                          dtype=torch.float64)
+    _, _, vals, ids, _ = oracle.dense_ce_topk(hidden, weight, torch.tensor([0]), 4)
+    assert ids.tolist() == [[1, 3, 0, 2]] and vals.tolist() == [[3.0, 3.0, 2.0, 2.0]]

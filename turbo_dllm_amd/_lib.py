@@ -113,6 +113,32 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_ce_topk_forward_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int, c_int64]
+    ),
+    "tlce_ce_topk_backward_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int, c_int64]
+    ),
+    "tlce_ce_topk_forward": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p,                       # hidden weight labels
+            c_int64, c_int64, c_int64, c_int, c_int,            # m h v dtype top_k
+            c_float, c_float,                                   # multiplier softcap
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # losses probs top_values top_ids lse
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
+    "tlce_ce_topk_backward": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p,             # hidden weight labels lse
+            c_void_p, c_void_p, c_void_p,                       # top_ids ce_scale grad_top_values
+            c_int64, c_int64, c_int64, c_int, c_int,            # m h v dtype top_k
+            c_float, c_float, c_void_p,                         # multiplier softcap grad_hidden
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
     "tlce_profile_begin": (c_int, []),
     "tlce_profile_end": (c_int, [c_void_p, c_void_p, c_int]),
     "tlce_query_plan": (

@@ -597,3 +597,104 @@ def dflash_kl_backward(
             "tlce_kl_backward",
         )
     return grad_hidden
+
+
+# ----------------------------------------------- cross entropy with exact top-k --
+def dflash_ce_topk_forward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    top_k: int,
+    row_block_size: int,
+    output_multiplier: float,
+    logit_softcap: float,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(loss, probability, top_values, top_ids, lse)`` of a frozen head
+    (reference shim, chunked_linear_ce_native.py:319-343).  ``row_block_size``
+    is accepted for signature parity and ignored."""
+    del row_block_size
+    device = _require_device(hidden, weight, labels)
+    if hidden.dim() != 2 or weight.dim() != 2 or weight.shape[1] != hidden.shape[1]:
+        raise RuntimeError("CE top-k expects hidden [N, D] and weight [V, D]")
+    if weight.dtype != hidden.dtype:
+        raise RuntimeError("native linear CE expects hidden and weight of one dtype")
+    hidden = hidden.contiguous()
+    weight = weight.contiguous()
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v = weight.shape[0]
+    k = int(top_k)
+    code = _dtype_code(hidden)
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        loss = torch.empty(m, dtype=torch.float32, device=device)
+        probability = torch.empty(m, dtype=torch.float32, device=device)
+        lse = torch.empty(m, dtype=torch.float32, device=device)
+        top_values = torch.empty((m, k), dtype=torch.float32, device=device)
+        top_ids = torch.empty((m, k), dtype=torch.long, device=device)
+        if m:
+            ws = _workspace(
+                lib.tlce_ce_topk_forward_workspace_bytes(m, h, v, code, PANEL_BYTES), device
+            )
+            _lib.check(
+                lib.tlce_ce_topk_forward(
+                    _ptr(hidden), _ptr(weight), _ptr(labels), m, h, v, code, k,
+                    float(output_multiplier), float(logit_softcap),
+                    _ptr(loss), _ptr(probability), _ptr(top_values), _ptr(top_ids), _ptr(lse),
+                    PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                ),
+                "tlce_ce_topk_forward",
+            )
+    return loss, probability, top_values, top_ids, lse
+
+
+def dflash_ce_topk_backward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    lse: torch.Tensor,
+    probabilities: torch.Tensor,
+    top_ids: torch.Tensor,
+    grad_loss: torch.Tensor,
+    grad_probability: torch.Tensor,
+    grad_top_values: torch.Tensor | None,
+    *,
+    row_block_size: int,
+    output_multiplier: float,
+    logit_softcap: float,
+) -> torch.Tensor:
+    """Gradient for ``hidden`` given the gradients of loss, probability and
+    top values (reference shim, chunked_linear_ce_native.py:346-380)."""
+    del row_block_size
+    device = _require_device(hidden, weight, labels, lse, probabilities, top_ids, grad_loss,
+                             grad_probability, grad_top_values)
+    hidden = hidden.contiguous()
+    weight = weight.contiguous()
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v = weight.shape[0]
+    k = int(top_ids.shape[1])
+    code = _dtype_code(hidden)
+    # d objective / d loss, with the probability's gradient folded in (p = exp(-loss))
+    ce_scale = (grad_loss.float() - grad_probability.float() * probabilities.float()).contiguous()
+    gtv = None if grad_top_values is None else grad_top_values.to(torch.float32).contiguous()
+    lse = lse.reshape(-1).to(torch.float32).contiguous()
+    top_ids = top_ids.to(torch.long).contiguous()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        grad_hidden = torch.empty((m, h), dtype=hidden.dtype, device=device)
+        if m:
+            ws = _workspace(
+                lib.tlce_ce_topk_backward_workspace_bytes(m, h, v, code, PANEL_BYTES), device
+            )
+            _lib.check(
+                lib.tlce_ce_topk_backward(
+                    _ptr(hidden), _ptr(weight), _ptr(labels), _ptr(lse), _ptr(top_ids),
+                    _ptr(ce_scale), _ptr(gtv), m, h, v, code, k,
+                    float(output_multiplier), float(logit_softcap), _ptr(grad_hidden),
+                    PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                ),
+                "tlce_ce_topk_backward",
+            )
+    return grad_hidden

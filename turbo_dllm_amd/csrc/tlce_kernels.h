@@ -225,6 +225,7 @@ struct ScaleArgs {
   int reduction;
   int64_t ignore;
   float constant;   // labels == null: every real row gets this scale
+  float multiplier; // applied to every scale
   float* scale;
 };
 
@@ -244,7 +245,7 @@ __global__ __launch_bounds__(256) void lce_token_scale_kernel(ScaleArgs p) {
       s = p.grad_output[0] / p.valid_count[0];
     }
   }
-  p.scale[r] = s;
+  p.scale[r] = s * p.multiplier;
 }
 
 // Recompute one logits^T tile of a vocabulary panel and turn it, in registers,
@@ -265,7 +266,11 @@ struct GradLogitsArgs {
   int64_t ignore, exclude;
   float softcap;
   int64_t label_offset;  // global id of weight row 0 (vocabulary shards), else 0
-  int probabilities;     // 1: g = softmax * scale (labels may be null; no onehot, no cap')
+  int probabilities;     // 1: g = softmax * scale (labels may be null; no onehot)
+  int cap_grad;          // 1: g carries the soft cap's derivative 1 - tanh^2 (a gradient
+                         // with respect to the raw logits), 0: it does not (probabilities)
+  float logit_scale;     // logits = cap(logit_scale * hidden . weight^T); needs bias == null
+                         // unless it is 1.  The caller folds it into `scale` for gradients.
   int v0;             // first vocabulary row of the panel
   int n_ttiles, n_ptiles;
   void* g;            // [mp, ldg]
@@ -307,7 +312,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   const int vbase = p.v0 + pv * E::kTile;
   eng.mainloop(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
 
-  const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
+  const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
+  const float log2e_scaled = TLCE_LOG2E * p.logit_scale;
   // per owned token column: row of its label inside this tile (-1: none here),
   // lse in base-2 units, and the loss scale (0 for ignored and padding rows,
   // which zeroes their whole column of g without a per-element test)
@@ -355,15 +361,18 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
       for (int j = 0; j < E::kCols; ++j) {
         float z = E::get(acc, j, i);
         float dcap = 1.0f;
+        float g;
         if (kSoftcap) {
-          const float t = fast_tanh(z * inv_cap);
+          const float t = fast_tanh(z * inv_cap);   // inv_cap includes logit_scale
           z = p.softcap * t;
           dcap = 1.0f - t * t;
+          g = fast_exp2(fmaf(z, TLCE_LOG2E, -lse2[j]));
+        } else {
+          g = fast_exp2(fmaf(z, log2e_scaled, -lse2[j]));
         }
-        float g = fast_exp2(fmaf(z, TLCE_LOG2E, -lse2[j]));
         if (kOnehot && row == label_row[j]) g -= 1.0f;
         g *= scale[j];
-        if (kSoftcap && !p.probabilities) g *= dcap;
+        if (kSoftcap && p.cap_grad) g *= dcap;
         if (kEdge) g = vok ? g : 0.0f;
         E::set(acc, j, i, g);
         row_sum += g;
@@ -657,6 +666,333 @@ __global__ __launch_bounds__(256) void lce_kl_finish_kernel(float* losses, const
                                                             const float* lse, int m) {
   const int r = blockIdx.x * 256 + threadIdx.x;
   if (r < m) losses[r] = losses[r] + tsum[r] * lse[r] + 1.0f;
+}
+
+// ------------------------------------------------- cross entropy + exact top-k --
+// Frozen-head cross entropy that also returns the k largest logits of every row
+// (dflash_ce_topk_forward / _backward, fused_linear_ce_cuda.cu:482-599,1511-1773;
+// torch form in dllm_parallel/core/kernels/dflash_linear_topk.py:100-225).
+// The logits z = cap(multiplier * hidden . weight^T) cross memory once, in
+// float32, in bounded vocabulary panels: lce_logits_panel_kernel writes a
+// panel, lce_topk_scan_kernel folds it into the row's running (max, sum exp)
+// and its running list of the k largest (value, id) pairs.
+struct LogitsPanelArgs {
+  const void* hidden;
+  const void* weight;
+  int m, h, v;
+  float softcap, logit_scale;
+  int v0;               // first vocabulary row of the panel
+  int n_ttiles, n_ptiles;
+  float* panel;         // [mp, ld] float32; columns past the vocabulary get -inf
+  int64_t ld;
+};
+
+template <class E, bool kSoftcap>
+__global__ __launch_bounds__(E::kThreads) void lce_logits_panel_kernel(LogitsPanelArgs p) {
+  extern __shared__ __align__(16) char smem[];
+  using T = typename E::T;
+  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
+  if (logical >= p.n_ttiles * p.n_ptiles) return;
+  int tt, pv;
+  grouped_tile(logical, p.n_ttiles, p.n_ptiles, 4, &tt, &pv);
+  E eng;
+  typename E::Acc acc;
+  E::zero(acc);
+  const int vbase = p.v0 + pv * E::kTile;
+  eng.mainloop(static_cast<const T*>(p.weight), p.h, vbase, p.v, static_cast<const T*>(p.hidden),
+               p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+  const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
+  const int prow = pv * E::kTile;
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    float* out = p.panel + ((int64_t)tt * E::kTile + eng.col(j)) * p.ld + prow;
+#pragma unroll
+    for (int i4 = 0; i4 < E::kRows; i4 += 4) {
+      float z[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const float raw = E::get(acc, j, i4 + u);
+        const float val = kSoftcap ? p.softcap * fast_tanh(raw * inv_cap) : raw * p.logit_scale;
+        z[u] = (vbase + eng.row(i4 + u) < p.v) ? val : -INFINITY;
+      }
+      *reinterpret_cast<float4*>(out + eng.row(i4)) = make_float4(z[0], z[1], z[2], z[3]);
+    }
+  }
+}
+
+// Ordering of (value, id) pairs: larger value first, then smaller id.
+__device__ __forceinline__ bool topk_before(float va, int64_t ia, float vb, int64_t ib) {
+  return va > vb || (va == vb && ia < ib);
+}
+
+// k rounds of "the best pair that comes after the previous pick" over the
+// pairs the workgroup's threads hold (kN per thread, pair i of this thread is
+// (val(i), id(i)); absent pairs are (-inf, INT64_MAX)).  Round r's pick goes to
+// list_val[r] / list_id[r].  No marking and no sorting network: a pick is
+// excluded from later rounds by the ordering alone.
+template <int kN, class Val, class Id>
+__device__ __forceinline__ void topk_select_rounds(int k, Val val, Id id, float* list_val,
+                                                   int64_t* list_id, float* red_val,
+                                                   int64_t* red_id) {
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  float prev_val = INFINITY;
+  int64_t prev_id = INT64_MIN;
+  for (int r = 0; r < k; ++r) {
+    float best_val = -INFINITY;
+    int64_t best_id = INT64_MAX;
+#pragma unroll
+    for (int i = 0; i < kN; ++i) {
+      const float v = val(i);
+      const int64_t d = id(i);
+      if (topk_before(prev_val, prev_id, v, d) && topk_before(v, d, best_val, best_id)) {
+        best_val = v;
+        best_id = d;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best_val, o, 64);
+      const int64_t oi = __shfl_xor(best_id, o, 64);
+      if (topk_before(ov, oi, best_val, best_id)) {
+        best_val = ov;
+        best_id = oi;
+      }
+    }
+    if (lane == 0) {
+      red_val[wave] = best_val;
+      red_id[wave] = best_id;
+    }
+    __syncthreads();
+    best_val = red_val[0];
+    best_id = red_id[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) {
+      if (topk_before(red_val[w], red_id[w], best_val, best_id)) {
+        best_val = red_val[w];
+        best_id = red_id[w];
+      }
+    }
+    if (t == 0) {
+      list_val[r] = best_val;
+      list_id[r] = best_id;
+    }
+    prev_val = best_val;
+    prev_id = best_id;
+    __syncthreads();
+  }
+}
+
+// One workgroup per row: folds `width` float32 logits of the row (vocabulary ids
+// v0 .. v0 + width) into run_max / run_sum (natural-log units) and into the
+// row's sorted list of the k largest pairs, 16384 logits at a time (64 per
+// thread, in registers).  Logits above the list's current k-th value are
+// gathered in LDS and merged with the list; when there are too many of them
+// (always so for a row's first logits) the rounds run over all 64 register
+// values per thread instead.  Ties go to the smaller id.  k <= 256.
+struct TopkScanArgs {
+  const float* panel;
+  int64_t ld;
+  int m;
+  int64_t v0;
+  int width;
+  int k;
+  int first;            // 1: the lists and statistics are empty
+  float* run_max;
+  float* run_sum;
+  float* top_values;    // [m, k]
+  int64_t* top_ids;     // [m, k]
+};
+
+__global__ __launch_bounds__(256) void lce_topk_scan_kernel(TopkScanArgs p) {
+  constexpr int kPerThread = 64;
+  constexpr int kChunk = kPerThread * 256;
+  constexpr int kSlots = 3;                       // gathered pairs per thread
+  constexpr int kCapacity = kSlots * 256;
+  __shared__ float list_val[256];
+  __shared__ int64_t list_id[256];
+  __shared__ float cand_val[kCapacity];
+  __shared__ int64_t cand_id[kCapacity];
+  __shared__ float red_val[4];
+  __shared__ int64_t red_id[4];
+  __shared__ float red_f[4];
+  __shared__ int cand_count;
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int row = blockIdx.x;
+  const float* src = p.panel + (int64_t)row * p.ld;
+  float run_max = p.first ? -INFINITY : p.run_max[row];
+  float run_sum = p.first ? 0.0f : p.run_sum[row];
+  if (t < p.k) {
+    // placeholders get distinct negative ids so that they stay distinguishable
+    list_val[t] = p.first ? -INFINITY : p.top_values[(int64_t)row * p.k + t];
+    list_id[t] = p.first ? (int64_t)(-1 - t) : p.top_ids[(int64_t)row * p.k + t];
+  }
+  if (t == 0) cand_count = 0;
+  __syncthreads();
+
+  for (int c0 = 0; c0 < p.width; c0 += kChunk) {
+    float vals[kPerThread];
+    float local_max = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int idx = c0 + t + 256 * i;
+      vals[i] = idx < p.width ? src[idx] : -INFINITY;
+      local_max = fmaxf(local_max, vals[i]);
+    }
+    // running softmax statistics
+    const float m = wave_max(local_max);
+    if (lane == 0) red_f[wave] = m;
+    __syncthreads();
+    const float new_max =
+        fmaxf(run_max, fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3])));
+    __syncthreads();
+    float local_sum = 0.0f;
+    if (new_max > -INFINITY) {
+#pragma unroll
+      for (int i = 0; i < kPerThread; ++i) local_sum += __expf(vals[i] - new_max);
+    }
+    local_sum = wave_sum(local_sum);
+    if (lane == 0) red_f[wave] = local_sum;
+    __syncthreads();
+    run_sum = (run_max > -INFINITY ? run_sum * __expf(run_max - new_max) : 0.0f) +
+              (red_f[0] + red_f[1] + red_f[2] + red_f[3]);
+    run_max = new_max;
+
+    // the list entry this thread carries into the selection
+    const float own_val = t < p.k ? list_val[t] : -INFINITY;
+    const int64_t own_id = t < p.k ? list_id[t] : INT64_MAX;
+    const float kth = list_val[p.k - 1];
+    auto chunk_id = [&](int i) -> int64_t {
+      return (c0 + t + 256 * i < p.width) ? p.v0 + c0 + t + 256 * i : INT64_MAX;
+    };
+    // gather the logits that beat the current k-th value
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      if (vals[i] > kth && c0 + t + 256 * i < p.width) {
+        const int pos = atomicAdd(&cand_count, 1);
+        if (pos < kCapacity) {
+          cand_val[pos] = vals[i];
+          cand_id[pos] = chunk_id(i);
+        }
+      }
+    }
+    __syncthreads();
+    const int n_cand = cand_count;
+    __syncthreads();
+    if (t == 0) cand_count = 0;
+    if (n_cand > kCapacity) {
+      topk_select_rounds<kPerThread + 1>(
+          p.k, [&](int i) { return i < kPerThread ? vals[i] : own_val; },
+          [&](int i) { return i < kPerThread ? chunk_id(i) : own_id; }, list_val, list_id,
+          red_val, red_id);
+    } else if (n_cand > 0) {
+      float gv[kSlots];
+      int64_t gi[kSlots];
+#pragma unroll
+      for (int q = 0; q < kSlots; ++q) {
+        const int pos = t + 256 * q;
+        gv[q] = pos < n_cand ? cand_val[pos] : -INFINITY;
+        gi[q] = pos < n_cand ? cand_id[pos] : INT64_MAX;
+      }
+      topk_select_rounds<kSlots + 1>(
+          p.k, [&](int i) { return i < kSlots ? gv[i] : own_val; },
+          [&](int i) { return i < kSlots ? gi[i] : own_id; }, list_val, list_id, red_val,
+          red_id);
+    }
+    __syncthreads();
+  }
+  if (t < p.k) {
+    p.top_values[(int64_t)row * p.k + t] = list_val[t];
+    p.top_ids[(int64_t)row * p.k + t] = list_id[t];
+  }
+  if (t == 0) {
+    p.run_max[row] = run_max;
+    p.run_sum[row] = run_sum;
+  }
+}
+
+// One wave per row: lse, the label's logit as a direct dot product, loss and
+// the label's probability exp(-loss).
+struct TopkFinishArgs {
+  const void* hidden;
+  const void* weight;
+  const int64_t* labels;
+  int m, h;
+  float softcap, logit_scale;
+  const float* run_max;
+  const float* run_sum;
+  float* lse;
+  float* losses;
+  float* probabilities;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void lce_topk_finish_kernel(TopkFinishArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= p.m) return;
+  const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
+  const T* wrow = static_cast<const T*>(p.weight) + p.labels[r] * (int64_t)p.h;
+  float dot = 0.0f;
+  for (int k = lane; k < p.h; k += 64) dot = fmaf(to_float<T>(hrow[k]), to_float<T>(wrow[k]), dot);
+  dot = wave_sum(dot) * p.logit_scale;
+  if (p.softcap > 0.0f) dot = p.softcap * tanhf(dot / p.softcap);
+  if (lane == 0) {
+    const float lse = p.run_max[r] + logf(p.run_sum[r]);
+    const float loss = lse - dot;
+    p.lse[r] = lse;
+    p.losses[r] = loss;
+    p.probabilities[r] = expf(-loss);
+  }
+}
+
+// grad_hidden terms that touch single weight rows, added to the float32
+// accumulator before the final cast (dflash_linear_topk.py:196-225):
+//   - ce_scale[r] * d'(label) * W[label]  +  sum_j grad_top_values[r, j] * d'(id_j) * W[id_j]
+// with d'(v) = multiplier * (1 - tanh^2(multiplier * h.W[v] / cap)) (multiplier without cap).
+struct TopkAdjustArgs {
+  const void* hidden;
+  const void* weight;
+  const int64_t* labels;
+  const int64_t* top_ids;          // [m, k]
+  const float* ce_scale;           // [m]
+  const float* grad_top_values;    // [m, k] or null
+  int m, h, k;
+  float softcap, logit_scale;
+  float* acc32;                    // [mp, h]
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void lce_topk_adjust_kernel(TopkAdjustArgs p) {
+  __shared__ float red[4];
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int r = blockIdx.x;
+  const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
+  float* out = p.acc32 + (int64_t)r * p.h;
+  const int n_entries = (p.grad_top_values != nullptr ? p.k : 0) + 1;
+  for (int e = 0; e < n_entries; ++e) {
+    const bool is_label = e == n_entries - 1;
+    const int64_t id = is_label ? p.labels[r] : p.top_ids[(int64_t)r * p.k + e];
+    const float weight_in = is_label ? -p.ce_scale[r] : p.grad_top_values[(int64_t)r * p.k + e];
+    if (weight_in == 0.0f) continue;   // workgroup-uniform
+    const T* wrow = static_cast<const T*>(p.weight) + id * (int64_t)p.h;
+    float dot = 0.0f;
+    for (int c = t; c < p.h; c += 256) dot = fmaf(to_float<T>(hrow[c]), to_float<T>(wrow[c]), dot);
+    dot = wave_sum(dot);
+    if (lane == 0) red[wave] = dot;
+    __syncthreads();
+    const float raw = (red[0] + red[1] + red[2] + red[3]) * p.logit_scale;
+    __syncthreads();
+    float deriv = p.logit_scale;
+    if (p.softcap > 0.0f) {
+      const float th = tanhf(raw / p.softcap);
+      deriv *= 1.0f - th * th;
+    }
+    const float coef = weight_in * deriv;
+    for (int c = t; c < p.h; c += 256) out[c] += coef * to_float<T>(wrow[c]);
+  }
 }
 
 // C[j][i] (op)= sum_k A[i][k] * B[j][k]  - the two gradient contractions, with

@@ -14,6 +14,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <functional>
 #include <vector>
 
 #include "tlce_common.h"
@@ -369,7 +370,8 @@ template <class E, class Producer>
 int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidden,
                        const void* weight, const int64_t* row_idx, int64_t m, int64_t n_out,
                        int64_t h, int64_t v, int dtype, void* grad_hidden, void* grad_weight,
-                       char* ws, hipStream_t stream, Producer&& produce) {
+                       char* ws, hipStream_t stream, Producer&& produce,
+                       const std::function<int(float*)>& before_cast = nullptr) {
   using T = typename E::T;
   const bool weight_grad = grad_weight != nullptr;
   float* acc32 = reinterpret_cast<float*>(ws + l.acc32);
@@ -445,6 +447,9 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     }
   }
 
+  if (before_cast) {
+    if (int rc = before_cast(acc32)) return rc;   // extra float32 terms of grad_hidden
+  }
   if (row_idx != nullptr) {
     if (int rc = fill_zero(grad_hidden, n_out * h * dtype_bytes(dtype), stream)) return rc;
   }
@@ -480,7 +485,7 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
   ScaleArgs sa;
   sa.labels = labels; sa.row_idx = row_idx; sa.grad_output = grad_output;
   sa.valid_count = valid_count; sa.m = (int)m; sa.mp = (int)p.mp; sa.reduction = reduction;
-  sa.ignore = ignore; sa.scale = scale; sa.constant = probabilities_scale;
+  sa.ignore = ignore; sa.scale = scale; sa.constant = probabilities_scale; sa.multiplier = 1.0f;
   if (int rc = launch_token_scale(sa, stream)) return rc;
   if (grad_bias != nullptr) {
     if (int rc = fill_zero(grad_bias, v * 4, stream)) return rc;
@@ -493,6 +498,8 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     ga.ignore = ignore; ga.exclude = exclude - vocab_start; ga.softcap = softcap;
     ga.label_offset = vocab_start;
     ga.probabilities = (labels == nullptr) ? 1 : 0;
+    ga.cap_grad = (labels == nullptr) ? 0 : 1;
+    ga.logit_scale = 1.0f;
     ga.v0 = (int)v0;
     ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
     ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
@@ -556,7 +563,7 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
   ga.labels = nullptr; ga.lse = teacher_lse; ga.scale = ones;
   ga.m = (int)m; ga.h = (int)ht; ga.v = (int)v;
   ga.ignore = 0; ga.exclude = -1; ga.softcap = softcap;
-  ga.label_offset = 0; ga.probabilities = 1;
+  ga.label_offset = 0; ga.probabilities = 1; ga.cap_grad = 0; ga.logit_scale = 1.0f;
   ga.v0 = (int)v0;
   ga.n_ttiles = pd.n_ttiles; ga.n_ptiles = (int)(width / pd.tile);
   ga.g = g; ga.ldg = pd.vc; ga.gt = nullptr; ga.ldgt = 0;
@@ -590,7 +597,7 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
   ScaleArgs sa;
   sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = nullptr; sa.valid_count = nullptr;
   sa.m = (int)m; sa.mp = (int)pd.mp; sa.reduction = TLCE_REDUCTION_SUM; sa.ignore = 0;
-  sa.scale = ones; sa.constant = 1.0f;
+  sa.scale = ones; sa.constant = 1.0f; sa.multiplier = 1.0f;
   if (int rc = launch_token_scale(sa, stream)) return rc;
   if (int rc = fill_zero(tsum, pd.mp * 4, stream)) return rc;
   if (int rc = fill_zero(losses, m * 4, stream)) return rc;
@@ -638,7 +645,7 @@ int kl_backward_impl(const Plan& pd, const KlLayout& l, const void* draft_hidden
   ScaleArgs sa;
   sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = nullptr; sa.valid_count = nullptr;
   sa.m = (int)m; sa.mp = (int)pd.mp; sa.reduction = TLCE_REDUCTION_NONE; sa.ignore = 0;
-  sa.scale = ones; sa.constant = 1.0f;
+  sa.scale = ones; sa.constant = 1.0f; sa.multiplier = 1.0f;
   if (int rc = launch_token_scale(sa, stream)) return rc;
   sa.grad_output = grad_output; sa.scale = scale;   // scale[r] = grad_output[r]
   if (int rc = launch_token_scale(sa, stream)) return rc;
@@ -649,6 +656,144 @@ int kl_backward_impl(const Plan& pd, const KlLayout& l, const void* draft_hidden
   };
   return panel_contractions<E>(pd, bl, draft_hidden, draft_weight, nullptr, m, m, hd, v, dtype,
                                grad_hidden, nullptr, bws, stream, produce);
+}
+
+// ------------------------------------------------ cross entropy + top-k ----
+struct TopkPlan {
+  Plan plan;            // engine, tiles and the backward's panels (input dtype)
+  int64_t vcf;          // columns of a float32 logits panel
+  int n_fpanels;
+  int64_t run_max, run_sum, fpanel, forward_total;
+  int64_t ce_scale, backward, backward_total;
+};
+
+TopkPlan topk_plan(int64_t m, int64_t h, int64_t v, int dtype, int64_t panel_bytes) {
+  TopkPlan t;
+  t.plan = make_plan(m, h, v, dtype, false, panel_bytes);
+  const Plan& p = t.plan;
+  if (panel_bytes <= 0) panel_bytes = kDefaultPanelBytes;
+  int64_t tiles = std::max<int64_t>(1, panel_bytes / (p.mp * 4) / p.tile);
+  tiles = std::min<int64_t>(tiles, p.n_vtiles);
+  if (tiles >= 16 && tiles < p.n_vtiles) tiles = tiles / 16 * 16;
+  t.vcf = tiles * p.tile;
+  t.n_fpanels = (int)ceil_div(p.vp, t.vcf);
+  int64_t off = 0;
+  t.run_max = off;  off += align256(m * 4);
+  t.run_sum = off;  off += align256(m * 4);
+  t.fpanel = off;   off += align256(p.mp * t.vcf * 4);
+  t.forward_total = off;
+  off = 0;
+  t.ce_scale = off; off += align256(p.mp * 4);
+  t.backward = off; off += backward_layout(p, m, h, dtype, false).total;
+  t.backward_total = off;
+  return t;
+}
+
+template <class E, bool kSoftcap>
+int launch_logits_panel_variant(const LogitsPanelArgs& a, hipStream_t stream) {
+  static LdsOptIn lds;
+  if (int rc = enable_large_lds(lce_logits_panel_kernel<E, kSoftcap>, E::kSmemBytes, lds))
+    return rc;
+  const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
+  ScopedTimer timer(kClassGradLogits, stream);
+  lce_logits_panel_kernel<E, kSoftcap><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+template <class E>
+int topk_forward_impl(const TopkPlan& t, const void* hidden, const void* weight,
+                      const int64_t* labels, int64_t m, int64_t h, int64_t v, int top_k,
+                      float multiplier, float softcap, float* losses, float* probabilities,
+                      float* top_values, int64_t* top_ids, float* lse, char* ws,
+                      hipStream_t stream) {
+  using T = typename E::T;
+  const Plan& p = t.plan;
+  float* run_max = reinterpret_cast<float*>(ws + t.run_max);
+  float* run_sum = reinterpret_cast<float*>(ws + t.run_sum);
+  float* panel = reinterpret_cast<float*>(ws + t.fpanel);
+  for (int pi = 0; pi < t.n_fpanels; ++pi) {
+    const int64_t v0 = (int64_t)pi * t.vcf;
+    const int64_t width = std::min<int64_t>(t.vcf, p.vp - v0);
+    const int64_t valid = std::min<int64_t>(t.vcf, v - v0);
+    LogitsPanelArgs la;
+    la.hidden = hidden; la.weight = weight;
+    la.m = (int)m; la.h = (int)h; la.v = (int)v;
+    la.softcap = softcap; la.logit_scale = multiplier;
+    la.v0 = (int)v0; la.n_ttiles = p.n_ttiles; la.n_ptiles = (int)(width / p.tile);
+    la.panel = panel; la.ld = t.vcf;
+    if (softcap > 0.0f) {
+      if (int rc = launch_logits_panel_variant<E, true>(la, stream)) return rc;
+    } else {
+      if (int rc = launch_logits_panel_variant<E, false>(la, stream)) return rc;
+    }
+    TopkScanArgs sa;
+    sa.panel = panel; sa.ld = t.vcf; sa.m = (int)m; sa.v0 = v0; sa.width = (int)valid;
+    sa.k = top_k; sa.first = pi == 0;
+    sa.run_max = run_max; sa.run_sum = run_sum; sa.top_values = top_values; sa.top_ids = top_ids;
+    {
+      ScopedTimer timer(kClassOther, stream);
+      lce_topk_scan_kernel<<<(int)m, 256, 0, stream>>>(sa);
+    }
+    TLCE_LAUNCH_CHECK();
+  }
+  TopkFinishArgs fa;
+  fa.hidden = hidden; fa.weight = weight; fa.labels = labels; fa.m = (int)m; fa.h = (int)h;
+  fa.softcap = softcap; fa.logit_scale = multiplier;
+  fa.run_max = run_max; fa.run_sum = run_sum;
+  fa.lse = lse; fa.losses = losses; fa.probabilities = probabilities;
+  {
+    ScopedTimer timer(kClassCombine, stream);
+    lce_topk_finish_kernel<T><<<(int)ceil_div(m, 4), 256, 0, stream>>>(fa);
+  }
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+template <class E>
+int topk_backward_impl(const TopkPlan& t, const void* hidden, const void* weight,
+                       const int64_t* labels, const float* lse, const int64_t* top_ids,
+                       const float* ce_scale, const float* grad_top_values, int64_t m, int64_t h,
+                       int64_t v, int dtype, int top_k, float multiplier, float softcap,
+                       void* grad_hidden, char* ws, hipStream_t stream) {
+  using T = typename E::T;
+  const Plan& p = t.plan;
+  char* bws = ws + t.backward;
+  const BackwardLayout bl = backward_layout(p, m, h, dtype, false);
+  float* scale = reinterpret_cast<float*>(bws + bl.scale);
+  // scale[r] = ce_scale[r] * multiplier: d loss / d raw logit carries the multiplier
+  ScaleArgs sa;
+  sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = ce_scale; sa.valid_count = nullptr;
+  sa.m = (int)m; sa.mp = (int)p.mp; sa.reduction = TLCE_REDUCTION_NONE; sa.ignore = 0;
+  sa.scale = scale; sa.constant = 0.0f; sa.multiplier = multiplier;
+  if (int rc = launch_token_scale(sa, stream)) return rc;
+  auto produce = [&](int64_t v0, int64_t width, void* g, void* gt) -> int {
+    GradLogitsArgs ga;
+    ga.hidden = hidden; ga.weight = weight; ga.bias = nullptr; ga.labels = nullptr;
+    ga.lse = lse; ga.scale = scale;
+    ga.m = (int)m; ga.h = (int)h; ga.v = (int)v;
+    ga.ignore = 0; ga.exclude = -1; ga.softcap = softcap;
+    ga.label_offset = 0; ga.probabilities = 1; ga.cap_grad = 1; ga.logit_scale = multiplier;
+    ga.v0 = (int)v0;
+    ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
+    ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
+    ga.grad_bias = nullptr;
+    return launch_grad_logits<E>(ga, stream);
+  };
+  auto single_rows = [&](float* acc32) -> int {
+    // with a K split the label / top-k terms go to the first slab only
+    TopkAdjustArgs aa;
+    aa.hidden = hidden; aa.weight = weight; aa.labels = labels; aa.top_ids = top_ids;
+    aa.ce_scale = ce_scale; aa.grad_top_values = grad_top_values;
+    aa.m = (int)m; aa.h = (int)h; aa.k = top_k;
+    aa.softcap = softcap; aa.logit_scale = multiplier; aa.acc32 = acc32;
+    ScopedTimer timer(kClassOther, stream);
+    lce_topk_adjust_kernel<T><<<(int)m, 256, 0, stream>>>(aa);
+    TLCE_LAUNCH_CHECK();
+    return 0;
+  };
+  return panel_contractions<E>(p, bl, hidden, weight, nullptr, m, m, h, v, dtype, grad_hidden,
+                               nullptr, bws, stream, produce, single_rows);
 }
 
 }  // namespace
@@ -1004,6 +1149,82 @@ extern "C" int tlce_kl_backward(const void* draft_hidden, const void* draft_weig
                                     teacher_weight, draft_lse, teacher_lse, grad_output, m,
                                     h_draft, h_teacher, v, dtype, logit_softcap, grad_hidden,
                                     static_cast<char*>(workspace), stream));
+}
+
+// ---------------------------------------------------- cross entropy + top-k --
+namespace {
+
+int topk_validate(const void* hidden, const void* weight, const int64_t* labels, int64_t m,
+                  int64_t h, int64_t v, int dtype, int top_k) {
+  if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  TLCE_REQUIRE(top_k >= 1 && top_k <= 256 && top_k <= v,
+               "ce_topk: top_k=%d must be in [1, min(256, v)]", top_k);
+  TLCE_REQUIRE(labels != nullptr || m == 0, "ce_topk: labels is null");
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int64_t tlce_ce_topk_forward_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                                        int dtype, int64_t panel_bytes) {
+  if (m < 0 || h <= 0 || v <= 0) return -1;
+  return topk_plan(m, h, v, dtype, panel_bytes).forward_total;
+}
+
+extern "C" int64_t tlce_ce_topk_backward_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                                         int dtype, int64_t panel_bytes) {
+  if (m < 0 || h <= 0 || v <= 0) return -1;
+  return topk_plan(m, h, v, dtype, panel_bytes).backward_total;
+}
+
+extern "C" int tlce_ce_topk_forward(const void* hidden, const void* weight, const int64_t* labels,
+                                    int64_t m, int64_t h, int64_t v, int dtype, int top_k,
+                                    float output_multiplier, float logit_softcap, float* losses,
+                                    float* probabilities, float* top_values, int64_t* top_ids,
+                                    float* lse, int64_t panel_bytes, void* workspace,
+                                    int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = topk_validate(hidden, weight, labels, m, h, v, dtype, top_k)) return rc;
+  if (m == 0) return 0;
+  TLCE_REQUIRE(losses && probabilities && top_values && top_ids && lse && workspace,
+               "ce_topk_forward: null pointer");
+  const TopkPlan t = topk_plan(m, h, v, dtype, panel_bytes);
+  TLCE_REQUIRE(workspace_bytes >= t.forward_total,
+               "ce_topk_forward: workspace too small (%lld < %lld)", (long long)workspace_bytes,
+               (long long)t.forward_total);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+               "ce_topk_forward: workspace must be 256-byte aligned");
+  TLCE_DISPATCH(t.plan, dtype,
+                topk_forward_impl<E>(t, hidden, weight, labels, m, h, v, top_k, output_multiplier,
+                                     logit_softcap, losses, probabilities, top_values, top_ids,
+                                     lse, static_cast<char*>(workspace), stream));
+}
+
+extern "C" int tlce_ce_topk_backward(const void* hidden, const void* weight,
+                                     const int64_t* labels, const float* lse,
+                                     const int64_t* top_ids, const float* ce_scale,
+                                     const float* grad_top_values, int64_t m, int64_t h, int64_t v,
+                                     int dtype, int top_k, float output_multiplier,
+                                     float logit_softcap, void* grad_hidden, int64_t panel_bytes,
+                                     void* workspace, int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = topk_validate(hidden, weight, labels, m, h, v, dtype, top_k)) return rc;
+  if (m == 0) return 0;
+  TLCE_REQUIRE(lse && top_ids && ce_scale && grad_hidden && workspace,
+               "ce_topk_backward: null pointer");
+  TLCE_REQUIRE(((uintptr_t)grad_hidden & 15) == 0,
+               "ce_topk_backward: grad_hidden must be 16-byte aligned");
+  const TopkPlan t = topk_plan(m, h, v, dtype, panel_bytes);
+  TLCE_REQUIRE(workspace_bytes >= t.backward_total,
+               "ce_topk_backward: workspace too small (%lld < %lld)", (long long)workspace_bytes,
+               (long long)t.backward_total);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+               "ce_topk_backward: workspace must be 256-byte aligned");
+  TLCE_DISPATCH(t.plan, dtype,
+                topk_backward_impl<E>(t, hidden, weight, labels, lse, top_ids, ce_scale,
+                                      grad_top_values, m, h, v, dtype, top_k, output_multiplier,
+                                      logit_softcap, grad_hidden, static_cast<char*>(workspace),
+                                      stream));
 }
 
 extern "C" int tlce_profile_begin(void) {
