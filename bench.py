@@ -157,6 +157,21 @@ def bench_next_objective(args) -> int:
 
         contractions, name = 6, "frozen-head KL fwd+bwd"   # 3 forward + 3 backward
         shape = f"M={m}, H_draft=H_teacher={h}, V={v}"
+    elif args.objective == "ce_topk":
+        from turbo_dllm_amd.dflash_linear_topk import frozen_linear_ce_topk
+
+        h, v, k = 4096, 151936, 16
+        weight = randn(v, h, 0.02)
+        hidden = randn(m, h, 1.0).requires_grad_(True)
+        labels = torch.randint(0, v, (m,), generator=gen).to(device)
+
+        def step():
+            hidden.grad = None
+            loss, prob, values, _ = frozen_linear_ce_topk(hidden, weight, labels, top_k=k)
+            (loss.sum() + prob.sum() + values.sum()).backward()
+
+        contractions, name = 3, "frozen-head CE + top-16 fwd+bwd"   # 1 forward + 2 backward
+        shape = f"M={m}, H={h}, V={v}, top_k={k}"
     else:
         h, v = 3840, 262144
         weight, hidden = randn(v, h, 0.02), randn(m, h, 1.0)
@@ -196,7 +211,7 @@ def bench_next_objective(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--objective", choices=("ce", "kl", "soft_embedding"), default="ce",
+    ap.add_argument("--objective", choices=("ce", "kl", "soft_embedding", "ce_topk"), default="ce",
                     help="ce: the headline fused linear cross-entropy (default); kl / "
                          "soft_embedding: the objectives built on the same kernels")
     ap.add_argument("--rows", type=int, default=8192, help="rows for --objective kl / soft_embedding")

@@ -192,7 +192,7 @@ int tlce_soft_embedding(const void* hidden, const void* weight, int64_t m,
 
 /* ---- frozen-head forward KL -------------------------------------------------
  * Replaces dflash_frozen_kl_forward / dflash_frozen_kl_backward
- * (fused_linear_ce.cpp:267-330; fused_linear_ce_cuda.cu:367-480,1270-1509):
+ * (fused_linear_ce.cpp:267-304; fused_linear_ce_cuda.cu:367-480,1270-1509):
  *   losses[r] = sum_v p_t (log p_t - log p_d),  p_x = softmax(cap(hidden_x[r] . weight_x^T))
  * for a draft and a teacher head over one vocabulary; only the draft hidden
  * states get a gradient,
@@ -228,7 +228,7 @@ int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
 
 /* ---- frozen-head cross entropy with exact top-k ---------------------------
  * Replaces dflash_ce_topk_forward / dflash_ce_topk_backward
- * (fused_linear_ce.cpp:332-354; fused_linear_ce_cuda.cu:482-599,1511-1773;
+ * (fused_linear_ce.cpp:306-354; fused_linear_ce_cuda.cu:482-599,1511-1773;
  * torch form in dllm_parallel/core/kernels/dflash_linear_topk.py:100-225):
  *   z = cap(output_multiplier * hidden . weight^T),  losses = lse(z) - z[label],
  *   probabilities = exp(-losses), top_values / top_ids = the top_k largest z of

@@ -53,6 +53,8 @@ GPU_CASES = [
     ("bf16_direct_softcap_mult", torch.bfloat16, 129, 128, 1536, 16, 5.0, 0.6, 0.3, 0),
     ("f16_three_panels_k1", torch.float16, 520, 64, 1024, 1, None, 1.0, 0.3, 768 * 512 * 4),
     ("bf16_wide_chunks_k33", torch.bfloat16, 40, 64, 40000, 33, None, 2.0, 0.2, 0),
+    # k = 256: far more logits reach the first threshold than the gather holds -> selection rounds
+    ("bf16_k256_rounds", torch.bfloat16, 33, 64, 20000, 256, None, 1.0, 0.3, 0),
 ]
 
 
@@ -121,3 +123,20 @@ def test_only_loss_gradient_matches_cross_entropy_backward(gpu_device):
     torch.testing.assert_close(loss.sum(), ref, rtol=1e-4, atol=1e-2)
     denom = float(b.grad.float().abs().max())
     assert float((a.grad.float() - b.grad.float()).abs().max()) <= 1e-2 * denom
+
+
+@pytest.mark.gpu
+def test_ties_go_to_the_smaller_id(gpu_device):
+    """All logits equal (zero hidden states): the top-k are ids 0 .. k-1, in
+    every path of the scan (gather overflow on the first logits, rank merge
+    with nothing to add afterwards)."""
+    n, h, v, k = 5, 64, 40000, 7
+    hidden = torch.zeros(n, h, dtype=torch.bfloat16, device=gpu_device)
+    weight = torch.randn(v, h, generator=torch.Generator().manual_seed(1)).bfloat16().to(gpu_device)
+    labels = torch.arange(n, device=gpu_device)
+    loss, prob, vals, ids = frozen_linear_ce_topk(hidden, weight, labels, top_k=k)
+    torch.cuda.synchronize()
+    assert ids.tolist() == [list(range(k))] * n
+    assert torch.count_nonzero(vals) == 0
+    torch.testing.assert_close(loss.cpu(), torch.full((n,), float(torch.log(torch.tensor(float(v))))),
+                               rtol=1e-5, atol=1e-5)

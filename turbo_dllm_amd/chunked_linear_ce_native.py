@@ -420,7 +420,7 @@ def vocab_parallel_backward_local(
     logit_softcap: float,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """One vocabulary shard's exact gradient contributions
-    (reference shim, chunked_linear_ce_native.py:219-256): ``grad_hidden`` is
+    (reference shim, chunked_linear_ce_native.py:218-256): ``grad_hidden`` is
     this shard's partial sum, ``grad_weight`` / ``grad_bias`` cover the shard."""
     device = _require_device(hidden, weight, bias, labels, global_lse, valid_count, grad_output)
     hidden = hidden.contiguous()
@@ -533,7 +533,7 @@ def dflash_kl_forward(
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """``(losses, draft_lse, teacher_lse)``, float32 [N]: per-token forward KL
     of the teacher head against the draft head without a logits buffer
-    (reference shim, chunked_linear_ce_native.py:259-283)."""
+    (reference shim, chunked_linear_ce_native.py:259-274)."""
     device, dh, dw, th, tw = _kl_operands(draft_hidden, draft_weight, teacher_hidden,
                                           teacher_weight)
     m, hd = dh.shape
@@ -569,7 +569,7 @@ def dflash_kl_backward(
     logit_softcap: float,
 ) -> torch.Tensor:
     """Gradient of the per-token KL with respect to the draft hidden states
-    (reference shim, chunked_linear_ce_native.py:286-316)."""
+    (reference shim, chunked_linear_ce_native.py:277-296)."""
     device, dh, dw, th, tw = _kl_operands(draft_hidden, draft_weight, teacher_hidden,
                                           teacher_weight)
     _require_device(draft_lse, teacher_lse, grad_output)
@@ -611,7 +611,7 @@ def dflash_ce_topk_forward(
     logit_softcap: float,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """``(loss, probability, top_values, top_ids, lse)`` of a frozen head
-    (reference shim, chunked_linear_ce_native.py:319-343).  ``row_block_size``
+    (reference shim, chunked_linear_ce_native.py:299-319).  ``row_block_size``
     is accepted for signature parity and ignored."""
     del row_block_size
     device = _require_device(hidden, weight, labels)
@@ -665,7 +665,7 @@ def dflash_ce_topk_backward(
     logit_softcap: float,
 ) -> torch.Tensor:
     """Gradient for ``hidden`` given the gradients of loss, probability and
-    top values (reference shim, chunked_linear_ce_native.py:346-380)."""
+    top values (reference shim, chunked_linear_ce_native.py:322-350)."""
     del row_block_size
     device = _require_device(hidden, weight, labels, lse, probabilities, top_ids, grad_loss,
                              grad_probability, grad_top_values)

@@ -725,71 +725,45 @@ __device__ __forceinline__ bool topk_before(float va, int64_t ia, float vb, int6
   return va > vb || (va == vb && ia < ib);
 }
 
-// k rounds of "the best pair that comes after the previous pick" over the
-// pairs the workgroup's threads hold (kN per thread, pair i of this thread is
-// (val(i), id(i)); absent pairs are (-inf, INT64_MAX)).  Round r's pick goes to
-// list_val[r] / list_id[r].  No marking and no sorting network: a pick is
-// excluded from later rounds by the ordering alone.
-template <int kN, class Val, class Id>
-__device__ __forceinline__ void topk_select_rounds(int k, Val val, Id id, float* list_val,
-                                                   int64_t* list_id, float* red_val,
-                                                   int64_t* red_id) {
-  const int t = threadIdx.x;
-  const int lane = t & 63, wave = t >> 6;
-  float prev_val = INFINITY;
-  int64_t prev_id = INT64_MIN;
-  for (int r = 0; r < k; ++r) {
-    float best_val = -INFINITY;
-    int64_t best_id = INT64_MAX;
+// The best (value, id) pair over the workgroup's 256 threads, returned to all
+// of them; ends on a barrier-free read of red_*, so callers synchronise before
+// the next call.
+__device__ __forceinline__ void topk_workgroup_best(float& best_val, int64_t& best_id,
+                                                    float* red_val, int64_t* red_id) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-    for (int i = 0; i < kN; ++i) {
-      const float v = val(i);
-      const int64_t d = id(i);
-      if (topk_before(prev_val, prev_id, v, d) && topk_before(v, d, best_val, best_id)) {
-        best_val = v;
-        best_id = d;
-      }
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(best_val, o, 64);
+    const int64_t oi = __shfl_xor(best_id, o, 64);
+    if (topk_before(ov, oi, best_val, best_id)) {
+      best_val = ov;
+      best_id = oi;
     }
+  }
+  if (lane == 0) {
+    red_val[wave] = best_val;
+    red_id[wave] = best_id;
+  }
+  __syncthreads();
+  best_val = red_val[0];
+  best_id = red_id[0];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(best_val, o, 64);
-      const int64_t oi = __shfl_xor(best_id, o, 64);
-      if (topk_before(ov, oi, best_val, best_id)) {
-        best_val = ov;
-        best_id = oi;
-      }
+  for (int w = 1; w < 4; ++w) {
+    if (topk_before(red_val[w], red_id[w], best_val, best_id)) {
+      best_val = red_val[w];
+      best_id = red_id[w];
     }
-    if (lane == 0) {
-      red_val[wave] = best_val;
-      red_id[wave] = best_id;
-    }
-    __syncthreads();
-    best_val = red_val[0];
-    best_id = red_id[0];
-#pragma unroll
-    for (int w = 1; w < 4; ++w) {
-      if (topk_before(red_val[w], red_id[w], best_val, best_id)) {
-        best_val = red_val[w];
-        best_id = red_id[w];
-      }
-    }
-    if (t == 0) {
-      list_val[r] = best_val;
-      list_id[r] = best_id;
-    }
-    prev_val = best_val;
-    prev_id = best_id;
-    __syncthreads();
   }
 }
 
 // One workgroup per row: folds `width` float32 logits of the row (vocabulary ids
 // v0 .. v0 + width) into run_max / run_sum (natural-log units) and into the
 // row's sorted list of the k largest pairs, 16384 logits at a time (64 per
-// thread, in registers).  Logits above the list's current k-th value are
-// gathered in LDS and merged with the list; when there are too many of them
-// (always so for a row's first logits) the rounds run over all 64 register
-// values per thread instead.  Ties go to the smaller id.  k <= 256.
+// thread, in registers).  Logits above the list's current k-th value (for a
+// row's first logits: at least the k-th largest per-thread maximum) are
+// gathered in LDS and merged with the list by rank; when there are too many
+// of them, k rounds of "the best pair after the previous pick" run over the
+// whole chunk instead.  Ties go to the smaller id.  k <= 256.
 struct TopkScanArgs {
   const float* panel;
   int64_t ld;
@@ -816,7 +790,8 @@ __global__ __launch_bounds__(256) void lce_topk_scan_kernel(TopkScanArgs p) {
   __shared__ float red_val[4];
   __shared__ int64_t red_id[4];
   __shared__ float red_f[4];
-  __shared__ int cand_count;
+  __shared__ int wave_total[4];
+  __shared__ float tmax[256];
   const int t = threadIdx.x;
   const int lane = t & 63, wave = t >> 6;
   const int row = blockIdx.x;
@@ -828,7 +803,6 @@ __global__ __launch_bounds__(256) void lce_topk_scan_kernel(TopkScanArgs p) {
     list_val[t] = p.first ? -INFINITY : p.top_values[(int64_t)row * p.k + t];
     list_id[t] = p.first ? (int64_t)(-1 - t) : p.top_ids[(int64_t)row * p.k + t];
   }
-  if (t == 0) cand_count = 0;
   __syncthreads();
 
   for (int c0 = 0; c0 < p.width; c0 += kChunk) {
@@ -862,43 +836,126 @@ __global__ __launch_bounds__(256) void lce_topk_scan_kernel(TopkScanArgs p) {
     // the list entry this thread carries into the selection
     const float own_val = t < p.k ? list_val[t] : -INFINITY;
     const int64_t own_id = t < p.k ? list_id[t] : INT64_MAX;
-    const float kth = list_val[p.k - 1];
+    float kth = list_val[p.k - 1];
+    bool inclusive = false;
+    if (kth == -INFINITY && p.k <= 256) {
+      // nothing to compare with yet (a row's first logits): the k-th largest
+      // of the 256 per-thread maxima is a value at least k logits reach
+      __syncthreads();
+      tmax[t] = local_max;
+      __syncthreads();
+      int before = 0;
+      for (int j = 0; j < 256; ++j) {
+        const float other = tmax[j];
+        before += (other > local_max || (other == local_max && j < t)) ? 1 : 0;
+      }
+      if (before == p.k - 1) red_f[0] = local_max;
+      __syncthreads();
+      kth = red_f[0];
+      inclusive = true;
+      __syncthreads();
+    }
+    auto beats = [&](float v) { return inclusive ? v >= kth : v > kth; };
     auto chunk_id = [&](int i) -> int64_t {
       return (c0 + t + 256 * i < p.width) ? p.v0 + c0 + t + 256 * i : INT64_MAX;
     };
-    // gather the logits that beat the current k-th value
+    // gather the logits that beat the current k-th value: count per thread,
+    // exclusive prefix over the workgroup (no atomics), then write
+    int mine = 0;
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      if (vals[i] > kth && c0 + t + 256 * i < p.width) {
-        const int pos = atomicAdd(&cand_count, 1);
-        if (pos < kCapacity) {
-          cand_val[pos] = vals[i];
-          cand_id[pos] = chunk_id(i);
+    for (int i = 0; i < kPerThread; ++i)
+      mine += (beats(vals[i]) && c0 + t + 256 * i < p.width) ? 1 : 0;
+    int scan = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(scan, o, 64);
+      if (lane >= o) scan += up;
+    }
+    if (lane == 63) wave_total[wave] = scan;
+    __syncthreads();
+    int offset = scan - mine;
+    for (int w = 0; w < wave; ++w) offset += wave_total[w];
+    const int n_cand = wave_total[0] + wave_total[1] + wave_total[2] + wave_total[3];
+    if (n_cand <= kCapacity && mine > 0) {
+#pragma unroll
+      for (int i = 0; i < kPerThread; ++i) {
+        if (beats(vals[i]) && c0 + t + 256 * i < p.width) {
+          cand_val[offset] = vals[i];
+          cand_id[offset] = chunk_id(i);
+          ++offset;
         }
       }
     }
     __syncthreads();
-    const int n_cand = cand_count;
-    __syncthreads();
-    if (t == 0) cand_count = 0;
     if (n_cand > kCapacity) {
-      topk_select_rounds<kPerThread + 1>(
-          p.k, [&](int i) { return i < kPerThread ? vals[i] : own_val; },
-          [&](int i) { return i < kPerThread ? chunk_id(i) : own_id; }, list_val, list_id,
-          red_val, red_id);
+      // too many to gather (rare): selection rounds over the whole chunk, eight
+      // logits per thread at a time, read again from memory
+      float prev_val = INFINITY;
+      int64_t prev_id = INT64_MIN;
+      for (int r = 0; r < p.k; ++r) {
+        float best_val = -INFINITY;
+        int64_t best_id = INT64_MAX;
+        if (t < p.k && topk_before(prev_val, prev_id, own_val, own_id)) {
+          best_val = own_val;
+          best_id = own_id;
+        }
+        for (int i = 0; i < kPerThread; ++i) {
+          const int idx = c0 + t + 256 * i;
+          if (idx >= p.width) break;
+          const float v = src[idx];
+          const int64_t d = p.v0 + idx;
+          if (topk_before(prev_val, prev_id, v, d) && topk_before(v, d, best_val, best_id)) {
+            best_val = v;
+            best_id = d;
+          }
+        }
+        topk_workgroup_best(best_val, best_id, red_val, red_id);
+        if (t == 0) {
+          list_val[r] = best_val;
+          list_id[r] = best_id;
+        }
+        prev_val = best_val;
+        prev_id = best_id;
+        __syncthreads();
+      }
     } else if (n_cand > 0) {
+      // merge by rank: the place of a pair in the new list is the number of
+      // pairs, old and gathered, that come before it (ids are unique)
+      int own_rank = t;
+      if (t < p.k) {
+        for (int c = 0; c < n_cand; ++c)
+          own_rank += topk_before(cand_val[c], cand_id[c], own_val, own_id) ? 1 : 0;
+      }
+      int rank[kSlots];
       float gv[kSlots];
       int64_t gi[kSlots];
 #pragma unroll
       for (int q = 0; q < kSlots; ++q) {
         const int pos = t + 256 * q;
-        gv[q] = pos < n_cand ? cand_val[pos] : -INFINITY;
-        gi[q] = pos < n_cand ? cand_id[pos] : INT64_MAX;
+        rank[q] = p.k;
+        if (pos < n_cand) {
+          gv[q] = cand_val[pos];
+          gi[q] = cand_id[pos];
+          int before = 0;
+          for (int j = 0; j < p.k; ++j)
+            before += topk_before(list_val[j], list_id[j], gv[q], gi[q]) ? 1 : 0;
+          for (int c = 0; c < n_cand; ++c)
+            before += topk_before(cand_val[c], cand_id[c], gv[q], gi[q]) ? 1 : 0;
+          rank[q] = before;
+        }
       }
-      topk_select_rounds<kSlots + 1>(
-          p.k, [&](int i) { return i < kSlots ? gv[i] : own_val; },
-          [&](int i) { return i < kSlots ? gi[i] : own_id; }, list_val, list_id, red_val,
-          red_id);
+      __syncthreads();
+      if (t < p.k && own_rank < p.k) {
+        list_val[own_rank] = own_val;
+        list_id[own_rank] = own_id;
+      }
+#pragma unroll
+      for (int q = 0; q < kSlots; ++q) {
+        if (rank[q] < p.k) {
+          list_val[rank[q]] = gv[q];
+          list_id[rank[q]] = gi[q];
+        }
+      }
     }
     __syncthreads();
   }
