@@ -15,11 +15,14 @@ __all__ = [
     "VocabParallelLinear",
     "chunked_linear_ce_native",
     "compact_valid_loss_rows",
+    "frozen_linear_ce_topk",
+    "frozen_linear_kl",
     "masked_token_loss",
     "tiled_linear_cross_entropy",
 ]
 
-_SUBMODULES = {"chunked_linear_ce_native", "compaction", "layers", "loss", "build"}
+_SUBMODULES = {"chunked_linear_ce_native", "compaction", "layers", "loss", "build",
+               "dflash_kl", "dflash_linear_topk", "streaming_soft_embedding"}
 
 
 def tiled_linear_cross_entropy(*args: Any, **kwargs: Any) -> Any:
@@ -36,6 +39,18 @@ def compact_valid_loss_rows(*args: Any, **kwargs: Any) -> Any:
 
 def masked_token_loss(*args: Any, **kwargs: Any) -> Any:
     from .loss import masked_token_loss as impl
+
+    return impl(*args, **kwargs)
+
+
+def frozen_linear_ce_topk(*args: Any, **kwargs: Any) -> Any:
+    from .dflash_linear_topk import frozen_linear_ce_topk as impl
+
+    return impl(*args, **kwargs)
+
+
+def frozen_linear_kl(*args: Any, **kwargs: Any) -> Any:
+    from .dflash_kl import frozen_linear_kl as impl
 
     return impl(*args, **kwargs)
 
