@@ -127,6 +127,28 @@ def measured_traffic(workload, kernel):
     return MEASURED_TRAFFIC_BYTES.get(workload, {}).get(kernel)
 
 
+def library_gemm_reference(torch, device, h, v, rows=8192, reps=5):
+    """What the vendor GEMM reaches on one contraction of this shape class
+    (bf16 [rows, h] x [v, h]^T, float32 accumulation) on this box: the
+    practical ceiling for a plain GEMM, reported next to the fused kernels."""
+    a = torch.randn(rows, h, device=device, dtype=torch.bfloat16)
+    b = torch.randn(v, h, device=device, dtype=torch.bfloat16) * 0.02
+    out = torch.empty(rows, v, device=device, dtype=torch.bfloat16)
+    for _ in range(2):
+        torch.matmul(a, b.t(), out=out)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        torch.matmul(a, b.t(), out=out)
+    stop.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(stop) / reps
+    tflops = 2.0 * rows * h * v / 1e12 / (ms / 1e3)
+    return {"shape": f"[{rows},{h}] x [{v},{h}]^T bf16", "ms": ms, "TFLOP_per_s": tflops,
+            "frac_of_bf16_peak": tflops / PEAK_BF16_TFLOPS}
+
+
 def bench_next_objective(args) -> int:
     """The objectives built on the same kernels: frozen-head forward KL
     (forward + backward) and the streaming soft embedding (forward only)."""
@@ -225,6 +247,8 @@ def main() -> int:
                     help="also run one plain row copy of the weight matrix (known HBM bytes) "
                          "so rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-library-gemm", action="store_true",
+                    help="skip timing torch.matmul (hipBLASLt) on one contraction of this shape")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path "
@@ -366,6 +390,8 @@ def main() -> int:
         },
     }
     result["compaction_gather"] = compaction
+    if not args.no_library_gemm:
+        result["library_gemm"] = library_gemm_reference(torch, device, h, v)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl, args.cpu_rows)
     print(json.dumps(result), flush=True)
