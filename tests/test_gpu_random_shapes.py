@@ -1,0 +1,118 @@
+"""Seeded sweep over small random shapes and option combinations, every
+objective against its float64 oracle: row counts around the 64 / 256 tile
+edges, hidden sizes for all three engines (multiples of 64, of 8, neither),
+vocabularies around the tile and panel edges, bias / soft cap / excluded
+column / reductions / frozen head at random."""
+
+import random
+
+import pytest
+import torch
+
+import linear_ce_oracle as oracle
+from turbo_dllm_amd.dflash_kl import frozen_linear_kl
+from turbo_dllm_amd.dflash_linear_topk import frozen_linear_ce_topk
+from turbo_dllm_amd.streaming_soft_embedding import streaming_soft_embedding
+from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+
+pytestmark = pytest.mark.gpu
+
+ROWS = [1, 2, 7, 63, 64, 65, 130, 255, 256, 257, 400, 700]
+WIDTHS = [8, 24, 64, 72, 128, 200, 256, 320, 33]
+VOCABS = [3, 17, 63, 64, 65, 255, 256, 257, 640, 1000, 1025, 2048, 3000]
+
+
+def draw(case):
+    rnd = random.Random(1000 + case)
+    return dict(
+        n=rnd.choice(ROWS), h=rnd.choice(WIDTHS), v=rnd.choice(VOCABS),
+        dtype=rnd.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32]),
+        bias=rnd.random() < 0.3, softcap=rnd.choice([None, None, 2.0, 30.0]),
+        exclude=rnd.random() < 0.3, reduction=rnd.choice(["none", "sum", "mean"]),
+        frozen=rnd.random() < 0.3, h_teacher=rnd.choice([8, 64, 72, 128]),
+        k=rnd.choice([1, 3, 8]),
+    )
+
+
+@pytest.mark.parametrize("case", range(48))
+def test_random_case(gpu_device, case):
+    c = draw(case)
+    print("[case]", case, c, flush=True)
+    dev = gpu_device
+    n, h, v, dtype, softcap = c["n"], c["h"], c["v"], c["dtype"], c["softcap"]
+    gen = torch.Generator().manual_seed(case)
+    hidden = torch.randn(n, h, generator=gen).to(dtype)
+    weight = (torch.randn(v, h, generator=gen) * (2.0 / h ** 0.5)).to(dtype)
+    bias = torch.randn(v, generator=gen).to(dtype) if c["bias"] else None
+    exclude = int(torch.randint(0, v, (1,), generator=gen)) if c["exclude"] else None
+    labels = torch.randint(0, v, (n,), generator=gen)
+    if exclude is not None:
+        labels[labels == exclude] = (exclude + 1) % v
+    labels[torch.rand(n, generator=gen) < 0.3] = -100
+    if int((labels != -100).sum()) == 0:
+        labels[0] = 0 if exclude != 0 else 1 % v
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    ltol = 1e-5 if dtype == torch.float32 else 1e-3
+
+    # cross entropy, forward and backward
+    x = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(not c["frozen"])
+    b = None if bias is None else bias.to(dev).requires_grad_(True)
+    loss = tiled_linear_cross_entropy(x, w, labels.to(dev), bias=b, reduction=c["reduction"],
+                                      exclude_index=exclude, logit_softcap=softcap, dtype=dtype,
+                                      weight_layout="vocab_first")
+    go = torch.randn(n, generator=gen) if c["reduction"] == "none" else torch.tensor(1.3)
+    loss.backward(go.to(dev))
+    torch.cuda.synchronize()
+    kw = dict(bias=bias, reduction=c["reduction"], exclude_index=exclude, logit_softcap=softcap)
+    ref = oracle.dense_linear_ce(hidden, weight, labels, **kw)
+    rdh, rdw, rdb = oracle.dense_linear_ce_grads(hidden, weight, labels, go, **kw)
+    torch.testing.assert_close(loss.detach().cpu().double(), ref.double(), rtol=ltol, atol=ltol)
+    assert oracle.relative_max_error(x.grad.cpu(), rdh) <= tol
+    if not c["frozen"]:
+        assert oracle.relative_max_error(w.grad.cpu(), rdw) <= tol
+    if bias is not None:
+        assert oracle.relative_max_error(b.grad.cpu(), rdb) <= tol
+
+    # soft embedding
+    soft = streaming_soft_embedding(hidden.to(dev), weight.to(dev), row_chunk_size=64,
+                                    vocab_chunk_size=64, logit_softcap=softcap)
+    expect = oracle.dense_soft_embedding(hidden, weight, logit_softcap=softcap)
+    assert oracle.relative_max_error(soft.cpu(), expect) <= tol
+
+    # forward KL against a teacher head of another width
+    ht = c["h_teacher"]
+    teacher_h = torch.randn(n, ht, generator=gen).to(dtype)
+    teacher_w = (torch.randn(v, ht, generator=gen) * (2.0 / ht ** 0.5)).to(dtype)
+    scale = torch.randn(n, generator=gen)
+    xk = hidden.to(dev).requires_grad_(True)
+    kl = frozen_linear_kl(xk, weight.to(dev), teacher_h.to(dev), teacher_w.to(dev),
+                          logit_softcap=softcap)
+    (kl * scale.to(dev)).sum().backward()
+    torch.cuda.synchronize()
+    torch.testing.assert_close(
+        kl.detach().cpu().double(),
+        oracle.dense_frozen_kl(hidden, weight, teacher_h, teacher_w, logit_softcap=softcap),
+        rtol=10 * ltol, atol=10 * ltol)
+    kl_grad = oracle.dense_frozen_kl_grad(hidden, weight, teacher_h, teacher_w, scale,
+                                          logit_softcap=softcap)
+    assert oracle.relative_max_error(xk.grad.cpu(), kl_grad) <= 2 * tol
+
+    # cross entropy with top-k (16-bit inputs run in the library)
+    if dtype != torch.float32:
+        k = min(v, c["k"])
+        targets = torch.randint(0, v, (n,), generator=gen)
+        xt = hidden.to(dev).requires_grad_(True)
+        l2, p2, values, ids = frozen_linear_ce_topk(xt, weight.to(dev), targets.to(dev), top_k=k,
+                                                    output_multiplier=0.8, logit_softcap=softcap)
+        gl, gp, gv = (torch.randn(n, generator=gen), torch.randn(n, generator=gen),
+                      torch.randn(n, k, generator=gen))
+        ((gl.to(dev) * l2).sum() + (gp.to(dev) * p2).sum() + (gv.to(dev) * values).sum()).backward()
+        torch.cuda.synchronize()
+        rl, _, rv, _, _ = oracle.dense_ce_topk(hidden, weight, targets, k, output_multiplier=0.8,
+                                               logit_softcap=softcap)
+        torch.testing.assert_close(l2.detach().cpu().double(), rl, rtol=1e-3, atol=1e-3)
+        torch.testing.assert_close(values.detach().cpu().double(), rv, rtol=1e-3, atol=1e-3)
+        rg = oracle.dense_ce_topk_grad(hidden, weight, targets, ids.cpu(), gl, gp, gv,
+                                       output_multiplier=0.8, logit_softcap=softcap)
+        assert oracle.relative_max_error(xt.grad.cpu(), rg) <= tol
