@@ -260,8 +260,8 @@ struct MfmaEngine : MfmaTileLayout<T_> {
 //           current one; slice 0 of the next tile is read in the two groups
 //           after the barrier, which sits in the middle of slice 3;
 //   loads : of the next tile's 16, six go out right after the barrier of the
-//           previous step, ten in groups 0..9 - the last one 16 MFMAs before
-//           the barrier that waits for it.
+//           previous step, ten in the first groups of the step (two per group
+//           in groups 0..4, or one per group in groups 0..9).
 template <typename T>
 struct Operand {
   const T* ptr;   // matrix base
@@ -427,6 +427,7 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
     };
 
     const int nk = (k_end - k_begin) / kBK;
+    constexpr bool kLoadsInPairs = !(kAKMajor && !kBKMajor);
     auto step = [&](int k, Frags& fa, Frags& fb, auto has_next_tag) {
       constexpr bool kHasNext = decltype(has_next_tag)::value;
       const int cur = k & 1;
@@ -452,7 +453,16 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
           if (sl < 3) {
             if (t == 0) read_one(fnext, cur, sl + 1, 2 * q);
             if (t == 2) read_one(fnext, cur, sl + 1, 2 * q + 1);
-            if (kHasNext && t == 1 && g < 10) issue_one(nxt, 0, 6 + g);
+            if (kHasNext) {
+              // loads 6..15 of the next tile: two per group in groups 0..4 (measured
+              // about 1 % faster), except for the K-major x K-contiguous pairing,
+              // which does better with one per group in groups 0..9
+              if (kLoadsInPairs) {
+                if ((t == 1 || t == 3) && g < 5) issue_one(nxt, 0, 6 + 2 * g + (t == 3));
+              } else {
+                if (t == 1 && g < 10) issue_one(nxt, 0, 6 + g);
+              }
+            }
           } else if (after_barrier) {
             if (q == 2) {
               if (t == 0) { read_one(fnext, nxt, 0, 0); read_one(fnext, nxt, 0, 1); }
