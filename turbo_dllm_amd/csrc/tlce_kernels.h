@@ -295,6 +295,18 @@ __device__ __forceinline__ void store4(T* dst, float a, float b, float c, float 
   }
 }
 
+// Streaming store for the logit-gradient panels, which are far larger than L2
+// and are read back only by later kernels: the non-temporal hint keeps them
+// from evicting the operand tiles the workgroups of an XCD share through L2
+// (3 % off the producing kernel; the same hint on the GEMM outputs and on the
+// float32 grad_hidden slabs measured slower and is not used there).
+__device__ __forceinline__ void stream_store16(void* dst, uint4 v) {
+  typedef unsigned u4_t __attribute__((ext_vector_type(4)));
+  u4_t x;
+  x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+  __builtin_nontemporal_store(x, reinterpret_cast<u4_t*>(dst));
+}
+
 template <class E, bool kSoftcap, bool kBias>
 __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(GradLogitsArgs p) {
   extern __shared__ __align__(16) char smem[];
@@ -419,8 +431,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
       const int ch = c & 31;
       const uint4 val =
           *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16));
-      *reinterpret_cast<uint4*>(g_out + ((int64_t)tt * E::kTile + tok) * p.ldg + prow + ch * 8) =
-          val;
+      stream_store16(g_out + ((int64_t)tt * E::kTile + tok) * p.ldg + prow + ch * 8, val);
     }
   } else {
 #pragma unroll
@@ -602,8 +613,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
         const int c = it * E::kThreads + threadIdx.x;
         const int tok = c >> 5;
         const int ch = c & 31;
-        *reinterpret_cast<uint4*>(panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 8) =
-            *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16));
+        stream_store16(panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 8,
+                       *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)));
       }
     }
   } else {
