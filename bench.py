@@ -127,26 +127,46 @@ def measured_traffic(workload, kernel):
     return MEASURED_TRAFFIC_BYTES.get(workload, {}).get(kernel)
 
 
-def library_gemm_reference(torch, device, h, v, rows=8192, reps=5):
-    """What the vendor GEMM reaches on one contraction of this shape class
-    (bf16 [rows, h] x [v, h]^T, float32 accumulation) on this box: the
+def library_gemm_reference(torch, device, h, v, rows=8192, panel=16384, reps=5):
+    """What the vendor GEMM (torch.matmul -> hipBLASLt) reaches on this box for
+    the three operand layouts of the path, bf16 with float32 accumulation: the
+    logits contraction [rows,h] x [v,h]^T, and one vocabulary panel of the two
+    gradient contractions, G [rows,panel] x W [panel,h] and G^T x hidden.  The
     practical ceiling for a plain GEMM, reported next to the fused kernels."""
-    a = torch.randn(rows, h, device=device, dtype=torch.bfloat16)
-    b = torch.randn(v, h, device=device, dtype=torch.bfloat16) * 0.02
-    out = torch.empty(rows, v, device=device, dtype=torch.bfloat16)
-    for _ in range(2):
-        torch.matmul(a, b.t(), out=out)
-    torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(reps):
-        torch.matmul(a, b.t(), out=out)
-    stop.record()
-    torch.cuda.synchronize()
-    ms = start.elapsed_time(stop) / reps
-    tflops = 2.0 * rows * h * v / 1e12 / (ms / 1e3)
-    return {"shape": f"[{rows},{h}] x [{v},{h}]^T bf16", "ms": ms, "TFLOP_per_s": tflops,
-            "frac_of_bf16_peak": tflops / PEAK_BF16_TFLOPS}
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / reps
+
+    def entry(shape, ms, flops):
+        tflops = flops / 1e12 / (ms / 1e3)
+        return {"shape": shape, "ms": ms, "TFLOP_per_s": tflops,
+                "frac_of_bf16_peak": tflops / PEAK_BF16_TFLOPS}
+
+    bf16 = dict(device=device, dtype=torch.bfloat16)
+    hidden = torch.randn(rows, h, **bf16)
+    weight = torch.randn(v, h, **bf16) * 0.02
+    out = torch.empty(rows, v, **bf16)
+    result = entry(f"[{rows},{h}] x [{v},{h}]^T bf16",
+                   timed(lambda: torch.matmul(hidden, weight.t(), out=out)), 2.0 * rows * h * v)
+    del out
+    m = 4 * rows
+    g = torch.randn(m, panel, **bf16) * 0.01
+    w_panel = weight[:panel]
+    hidden_m = torch.randn(m, h, **bf16)
+    flops = 2.0 * m * panel * h
+    result["grad_hidden_panel"] = entry(f"[{m},{panel}] x [{panel},{h}] bf16",
+                                        timed(lambda: torch.matmul(g, w_panel)), flops)
+    result["grad_weight_panel"] = entry(f"[{m},{panel}]^T x [{m},{h}] bf16",
+                                        timed(lambda: torch.matmul(g.t(), hidden_m)), flops)
+    return result
 
 
 def bench_next_objective(args) -> int:
