@@ -74,6 +74,11 @@ struct MfmaTileLayout {
   __device__ __forceinline__ int col(int j) const {
     return wn * (kTN * 32) + j * 32 + (lane & 31);
   }
+  // The tile columns that have owned index j in some thread: number t of them.
+  static constexpr int kTokensPerIndex = kWavesN * 32;
+  static __device__ __forceinline__ int token_of_index(int j, int t) {
+    return (t >> 5) * (kTN * 32) + j * 32 + (t & 31);
+  }
   __device__ __forceinline__ int row(int i) const {
     return wm * 128 + (i >> 4) * 32 + ((i >> 2) & 3) * 8 + (lane >> 5) * 4 + (i & 3);
   }

@@ -360,80 +360,125 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   const bool onehot = __ballot(label_here) != 0ull;
 
   const int excluded = (int)p.exclude;
-  auto transform = [&](auto edge_tag, auto onehot_tag) {
+  // one logit -> its entry of g (kEdge: the tile holds rows past v or the
+  // excluded column; kOnehot: some lane of this wave owns a label of the tile)
+  auto grad_of = [&](float z, int j, int row, bool vok, auto edge_tag, auto onehot_tag) -> float {
     constexpr bool kEdge = decltype(edge_tag)::value;
     constexpr bool kOnehot = decltype(onehot_tag)::value;
-    asm volatile("" ::: "memory");   // one real branch per variant, no merged selects
-#pragma unroll
-    for (int i = 0; i < E::kRows; ++i) {
-      const int row = eng.row(i);
-      const bool vok = !kEdge || ((vbase + row < p.v) && (vbase + row != excluded));
-      float row_sum = 0.0f;
-#pragma unroll
-      for (int j = 0; j < E::kCols; ++j) {
-        float z = E::get(acc, j, i);
-        float dcap = 1.0f;
-        float g;
-        if (kSoftcap) {
-          const float t = fast_tanh(z * inv_cap);   // inv_cap includes logit_scale
-          z = p.softcap * t;
-          dcap = 1.0f - t * t;
-          g = fast_exp2(fmaf(z, TLCE_LOG2E, -lse2[j]));
-        } else {
-          g = fast_exp2(fmaf(z, log2e_scaled, -lse2[j]));
-        }
-        if (kOnehot && row == label_row[j]) g -= 1.0f;
-        g *= scale[j];
-        if (kSoftcap && p.cap_grad) g *= dcap;
-        if (kEdge) g = vok ? g : 0.0f;
-        E::set(acc, j, i, g);
-        row_sum += g;
-      }
-      if (kBias) {
-        const int v = vbase + row;
-        row_sum = eng.reduce_over_cols(row_sum);
-        if (eng.col_leader() && v < p.v && row_sum != 0.0f) atomicAdd(p.grad_bias + v, row_sum);
-      }
+    float dcap = 1.0f;
+    float g;
+    if (kSoftcap) {
+      const float t = fast_tanh(z * inv_cap);   // inv_cap includes logit_scale
+      z = p.softcap * t;
+      dcap = 1.0f - t * t;
+      g = fast_exp2(fmaf(z, TLCE_LOG2E, -lse2[j]));
+    } else {
+      g = fast_exp2(fmaf(z, log2e_scaled, -lse2[j]));
     }
+    if (kOnehot && row == label_row[j]) g -= 1.0f;
+    g *= scale[j];
+    if (kSoftcap && p.cap_grad) g *= dcap;
+    if (kEdge) g = vok ? g : 0.0f;
+    return g;
   };
-  if (edge) {
-    transform(std::true_type{}, std::true_type{});
-  } else if (onehot) {
-    transform(std::false_type{}, std::true_type{});
-  } else {
-    transform(std::false_type{}, std::false_type{});
-  }
+  auto add_grad_bias = [&](int row, float row_sum) {
+    const int v = vbase + row;
+    row_sum = eng.reduce_over_cols(row_sum);
+    if (eng.col_leader() && v < p.v && row_sum != 0.0f) atomicAdd(p.grad_bias + v, row_sum);
+  };
 
   T* g_out = static_cast<T*>(p.g);
   T* gt_out = static_cast<T*>(p.gt);
   const int prow = pv * E::kTile;  // first panel column of this tile
   if constexpr (E::kHasKMajor && sizeof(T) == 2) {
-    // The MFMA engine's LDS is free after the main loop: stage the tile there
+    // The MFMA engine's LDS is free after the main loop: the tile is staged there
     // as [token][vocab] (512-byte rows, 16-byte chunk c of token t in slot
-    // c ^ (t & 31)) and write G in whole 512-byte rows.
+    // c ^ (t & 31)) and G is written in whole 512-byte rows.  The work goes by
+    // owned column index j: the tokens with index j (a quarter of the tile) are
+    // transformed, staged and stored while the next quarter is being transformed,
+    // so that only the last quarter's stores are still in flight when the
+    // workgroup ends and frees its CU.
+    auto emit = [&](auto edge_tag, auto onehot_tag) {
+      constexpr bool kEdge = decltype(edge_tag)::value;
+      asm volatile("" ::: "memory");   // one real branch per variant, no merged selects
+      float row_sum[kBias ? E::kRows : 1];
+      if (kBias) {
 #pragma unroll
-    for (int j = 0; j < E::kCols; ++j) {
-      const int tok = eng.col(j);
-#pragma unroll
-      for (int i = 0; i < E::kRows; i += 4) {
-        const int vq = eng.row(i) >> 2;
-        T* dst = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
-                                      (vq & 1) * 8);
-        store4<T>(dst, E::get(acc, j, i), E::get(acc, j, i + 1), E::get(acc, j, i + 2),
-                  E::get(acc, j, i + 3));
+        for (int i = 0; i < E::kRows; ++i) row_sum[i] = 0.0f;
       }
-    }
-    __syncthreads();
-#pragma unroll 4
-    for (int it = 0; it < (E::kTile * 32) / E::kThreads; ++it) {
-      const int c = it * E::kThreads + threadIdx.x;
-      const int tok = c >> 5;
-      const int ch = c & 31;
-      const uint4 val =
-          *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16));
-      stream_store16(g_out + ((int64_t)tt * E::kTile + tok) * p.ldg + prow + ch * 8, val);
+#pragma unroll
+      for (int j = 0; j < E::kCols; ++j) {
+        const int tok = eng.col(j);
+        const int64_t r = (int64_t)tt * E::kTile + tok;
+#pragma unroll
+        for (int i = 0; i < E::kRows; i += 4) {
+          float g4[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int row = eng.row(i + q);
+            const bool vok = !kEdge || ((vbase + row < p.v) && (vbase + row != excluded));
+            g4[q] = grad_of(E::get(acc, j, i + q), j, row, vok, edge_tag, onehot_tag);
+            if (kBias) row_sum[i + q] += g4[q];
+          }
+          const int vq = eng.row(i) >> 2;
+          T* dst = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
+                                        (vq & 1) * 8);
+          store4<T>(dst, g4[0], g4[1], g4[2], g4[3]);
+          if (gt_out != nullptr) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              gt_out[(int64_t)(prow + eng.row(i + q)) * p.ldgt + r] = from_float<T>(g4[q]);
+          }
+        }
+        __syncthreads();
+        constexpr int kPieces = E::kTokensPerIndex * 32;   // 16-byte pieces of this quarter
+#pragma unroll
+        for (int it = 0; it < kPieces / E::kThreads; ++it) {
+          const int c = it * E::kThreads + threadIdx.x;
+          const int t = E::token_of_index(j, c >> 5);
+          const int ch = c & 31;
+          const uint4 val =
+              *reinterpret_cast<const uint4*>(smem + t * 512 + ((ch ^ (t & 31)) * 16));
+          stream_store16(g_out + ((int64_t)tt * E::kTile + t) * p.ldg + prow + ch * 8, val);
+        }
+      }
+      if (kBias) {
+#pragma unroll
+        for (int i = 0; i < E::kRows; ++i) add_grad_bias(eng.row(i), row_sum[i]);
+      }
+    };
+    if (edge) {
+      emit(std::true_type{}, std::true_type{});
+    } else if (onehot) {
+      emit(std::false_type{}, std::true_type{});
+    } else {
+      emit(std::false_type{}, std::false_type{});
     }
   } else {
+    auto transform = [&](auto edge_tag, auto onehot_tag) {
+      constexpr bool kEdge = decltype(edge_tag)::value;
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int i = 0; i < E::kRows; ++i) {
+        const int row = eng.row(i);
+        const bool vok = !kEdge || ((vbase + row < p.v) && (vbase + row != excluded));
+        float row_sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < E::kCols; ++j) {
+          const float g = grad_of(E::get(acc, j, i), j, row, vok, edge_tag, onehot_tag);
+          E::set(acc, j, i, g);
+          row_sum += g;
+        }
+        if (kBias) add_grad_bias(row, row_sum);
+      }
+    };
+    if (edge) {
+      transform(std::true_type{}, std::true_type{});
+    } else if (onehot) {
+      transform(std::false_type{}, std::true_type{});
+    } else {
+      transform(std::false_type{}, std::false_type{});
+    }
 #pragma unroll
     for (int j = 0; j < E::kCols; ++j) {
       const int64_t r = (int64_t)tt * E::kTile + eng.col(j);
@@ -443,14 +488,14 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
                   E::get(acc, j, i + 1), E::get(acc, j, i + 2), E::get(acc, j, i + 3));
       }
     }
-  }
-  if (gt_out != nullptr) {
+    if (gt_out != nullptr) {
 #pragma unroll
-    for (int j = 0; j < E::kCols; ++j) {
-      const int64_t r = (int64_t)tt * E::kTile + eng.col(j);
+      for (int j = 0; j < E::kCols; ++j) {
+        const int64_t r = (int64_t)tt * E::kTile + eng.col(j);
 #pragma unroll
-      for (int i = 0; i < E::kRows; ++i)
-        gt_out[(int64_t)(prow + eng.row(i)) * p.ldgt + r] = from_float<T>(E::get(acc, j, i));
+        for (int i = 0; i < E::kRows; ++i)
+          gt_out[(int64_t)(prow + eng.row(i)) * p.ldgt + r] = from_float<T>(E::get(acc, j, i));
+      }
     }
   }
 }
@@ -605,16 +650,20 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
         process(j, i4, t, g);
         if (grad) store4<T>(cell, g[0], g[1], g[2], g[3]);
       }
-    }
-    if (grad) {
-      __syncthreads();
-#pragma unroll 4
-      for (int it = 0; it < (E::kTile * 32) / E::kThreads; ++it) {
-        const int c = it * E::kThreads + threadIdx.x;
-        const int tok = c >> 5;
-        const int ch = c & 31;
-        stream_store16(panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 8,
-                       *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)));
+      if (grad) {
+        // the tokens with owned index j are complete: their rows go out while
+        // the next quarter of the tile is being processed
+        __syncthreads();
+        constexpr int kPieces = E::kTokensPerIndex * 32;
+#pragma unroll
+        for (int it = 0; it < kPieces / E::kThreads; ++it) {
+          const int c = it * E::kThreads + threadIdx.x;
+          const int tok = E::token_of_index(j, c >> 5);
+          const int ch = c & 31;
+          stream_store16(
+              panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 8,
+              *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)));
+        }
       }
     }
   } else {
