@@ -71,6 +71,11 @@ struct MfmaTileLayout {
     wn = wave % kWavesN;
   }
 
+  // An empty asm that "modifies" the lane index: values derived from it before
+  // this point are not reused after it, so a kernel that loops over tiles can
+  // keep the compiler from hoisting (and then spilling) per-lane addresses.
+  __device__ __forceinline__ void forget_lane_invariants() { asm volatile("" : "+v"(lane)); }
+
   __device__ __forceinline__ int col(int j) const {
     return wn * (kTN * 32) + j * 32 + (lane & 31);
   }
@@ -223,6 +228,15 @@ struct MfmaEngine : MfmaTileLayout<T_> {
       if (more) sstore(cur ^ 1);
       __syncthreads();
     }
+  }
+
+  // acc = A * B^T (same operands as mainloop).
+  __device__ __forceinline__ void mainloop_set(const T* __restrict__ A, int64_t lda, int a_row0,
+                                               int a_rows, const T* __restrict__ B, int64_t ldb,
+                                               int b_row0, int b_rows, int k_begin, int k_end,
+                                               Acc& acc, char* smem) const {
+    Base::zero(acc);
+    mainloop(A, lda, a_row0, a_rows, B, ldb, b_row0, b_rows, k_begin, k_end, acc, smem);
   }
 };
 
@@ -406,7 +420,10 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
   // x.rows - 1).  K-major operand: tile columns row0 .. row0+256 of x (16-byte
   // column chunks clamped to the last valid one; x.rows is a multiple of 8);
   // all K rows in [k_begin, k_end) must exist.
-  template <bool kAKMajor, bool kBKMajor>
+  // kOverwrite: acc = A-tile * B-tile^T instead (the incoming acc is ignored: the
+  // first 16 MFMAs take a zero constant as their addend, which saves zeroing
+  // 256 accumulator registers per tile).
+  template <bool kAKMajor, bool kBKMajor, bool kOverwrite = false>
   __device__ __forceinline__ void mainloop_ex(const Operand<T>& A, const Operand<T>& B,
                                               int k_begin, int k_end, Acc& acc,
                                               char* smem) const {
@@ -433,8 +450,9 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
 
     const int nk = (k_end - k_begin) / kBK;
     constexpr bool kLoadsInPairs = !(kAKMajor && !kBKMajor);
-    auto step = [&](int k, Frags& fa, Frags& fb, auto has_next_tag) {
+    auto step = [&](int k, Frags& fa, Frags& fb, auto has_next_tag, auto first_tag) {
       constexpr bool kHasNext = decltype(has_next_tag)::value;
+      constexpr bool kFirst = decltype(first_tag)::value;   // first step of an overwriting loop
       const int cur = k & 1;
       const int nxt = cur ^ 1;
       const bool more = (k + 2 < nk);
@@ -454,7 +472,12 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
         }
 #pragma unroll
         for (int t = 0; t < kTN; ++t) {
-          acc.c[q][t] = Op::mma(fcur.a[q], fcur.b[t], acc.c[q][t]);
+          if (kFirst && sl == 0) {
+            const f32x16_t zero = {};
+            acc.c[q][t] = Op::mma(fcur.a[q], fcur.b[t], zero);
+          } else {
+            acc.c[q][t] = Op::mma(fcur.a[q], fcur.b[t], acc.c[q][t]);
+          }
           if (sl < 3) {
             if (t == 0) read_one(fnext, cur, sl + 1, 2 * q);
             if (t == 2) read_one(fnext, cur, sl + 1, 2 * q + 1);
@@ -498,8 +521,18 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
 #pragma unroll
     for (int r = 0; r < 8; ++r) read_one(f0, 0, 0, r);
     // a step consumes slices from f0,f1,f0,f1 and leaves the next tile's slice 0 in f0
-    for (int k = 0; k + 1 < nk; ++k) step(k, f0, f1, std::true_type{});
-    step(nk - 1, f0, f1, std::false_type{});
+    if constexpr (kOverwrite) {
+      if (nk > 1) {
+        step(0, f0, f1, std::true_type{}, std::true_type{});
+        for (int k = 1; k + 1 < nk; ++k) step(k, f0, f1, std::true_type{}, std::false_type{});
+        step(nk - 1, f0, f1, std::false_type{}, std::false_type{});
+      } else {
+        step(0, f0, f1, std::false_type{}, std::true_type{});
+      }
+    } else {
+      for (int k = 0; k + 1 < nk; ++k) step(k, f0, f1, std::true_type{}, std::false_type{});
+      step(nk - 1, f0, f1, std::false_type{}, std::false_type{});
+    }
     __syncthreads();
   }
 
@@ -510,6 +543,16 @@ struct MfmaDirect4Engine : MfmaTileLayout<T_, 2, 4> {
     const Operand<T> a = {A, lda, a_row0, a_rows};
     const Operand<T> b = {B, ldb, b_row0, b_rows};
     mainloop_ex<false, false>(a, b, k_begin, k_end, acc, smem);
+  }
+
+  // acc = A * B^T over a non-empty K range (same operands as mainloop).
+  __device__ __forceinline__ void mainloop_set(const T* __restrict__ A, int64_t lda, int a_row0,
+                                               int a_rows, const T* __restrict__ B, int64_t ldb,
+                                               int b_row0, int b_rows, int k_begin, int k_end,
+                                               Acc& acc, char* smem) const {
+    const Operand<T> a = {A, lda, a_row0, a_rows};
+    const Operand<T> b = {B, ldb, b_row0, b_rows};
+    mainloop_ex<false, false, true>(a, b, k_begin, k_end, acc, smem);
   }
 };
 

@@ -46,6 +46,7 @@ struct SimtEngine {
   // every lane of a wave owns a different tile column
   __device__ __forceinline__ float reduce_over_rows_in_wave(float v) const { return v; }
   __device__ __forceinline__ bool row_leader() const { return true; }
+  __device__ __forceinline__ void forget_lane_invariants() {}
 
   __device__ __forceinline__ void mainloop(const T* __restrict__ A, int64_t lda, int a_row0,
                                            int a_rows, const T* __restrict__ B, int64_t ldb,
@@ -76,6 +77,15 @@ struct SimtEngine {
       }
       __syncthreads();
     }
+  }
+
+  // acc = A * B^T (same operands as mainloop).
+  __device__ __forceinline__ void mainloop_set(const T* __restrict__ A, int64_t lda, int a_row0,
+                                               int a_rows, const T* __restrict__ B, int64_t ldb,
+                                               int b_row0, int b_rows, int k_begin, int k_end,
+                                               Acc& acc, char* smem) const {
+    zero(acc);
+    mainloop(A, lda, a_row0, a_rows, B, ldb, b_row0, b_rows, k_begin, k_end, acc, smem);
   }
 };
 

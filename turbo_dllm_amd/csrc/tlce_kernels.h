@@ -56,10 +56,13 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
   }
 
   for (int vt = vt0; vt < vt1; ++vt) {
+    // Everything derived from the lane index is recomputed per tile: kept live as
+    // loop invariants, those addresses get spilled across the epilogue below and
+    // reloaded from scratch at the top of every tile (3 % of this kernel).
+    eng.forget_lane_invariants();
     typename E::Acc acc;
-    E::zero(acc);
-    eng.mainloop(weight, p.h, vt * E::kTile, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc,
-                 smem);
+    eng.mainloop_set(weight, p.h, vt * E::kTile, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h,
+                     acc, smem);
     const int vbase = vt * E::kTile;
     if (kBias) {
 #pragma unroll
@@ -320,9 +323,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   const T* hidden = static_cast<const T*>(p.hidden);
   const T* weight = static_cast<const T*>(p.weight);
   typename E::Acc acc;
-  E::zero(acc);
   const int vbase = p.v0 + pv * E::kTile;
-  eng.mainloop(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+  eng.mainloop_set(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
 
   const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
   const float log2e_scaled = TLCE_LOG2E * p.logit_scale;
@@ -409,7 +411,6 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 #pragma unroll
       for (int j = 0; j < E::kCols; ++j) {
         const int tok = eng.col(j);
-        const int64_t r = (int64_t)tt * E::kTile + tok;
 #pragma unroll
         for (int i = 0; i < E::kRows; i += 4) {
           float g4[4];
@@ -424,11 +425,6 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
           T* dst = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
                                         (vq & 1) * 8);
           store4<T>(dst, g4[0], g4[1], g4[2], g4[3]);
-          if (gt_out != nullptr) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-              gt_out[(int64_t)(prow + eng.row(i + q)) * p.ldgt + r] = from_float<T>(g4[q]);
-          }
         }
         __syncthreads();
         constexpr int kPieces = E::kTokensPerIndex * 32;   // 16-byte pieces of this quarter
@@ -453,6 +449,17 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
       emit(std::false_type{}, std::true_type{});
     } else {
       emit(std::false_type{}, std::false_type{});
+    }
+    if (gt_out != nullptr) {
+      // transposed copy for the contractions that cannot read G K-major (vocabulary
+      // not a multiple of 64): the whole tile is still staged; thread = token
+      const int tok = threadIdx.x % E::kTile;
+      for (int vrow = threadIdx.x / E::kTile; vrow < E::kTile; vrow += E::kThreads / E::kTile) {
+        const T val = *reinterpret_cast<const T*>(smem + tok * 512 +
+                                                  (((vrow >> 3) ^ (tok & 31)) * 16) +
+                                                  (vrow & 7) * 2);
+        gt_out[(int64_t)(prow + vrow) * p.ldgt + (int64_t)tt * E::kTile + tok] = val;
+      }
     }
   } else {
     auto transform = [&](auto edge_tag, auto onehot_tag) {
@@ -549,10 +556,9 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
 
   E eng;
   typename E::Acc acc;
-  E::zero(acc);
   const int vbase = p.v0 + pv * E::kTile;
-  eng.mainloop(static_cast<const T*>(p.weight), p.h, vbase, p.v, static_cast<const T*>(p.hidden),
-               p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+  eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
+                   static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
 
   const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
   const bool grad = p.mode == kKlGrad;
@@ -757,10 +763,9 @@ __global__ __launch_bounds__(E::kThreads) void lce_logits_panel_kernel(LogitsPan
   grouped_tile(logical, p.n_ttiles, p.n_ptiles, 4, &tt, &pv);
   E eng;
   typename E::Acc acc;
-  E::zero(acc);
   const int vbase = p.v0 + pv * E::kTile;
-  eng.mainloop(static_cast<const T*>(p.weight), p.h, vbase, p.v, static_cast<const T*>(p.hidden),
-               p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+  eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
+                   static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
   const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
   const int prow = pv * E::kTile;
 #pragma unroll
@@ -1160,17 +1165,16 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
 
   E eng;
   typename E::Acc acc;
-  E::zero(acc);
   if (k_begin >= k_end) {
-    // nothing to accumulate
+    E::zero(acc);   // nothing to accumulate
   } else if constexpr (E::kHasKMajor) {
     const Operand<T> a = {static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows};
     const Operand<T> b = {static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows};
-    eng.template mainloop_ex<kAKMajor, kBKMajor>(a, b, k_begin, k_end, acc, smem);
+    eng.template mainloop_ex<kAKMajor, kBKMajor, true>(a, b, k_begin, k_end, acc, smem);
   } else {
-    eng.mainloop(static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows,
-                 static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows, k_begin, k_end,
-                 acc, smem);
+    eng.mainloop_set(static_cast<const T*>(p.a), p.lda, ti * E::kTile, p.a_rows,
+                     static_cast<const T*>(p.b), p.ldb, tj * E::kTile, p.b_rows, k_begin, k_end,
+                     acc, smem);
   }
 
   // runs of 4 can be moved as one vector when every row start keeps them aligned
