@@ -165,55 +165,90 @@ struct CombineArgs {
   float* target_logits;
 };
 
+// Dot product of two rows of length h by one wave (every lane gets the sum):
+// 16 bytes per lane and load for 2-byte types when the rows allow it.
+template <typename T>
+__device__ __forceinline__ float wave_dot(const T* a_row, const T* b_row, int h, int lane) {
+  float dot = 0.0f;
+  if (sizeof(T) == 2 && (h % 8) == 0 &&
+      ((reinterpret_cast<uintptr_t>(a_row) | reinterpret_cast<uintptr_t>(b_row)) & 15) == 0) {
+    typedef T v8_t __attribute__((ext_vector_type(8)));
+    for (int k = lane * 8; k < h; k += 64 * 8) {
+      const v8_t a = *reinterpret_cast<const v8_t*>(a_row + k);
+      const v8_t b = *reinterpret_cast<const v8_t*>(b_row + k);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot = fmaf(to_float<T>(a[e]), to_float<T>(b[e]), dot);
+    }
+  } else {
+    for (int k = lane; k < h; k += 64) dot = fmaf(to_float<T>(a_row[k]), to_float<T>(b_row[k]), dot);
+  }
+  return wave_sum(dot);
+}
+
+// Rows per workgroup of lce_combine_loss_kernel: 4 waves x 4 rows, so that the
+// count of valid rows costs one global atomic per 16 rows (one per row
+// serialises 32768 atomics on a single address: two thirds of this kernel).
+constexpr int kCombineRowsPerBlock = 16;
+
 template <typename T>
 __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
+  __shared__ int block_valid;
   const int lane = threadIdx.x & 63;
-  const int r = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= p.m) return;
-  float mx = -INFINITY;
-  for (int s = lane; s < p.nsplit; s += 64) mx = fmaxf(mx, p.part_max[(int64_t)s * p.part_ld + r]);
-  mx = wave_max(mx);
-  float sum = 0.0f;
-  for (int s = lane; s < p.nsplit; s += 64) {
-    const float pm = p.part_max[(int64_t)s * p.part_ld + r];
-    if (pm > -INFINITY) sum += p.part_sum[(int64_t)s * p.part_ld + r] * fast_exp2(pm - mx);
-  }
-  sum = wave_sum(sum);
-  const float lse = (mx + log2f(sum)) * TLCE_LN2;
-
-  if (p.labels == nullptr) {   // statistics only (soft embedding): no targets, no loss
-    if (lane == 0) p.lse[r] = lse;
-    return;
-  }
-  const int64_t label = p.labels[r];
-  const bool valid = (label != p.ignore);
-  const int64_t y = label - p.label_offset;   // row of the label in this weight
-  const bool here = valid && y >= 0 && y < p.v;
-  const bool has_target = here && label != p.exclude;
-  float target = 0.0f;
-  if (has_target) {
-    const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
-    const T* wrow = static_cast<const T*>(p.weight) + y * (int64_t)p.h;
-    float dot = 0.0f;
-    for (int k = lane; k < p.h; k += 64) dot = fmaf(to_float<T>(hrow[k]), to_float<T>(wrow[k]), dot);
-    dot = wave_sum(dot);
-    if (p.bias != nullptr) dot += p.bias[y];
-    if (p.softcap > 0.0f) dot = p.softcap * tanhf(dot / p.softcap);
-    target = dot;
-  }
-  if (lane == 0) {
-    if (p.local_max != nullptr) {
-      // the partials are in base-2 units: max2 = max * log2(e), sum = sum exp(z - max)
-      p.local_max[r] = mx * TLCE_LN2;
-      p.local_sum[r] = (mx > -INFINITY) ? sum : 0.0f;
-      p.target_logits[r] = (here && label == p.exclude) ? -INFINITY : target;
-    } else {
-      p.lse[r] = lse;
-      const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r;
-      p.losses[o] = valid ? (lse - target) : 0.0f;
+  const int wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) block_valid = 0;
+  __syncthreads();
+  int wave_valid = 0;
+  for (int i = 0; i < kCombineRowsPerBlock / 4; ++i) {
+    const int r = blockIdx.x * kCombineRowsPerBlock + wave * (kCombineRowsPerBlock / 4) + i;
+    if (r >= p.m) break;
+    float mx = -INFINITY;
+    for (int s = lane; s < p.nsplit; s += 64)
+      mx = fmaxf(mx, p.part_max[(int64_t)s * p.part_ld + r]);
+    mx = wave_max(mx);
+    float sum = 0.0f;
+    for (int s = lane; s < p.nsplit; s += 64) {
+      const float pm = p.part_max[(int64_t)s * p.part_ld + r];
+      if (pm > -INFINITY) sum += p.part_sum[(int64_t)s * p.part_ld + r] * fast_exp2(pm - mx);
     }
-    if (valid) atomicAdd(p.valid_count, 1.0f);
+    sum = wave_sum(sum);
+    const float lse = (mx + log2f(sum)) * TLCE_LN2;
+
+    if (p.labels == nullptr) {   // statistics only (soft embedding): no targets, no loss
+      if (lane == 0) p.lse[r] = lse;
+      continue;
+    }
+    const int64_t label = p.labels[r];
+    const bool valid = (label != p.ignore);
+    const int64_t y = label - p.label_offset;   // row of the label in this weight
+    const bool here = valid && y >= 0 && y < p.v;
+    const bool has_target = here && label != p.exclude;
+    float target = 0.0f;
+    if (has_target) {
+      const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
+      const T* wrow = static_cast<const T*>(p.weight) + y * (int64_t)p.h;
+      float dot = wave_dot<T>(hrow, wrow, p.h, lane);
+      if (p.bias != nullptr) dot += p.bias[y];
+      if (p.softcap > 0.0f) dot = p.softcap * tanhf(dot / p.softcap);
+      target = dot;
+    }
+    if (lane == 0) {
+      if (p.local_max != nullptr) {
+        // the partials are in base-2 units: max2 = max * log2(e), sum = sum exp(z - max)
+        p.local_max[r] = mx * TLCE_LN2;
+        p.local_sum[r] = (mx > -INFINITY) ? sum : 0.0f;
+        p.target_logits[r] = (here && label == p.exclude) ? -INFINITY : target;
+      } else {
+        p.lse[r] = lse;
+        const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r;
+        p.losses[o] = valid ? (lse - target) : 0.0f;
+      }
+    }
+    wave_valid += valid ? 1 : 0;
   }
+  if (p.valid_count == nullptr) return;   // uniform: statistics-only callers
+  if (lane == 0 && wave_valid != 0) atomicAdd(&block_valid, wave_valid);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_valid != 0) atomicAdd(p.valid_count, (float)block_valid);
 }
 
 // ----------------------------------------------------------------- backward --
@@ -1056,9 +1091,7 @@ __global__ __launch_bounds__(256) void lce_topk_finish_kernel(TopkFinishArgs p) 
   if (r >= p.m) return;
   const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
   const T* wrow = static_cast<const T*>(p.weight) + p.labels[r] * (int64_t)p.h;
-  float dot = 0.0f;
-  for (int k = lane; k < p.h; k += 64) dot = fmaf(to_float<T>(hrow[k]), to_float<T>(wrow[k]), dot);
-  dot = wave_sum(dot) * p.logit_scale;
+  float dot = wave_dot<T>(hrow, wrow, p.h, lane) * p.logit_scale;
   if (p.softcap > 0.0f) dot = p.softcap * tanhf(dot / p.softcap);
   if (lane == 0) {
     const float lse = p.run_max[r] + logf(p.run_sum[r]);

@@ -354,7 +354,7 @@ int forward_impl(const Plan& p, const void* hidden, const void* weight, const fl
   ca.target_logits = shard.target_logits;
   {
     ScopedTimer timer(kClassCombine, stream);
-    lce_combine_loss_kernel<T><<<(int)ceil_div(m, 4), 256, 0, stream>>>(ca);
+    lce_combine_loss_kernel<T><<<(int)ceil_div(m, kCombineRowsPerBlock), 256, 0, stream>>>(ca);
   }
   TLCE_LAUNCH_CHECK();
   return 0;
@@ -624,7 +624,7 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
   ca.label_offset = 0; ca.local_max = nullptr; ca.local_sum = nullptr; ca.target_logits = nullptr;
   {
     ScopedTimer timer(kClassCombine, stream);
-    lce_combine_loss_kernel<T><<<(int)ceil_div(m, 4), 256, 0, stream>>>(ca);
+    lce_combine_loss_kernel<T><<<(int)ceil_div(m, kCombineRowsPerBlock), 256, 0, stream>>>(ca);
     lce_kl_finish_kernel<<<(int)ceil_div(m, 256), 256, 0, stream>>>(losses, tsum, draft_lse,
                                                                     (int)m);
   }
