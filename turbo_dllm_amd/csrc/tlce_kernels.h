@@ -803,19 +803,57 @@ __global__ __launch_bounds__(E::kThreads) void lce_logits_panel_kernel(LogitsPan
                    static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
   const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
   const int prow = pv * E::kTile;
+  auto logits4 = [&](int j, int i4) -> float4 {
+    float z[4];
 #pragma unroll
-  for (int j = 0; j < E::kCols; ++j) {
-    float* out = p.panel + ((int64_t)tt * E::kTile + eng.col(j)) * p.ld + prow;
+    for (int u = 0; u < 4; ++u) {
+      const float raw = E::get(acc, j, i4 + u);
+      const float val = kSoftcap ? p.softcap * fast_tanh(raw * inv_cap) : raw * p.logit_scale;
+      z[u] = (vbase + eng.row(i4 + u) < p.v) ? val : -INFINITY;
+    }
+    return make_float4(z[0], z[1], z[2], z[3]);
+  };
+  if constexpr (E::kHasKMajor && E::kCols == 4) {
+    // The float32 tile is twice the engine's LDS: it is staged and written in two
+    // halves (the tokens of two owned column indices = 128 rows of 1 KiB, 16-byte
+    // chunk c of staged row s in slot c ^ (s & 63)), so that G leaves in whole
+    // 1 KiB rows instead of 16-byte pieces a row apart.
+    constexpr int kPerIndex = E::kTokensPerIndex;     // 64 tokens per owned index
 #pragma unroll
-    for (int i4 = 0; i4 < E::kRows; i4 += 4) {
-      float z[4];
+    for (int half = 0; half < 2; ++half) {
+      if (half) __syncthreads();                      // the first half has been read out
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const float raw = E::get(acc, j, i4 + u);
-        const float val = kSoftcap ? p.softcap * fast_tanh(raw * inv_cap) : raw * p.logit_scale;
-        z[u] = (vbase + eng.row(i4 + u) < p.v) ? val : -INFINITY;
+      for (int jj = 0; jj < 2; ++jj) {
+        const int j = 2 * half + jj;
+        // position of this lane's token among those with index j, as token_of_index counts
+        const int t = (eng.col(j) / (E::kTile / 2)) * 32 + (eng.col(j) & 31);
+        const int s_row = jj * kPerIndex + t;
+#pragma unroll
+        for (int i4 = 0; i4 < E::kRows; i4 += 4) {
+          const int c = eng.row(i4) >> 2;
+          *reinterpret_cast<float4*>(smem + s_row * 1024 + ((c ^ (s_row & 63)) * 16)) =
+              logits4(j, i4);
+        }
       }
-      *reinterpret_cast<float4*>(out + eng.row(i4)) = make_float4(z[0], z[1], z[2], z[3]);
+      __syncthreads();
+#pragma unroll 4
+      for (int it = 0; it < (2 * kPerIndex * 64) / E::kThreads; ++it) {
+        const int idx = it * E::kThreads + threadIdx.x;
+        const int s_row = idx >> 6;
+        const int ch = idx & 63;
+        const int tok = E::token_of_index(2 * half + s_row / kPerIndex, s_row % kPerIndex);
+        const uint4 val =
+            *reinterpret_cast<const uint4*>(smem + s_row * 1024 + ((ch ^ (s_row & 63)) * 16));
+        stream_store16(p.panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 4, val);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      float* out = p.panel + ((int64_t)tt * E::kTile + eng.col(j)) * p.ld + prow;
+#pragma unroll
+      for (int i4 = 0; i4 < E::kRows; i4 += 4)
+        *reinterpret_cast<float4*>(out + eng.row(i4)) = logits4(j, i4);
     }
   }
 }
