@@ -580,7 +580,7 @@ struct KlPanelArgs {
   int mode;
 };
 
-template <class E, bool kSoftcap>
+template <class E, bool kSoftcap, bool kGrad>
 __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
@@ -596,7 +596,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
                    static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
 
   const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
-  const bool grad = p.mode == kKlGrad;
+  constexpr bool grad = kGrad;   // p.mode, fixed at compile time: no mode test per group of 4
   float lse2[E::kCols], scale[E::kCols], partial[E::kCols], tsum[E::kCols];
   float tile_max[E::kCols], tile_sum[E::kCols];
   bool live[E::kCols];
@@ -652,12 +652,14 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
         g[u] = vok ? v : 0.0f;
       } else {
         // z already is the capped draft logit in base-2 units (-inf past the vocabulary)
+        // selects, not branches: the lanes of a wave disagree on tv > 0
         const float tv = t[u];
-        if (vok) tile_sum[j] += fast_exp2(z - tile_max[j]);
-        if (vok && tv > 0.0f) {
-          partial[j] += tv * ((fast_log2(tv) - z) * TLCE_LN2) - tv;
-          tsum[j] += tv;
-        }
+        const float e = fast_exp2(z - tile_max[j]);
+        tile_sum[j] += vok ? e : 0.0f;
+        const bool use = vok && tv > 0.0f;
+        const float term = tv * ((fast_log2(tv) - z) * TLCE_LN2) - tv;
+        partial[j] += use ? term : 0.0f;
+        tsum[j] += use ? tv : 0.0f;
       }
     }
   };

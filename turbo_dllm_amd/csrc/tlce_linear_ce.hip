@@ -533,21 +533,27 @@ KlLayout kl_layout(const Plan& pd, const Plan& pt, int64_t m, int64_t hd, int dt
   return l;
 }
 
-template <class E, bool kSoftcap>
+template <class E, bool kSoftcap, bool kGrad>
 int launch_kl_panel_variant(const KlPanelArgs& a, hipStream_t stream) {
   static LdsOptIn lds;
-  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap>, E::kSmemBytes, lds)) return rc;
+  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap, kGrad>, E::kSmemBytes, lds))
+    return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
   ScopedTimer timer(kClassGradLogits, stream);
-  lce_kl_panel_kernel<E, kSoftcap><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  lce_kl_panel_kernel<E, kSoftcap, kGrad><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
 
 template <class E>
 int launch_kl_panel(const KlPanelArgs& a, hipStream_t stream) {
-  if (a.softcap > 0.0f) return launch_kl_panel_variant<E, true>(a, stream);
-  return launch_kl_panel_variant<E, false>(a, stream);
+  const bool grad = a.mode == kKlGrad;
+  if (a.softcap > 0.0f) {
+    return grad ? launch_kl_panel_variant<E, true, true>(a, stream)
+                : launch_kl_panel_variant<E, true, false>(a, stream);
+  }
+  return grad ? launch_kl_panel_variant<E, false, true>(a, stream)
+              : launch_kl_panel_variant<E, false, false>(a, stream);
 }
 
 // Teacher probabilities of the panel [v0, v0 + width), then the draft pass over it.
