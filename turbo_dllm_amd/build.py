@@ -3,8 +3,10 @@
 The reference JIT-builds its CUDA extension through torch.utils.cpp_extension
 with ``-O3 --use_fast_math -lcublas``
 (dllm_parallel/core/kernels/_native_specs.py:63-143).  This library has no
-torch or BLAS dependency, so the build is one hipcc command; the result sits
-next to this file where the ctypes loader looks for it.
+torch or BLAS dependency: every source is compiled to an object with one hipcc
+command (in parallel, one translation unit per tile engine) and the objects
+are linked into a shared library that sits next to this file, where the ctypes
+loader looks for it.
 """
 
 from __future__ import annotations
@@ -13,13 +15,33 @@ import os
 import shutil
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 PACKAGE_DIR = Path(__file__).resolve().parent
 CSRC_DIR = PACKAGE_DIR / "csrc"
+OBJECT_DIR = CSRC_DIR / "build"
 LIBRARY_NAME = "libtlce_gfx950.so"
 LIBRARY_PATH = PACKAGE_DIR / LIBRARY_NAME
-SOURCES = ("tlce_compact.hip", "tlce_linear_ce.hip")
+# (object name, source, extra definitions).  tlce_engine_unit.hip is compiled once
+# per engine, and once per kernel family for the two direct-to-LDS MFMA engines,
+# whose kernels take the longest to compile.
+_SPLIT_ENGINES = {"direct_bf16": "MfmaDirect4Engine<__bf16>",
+                  "direct_f16": "MfmaDirect4Engine<_Float16>"}
+_WHOLE_ENGINES = {"staged_bf16": "MfmaEngine<__bf16>", "staged_f16": "MfmaEngine<_Float16>",
+                  "generic_f32": "SimtEngine<float>", "generic_bf16": "SimtEngine<__bf16>",
+                  "generic_f16": "SimtEngine<_Float16>"}
+_PARTS = {2: "grad_logits", 7: "grad_logits_cap", 8: "grad_logits_bias", 9: "grad_logits_cap_bias",
+          1: "forward", 3: "gemm", 4: "kl", 5: "logits", 6: "sequences"}
+UNITS = (
+    [(f"engine_{tag}_{name}", "tlce_engine_unit.hip",
+      (f"-DTLCE_UNIT_ENGINE={engine}", f"-DTLCE_UNIT_PART={part}"))
+     for tag, engine in _SPLIT_ENGINES.items() for part, name in _PARTS.items()]
+    + [(f"engine_{tag}", "tlce_engine_unit.hip",
+        (f"-DTLCE_UNIT_ENGINE={engine}", "-DTLCE_UNIT_PART=0"))
+       for tag, engine in _WHOLE_ENGINES.items()]
+    + [("linear_ce", "tlce_linear_ce.hip", ()), ("compact", "tlce_compact.hip", ())]
+)
 OFFLOAD_ARCH = "gfx950"
 
 HIPCC_FLAGS = (
@@ -27,7 +49,6 @@ HIPCC_FLAGS = (
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-munsafe-fp-atomics",
     # the direct-to-LDS loads name m0 (reserved) in their inline-asm clobber list
     "-Wno-inline-asm",
@@ -43,11 +64,7 @@ def find_hipcc() -> str:
     raise RuntimeError("hipcc not found; install ROCm or set HIPCC")
 
 
-def build_library(verbose: bool = False) -> Path:
-    """Compiles every HIP source for gfx950 and links the shared library."""
-    command = [find_hipcc(), *HIPCC_FLAGS]
-    command += [str(CSRC_DIR / name) for name in SOURCES]
-    command += ["-o", str(LIBRARY_PATH)]
+def _run(command: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(command), flush=True)
     result = subprocess.run(command, capture_output=True, text=True)
@@ -56,9 +73,26 @@ def build_library(verbose: bool = False) -> Path:
         line for line in result.stderr.splitlines() if "packed-fp32-ops" not in line
     )
     if result.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({result.returncode}):\n{stderr}")
+        raise RuntimeError(f"hipcc failed ({result.returncode}): {' '.join(command)}\n{stderr}")
     if verbose and stderr.strip():
         print(stderr, file=sys.stderr)
+
+
+def build_library(verbose: bool = False, jobs: int | None = None) -> Path:
+    """Compiles every HIP source for gfx950 and links the shared library."""
+    hipcc = find_hipcc()
+    OBJECT_DIR.mkdir(exist_ok=True)
+    objects = [OBJECT_DIR / (name + ".o") for name, _, _ in UNITS]
+    commands = [
+        [hipcc, *HIPCC_FLAGS, *defines, "-c", str(CSRC_DIR / source), "-o", str(obj)]
+        for (_, source, defines), obj in zip(UNITS, objects)
+    ]
+    if jobs is None:
+        jobs = min(len(commands), os.cpu_count() or 1, 16)
+    with ThreadPoolExecutor(max_workers=max(int(jobs), 1)) as pool:
+        list(pool.map(lambda command: _run(command, verbose), commands))
+    _run([hipcc, f"--offload-arch={OFFLOAD_ARCH}", "-shared", "-fPIC",
+          *[str(obj) for obj in objects], "-o", str(LIBRARY_PATH)], verbose)
     return LIBRARY_PATH
 
 
