@@ -111,6 +111,32 @@ int tlce_forward(const void* hidden, const void* weight, const float* bias,
                  float* losses, float* lse, float* valid_count,
                  void* workspace, int64_t workspace_bytes, void* stream);
 
+/* tlce_forward for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same arguments and results as tlce_forward
+ * minus the workspace: the per-split softmax partials, the forward's only
+ * scratch memory, live in a device array of TLCE_FORWARD_NOALLOC_SCRATCH_BYTES
+ * that is part of the library image (every GPU the library runs on holds its
+ * copy until the process ends).  The call allocates and frees nothing.
+ *   - m beyond TLCE_FORWARD_NOALLOC_MAX_ROWS (more partials than the array
+ *     holds) is rejected with an error; nothing is launched then.
+ *   - All calls on one GPU share that GPU's array: calls that overlap on one
+ *     GPU (two streams, two threads) race.  Nothing in it has to start at zero,
+ *     every partial a call reads was written by that call.
+ *   - The first call on a device looks the array's address up
+ *     (hipGetSymbolAddress) and, like every entry point, raises its kernels'
+ *     LDS limit: make one call per device before capturing a graph. */
+#define TLCE_FORWARD_NOALLOC_SCRATCH_BYTES (4 << 20)
+#define TLCE_FORWARD_NOALLOC_MAX_ROWS 524288
+
+int tlce_forward_noalloc(const void* hidden, const void* weight, const float* bias,
+                         const int64_t* labels, const int64_t* row_idx,
+                         int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                         int64_t ignore_index, int64_t exclude_index,
+                         float logit_softcap,
+                         float* losses, float* lse, float* valid_count,
+                         void* stream);
+
 /* ---- backward ------------------------------------------------------------
  * Replaces chunked_linear_ce_backward and ..._backward_frozen_weight
  * (fused_linear_ce.cpp:125-207).  grad_weight == NULL selects the

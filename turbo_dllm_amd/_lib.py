@@ -44,6 +44,16 @@ SIGNATURES = {
             c_void_p, c_int64, c_void_p,                        # workspace bytes stream
         ],
     ),
+    "tlce_forward_noalloc": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden weight bias labels row_idx
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m n_out h v dtype
+            c_int64, c_int64, c_float,                          # ignore exclude softcap
+            c_void_p, c_void_p, c_void_p,                       # losses lse valid_count
+            c_void_p,                                           # stream
+        ],
+    ),
     "tlce_backward_workspace_bytes": (
         c_int64,
         [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int64],

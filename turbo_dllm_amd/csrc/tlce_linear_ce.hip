@@ -166,6 +166,58 @@ extern "C" int tlce_forward(const void* hidden, const void* weight, const float*
                        workspace, workspace_bytes, static_cast<hipStream_t>(stream));
 }
 
+// ------------------------------------------- forward without a workspace ----
+// The forward's only scratch memory (the per-split softmax partials) in a
+// file-scope device array, for callers that may not allocate.  Each GPU holds
+// its own copy of the array at its own address: the address is looked up once
+// per device, with that device current, and only that pointer (never the
+// array's name, which on the host is a stand-in and not a device address) is
+// handed to kernels.
+static __device__ __align__(256) unsigned char scratch[TLCE_FORWARD_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+std::atomic<void*> g_scratch_ptr[kMaxDevices] = {};
+
+// Device address of `scratch` on the current device.
+int scratch_pointer(void** out) {
+  int device = 0;
+  TLCE_HIP(hipGetDevice(&device));
+  TLCE_REQUIRE(device >= 0 && device < kMaxDevices, "device index %d out of range", device);
+  void* ptr = g_scratch_ptr[device].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    TLCE_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    TLCE_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null scratch address");
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int tlce_forward_noalloc(const void* hidden, const void* weight, const float* bias,
+                                    const int64_t* labels, const int64_t* row_idx, int64_t m,
+                                    int64_t n_out, int64_t h, int64_t v, int dtype,
+                                    int64_t ignore_index, int64_t exclude_index,
+                                    float logit_softcap, float* losses, float* lse,
+                                    float* valid_count, void* stream) {
+  TLCE_REQUIRE(m >= 0 && h > 0 && v > 0, "forward_noalloc: bad shape m=%lld h=%lld v=%lld",
+               (long long)m, (long long)h, (long long)v);
+  const int64_t need = forward_layout(make_plan(m, h, v, dtype, false, 0)).total;
+  TLCE_REQUIRE(need <= (int64_t)TLCE_FORWARD_NOALLOC_SCRATCH_BYTES,
+               "forward_noalloc: m=%lld needs %lld bytes of softmax partials, the static scratch "
+               "array holds %lld (at most %lld rows); use tlce_forward with a workspace",
+               (long long)m, (long long)need, (long long)TLCE_FORWARD_NOALLOC_SCRATCH_BYTES,
+               (long long)TLCE_FORWARD_NOALLOC_MAX_ROWS);
+  void* ptr = nullptr;
+  if (int rc = scratch_pointer(&ptr)) return rc;
+  return forward_entry(hidden, weight, bias, labels, row_idx, m, n_out, h, v, dtype, ignore_index,
+                       exclude_index, logit_softcap, losses, lse, valid_count, ShardStats{}, ptr,
+                       (int64_t)TLCE_FORWARD_NOALLOC_SCRATCH_BYTES,
+                       static_cast<hipStream_t>(stream));
+}
+
 extern "C" int tlce_forward_local(const void* hidden, const void* weight, const float* bias,
                                   const int64_t* labels, int64_t m, int64_t h, int64_t v_local,
                                   int dtype, int64_t vocab_start, int64_t ignore_index,
