@@ -90,6 +90,25 @@ int tlce_gather_rows(const void* src, const int64_t* row_idx, int64_t m,
 int tlce_scatter_rows(const void* src, const int64_t* row_idx, int64_t m,
                       int64_t row_bytes, void* dst, void* stream);
 
+/* The compaction gather of the masked-token loss in one launch and without a
+ * host read-back of the row count (the reference reads it at
+ * `row_indices.numel()`, nemotron/model.py:4247): for r < *row_count
+ *   hidden_dst[r] = hidden_src[row_idx[r]], labels_dst[r] = labels_src[row_idx[r]],
+ *   weights_dst[r] = weights_src[row_idx[r]]   (weights optional: both NULL or neither);
+ * the rows from *row_count up to the next multiple of 64 (at most padded_rows)
+ * become zero rows with label ignore_index and weight 0.  row_idx and
+ * row_count are what tlce_compact_rows wrote; `capacity` is the length of the
+ * source (the most rows there can be), hidden_dst holds padded_rows >= capacity
+ * rows of row_bytes bytes, labels_dst / weights_dst
+ * padded_rows entries.  Rows past that stay untouched: consumers given
+ * row_count never read them. */
+int tlce_gather_loss_rows(const void* hidden_src, const int64_t* labels_src,
+                          const float* weights_src, const int64_t* row_idx,
+                          const int64_t* row_count, int64_t capacity,
+                          int64_t padded_rows, int64_t row_bytes,
+                          int64_t ignore_index, void* hidden_dst,
+                          int64_t* labels_dst, float* weights_dst, void* stream);
+
 /* Zero-fills `bytes` bytes at dst with a kernel (safe inside graph capture). */
 int tlce_fill_zero(void* dst, int64_t bytes, void* stream);
 
@@ -163,6 +182,62 @@ int tlce_backward(const void* hidden, const void* weight, const float* bias,
                   void* grad_hidden, void* grad_weight, float* grad_bias,
                   int64_t panel_bytes,
                   void* workspace, int64_t workspace_bytes, void* stream);
+
+/* ---- masked-token loss ---------------------------------------------------
+ * The arithmetic the reference's loss method wraps around the operator
+ * (distributed_block_diffusion_loss, nemotron/model.py:2084-2151;
+ * _native_token_cross_entropy, :1866-1902), folded into the kernels:
+ *   z      = cap(logit_multiplier * hidden . weight^T + bias)
+ *            (the reference multiplies a copy of the hidden states, :2084-2086)
+ *   loss_r = lse(z_r) - z_r[label_r]                 (0 for ignored rows)
+ *   weighted_sum[0] = sum_r token_weights[r] * loss_r      (:2109, :2126-2128)
+ * and in the backward, with g = the scale tlce_backward derives from
+ * grad_output and reduction_code (for the weighted sum: TLCE_REDUCTION_SUM and
+ * grad_output[0] = d objective / d weighted_sum, which carries the caller's
+ * `/ valid_token_count * loss_scale`, :2146-2151):
+ *   d z_r = (softmax(z_r) - onehot) * g * token_weights[r] * cap'
+ *   grad_hidden = logit_multiplier * d z . weight,  grad_weight = logit_multiplier * d z^T . hidden,
+ *   grad_bias = sum_r d z_r.
+ * No scaled copy of the hidden states, no per-token weighting pass, and the sum
+ * is formed in a fixed order (reproducible).
+ *   token_weights: float32 [m] aligned with the (compacted) rows, NULL = all 1.
+ *   row_count: device int64 or NULL.  With it, m is only the capacity the
+ *   launches are sized for: rows r >= *row_count carry no loss and no gradient,
+ *   tiles beyond them exit at once, and the kernels re-derive the tile plan
+ *   from the real count, so no host synchronisation is needed between the
+ *   compaction and the loss.  hidden must then hold round_up(m, 64) rows and
+ *   the rows in [*row_count, round_up(*row_count, 64)) must be finite
+ *   (tlce_gather_loss_rows writes zeros there).
+ *   losses and weighted_sum are each optional (NULL to skip; one of them must
+ *   be given): per-token losses at row_idx positions as tlce_forward writes
+ *   them, and the weighted sum.  logit_multiplier must be positive.
+ *   Workspaces: tlce_masked_loss_forward_workspace_bytes for the forward,
+ *   tlce_backward_workspace_bytes for the backward. */
+int64_t tlce_masked_loss_forward_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                                 int dtype, int dynamic_rows);
+
+int tlce_masked_loss_forward(const void* hidden, const void* weight, const float* bias,
+                             const int64_t* labels, const float* token_weights,
+                             const int64_t* row_idx, const int64_t* row_count,
+                             int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                             int64_t ignore_index, int64_t exclude_index,
+                             float logit_softcap, float logit_multiplier,
+                             float* losses, float* lse, float* valid_count,
+                             float* weighted_sum,
+                             void* workspace, int64_t workspace_bytes, void* stream);
+
+int tlce_masked_loss_backward(const void* hidden, const void* weight, const float* bias,
+                              const int64_t* labels, const float* token_weights,
+                              const int64_t* row_idx, const int64_t* row_count,
+                              const float* lse, const float* valid_count,
+                              const float* grad_output,
+                              int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                              int reduction_code,
+                              int64_t ignore_index, int64_t exclude_index,
+                              float logit_softcap, float logit_multiplier,
+                              void* grad_hidden, void* grad_weight, float* grad_bias,
+                              int64_t panel_bytes,
+                              void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- vocabulary shards ---------------------------------------------------
  * Replace vocab_parallel_ce_forward_local / vocab_parallel_ce_backward_local

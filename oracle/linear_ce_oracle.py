@@ -34,6 +34,10 @@ What each function follows in the reference (paths relative to its tree):
   dense_ce_topk(_grad)     frozen-head CE with the label's probability and the exact
                            top-k logits, and its gradient for hidden
                            (dllm_parallel/core/kernels/dflash_linear_topk.py:100-225).
+  masked_token_loss(_grads) the loss method around the operator: hidden * output_multiplier,
+                           per-token CE * loss weights, / valid_token_count * loss scale
+                           (distributed_block_diffusion_loss,
+                           dllm_parallel/core/models/backbones/nemotron/model.py:2084-2151).
   combine_vocab_shards     the MAX / SUM reductions over shards and the loss of
                            dllm_parallel/core/parallel/tensor_parallel/cross_entropy.py:238-252.
 
@@ -373,3 +377,60 @@ def dense_ce_topk_grad(hidden, weight, labels, top_ids, grad_loss, grad_probabil
     if grad_top_values is not None:
         g.scatter_add_(1, top_ids.to(torch.long), grad_top_values.to(dtype))
     return (g * dz) @ weight.to(dtype)
+
+
+def masked_token_loss(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    loss_weights: torch.Tensor,
+    valid_token_count: float,
+    *,
+    bias: Optional[torch.Tensor] = None,
+    exclude_index: Optional[int] = None,
+    output_multiplier: Optional[float] = None,
+    logit_softcap: Optional[float] = None,
+    loss_scale: float = 1.0,
+    dtype: torch.dtype = torch.float64,
+):
+    """``sum_r CE_r * w_r / valid_token_count * loss_scale`` over the rows whose
+    label is not -100, CE taken on ``hidden * output_multiplier``
+    (nemotron/model.py:2084-2086, :2099-2151).  The multiplication is done in
+    ``dtype`` (the reference rounds the product to the hidden dtype first)."""
+    h = hidden.reshape(-1, hidden.shape[-1]).to(dtype)
+    if output_multiplier is not None:
+        h = h * float(output_multiplier)
+    token_losses = dense_linear_ce(h, weight, labels.reshape(-1), bias=bias, reduction="none",
+                                   exclude_index=exclude_index, logit_softcap=logit_softcap,
+                                   dtype=dtype)
+    w = loss_weights.reshape(-1).to(dtype)
+    keep = labels.reshape(-1) != -100
+    loss_sum = (token_losses * torch.where(keep, w, torch.zeros_like(w))).sum()
+    return loss_sum / valid_token_count * float(loss_scale)
+
+
+def masked_token_loss_grads(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    loss_weights: torch.Tensor,
+    valid_token_count: float,
+    *,
+    bias: Optional[torch.Tensor] = None,
+    exclude_index: Optional[int] = None,
+    output_multiplier: Optional[float] = None,
+    logit_softcap: Optional[float] = None,
+    loss_scale: float = 1.0,
+    dtype: torch.dtype = torch.float64,
+):
+    """Analytic (grad_hidden, grad_weight, grad_bias) of ``masked_token_loss``:
+    the per-token scale is ``w_r / valid_token_count * loss_scale``; the chain
+    rule through ``hidden * output_multiplier`` multiplies grad_hidden by the
+    multiplier while grad_weight sees the multiplied hidden states."""
+    mult = 1.0 if output_multiplier is None else float(output_multiplier)
+    h = hidden.reshape(-1, hidden.shape[-1]).to(dtype) * mult
+    per_token = loss_weights.reshape(-1).to(dtype) / valid_token_count * float(loss_scale)
+    grad_scaled, grad_weight, grad_bias = dense_linear_ce_grads(
+        h, weight, labels.reshape(-1), per_token, bias=bias, reduction="none",
+        exclude_index=exclude_index, logit_softcap=logit_softcap, dtype=dtype)
+    return (grad_scaled * mult).reshape(hidden.shape), grad_weight, grad_bias

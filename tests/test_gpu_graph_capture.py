@@ -62,3 +62,70 @@ def test_forward_backward_graph_replays_match_eager(gpu_device, n, h, v):
         torch.cuda.synchronize()
         for name, a, b in zip(("losses", "grad_hidden", "grad_weight"), got, eager):
             assert torch.equal(a, b), (replay, name)
+
+
+@pytest.mark.parametrize("n,h,v", [(700, 128, 1536), (260, 72, 1025)])
+def test_whole_loss_with_device_row_count_replays_for_any_mask(gpu_device, n, h, v):
+    """Compaction, fused gather, forward and backward of the masked-token loss in
+    ONE graph: the count of loss-bearing rows never leaves the device, so the
+    same graph serves masks with different counts (down to none at all).  Every
+    replay is compared bit for bit with an eager run of the same calls and, for
+    the weighted sum, with the synchronising path."""
+    print("[case] whole-loss graph capture", n, h, v, flush=True)
+    dev = gpu_device
+    gen = torch.Generator().manual_seed(n + 1)
+    weight = (torch.randn(v, h, generator=gen) * 0.2).bfloat16().to(dev)
+    go = torch.full((1,), 0.5, device=dev)
+    kw = dict(ignore_index=-100, exclude_index=3, logit_softcap=0.0, logit_multiplier=0.5)
+
+    def make(rate):
+        hidden = torch.randn(n, h, generator=gen).bfloat16()
+        labels = torch.randint(4, v, (n,), generator=gen)
+        labels[torch.rand(n, generator=gen) < rate] = -100
+        weights = torch.rand(n, generator=gen) + 0.5
+        return hidden, labels, weights
+
+    def run(hidden, labels, weights):
+        row_idx, count = native.compact_rows_device(labels, -100)
+        rows, targets, w = native.gather_loss_rows(hidden, labels, weights, row_idx, count, -100)
+        _, lse, _, total = native.masked_loss_forward(
+            rows, weight, None, targets, w, m=n, row_idx=row_idx, row_count=count, n_out=n,
+            want_losses=False, want_sum=True, **kw)
+        dh, dw, _ = native.masked_loss_backward(
+            rows, weight, None, targets, w, lse, None, go, reduction="sum", m=n,
+            row_idx=row_idx, row_count=count, n_out=n, **kw)
+        return total, dh, dw, count
+
+    static = [torch.zeros(n, h, dtype=torch.bfloat16, device=dev),
+              torch.zeros(n, dtype=torch.long, device=dev),
+              torch.zeros(n, dtype=torch.float32, device=dev)]
+    first = make(0.5)
+    for s, t in zip(static, first):
+        s.copy_(t)
+    run(*static)                                  # warm-up: one-time kernel attributes
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outputs = run(*static)
+    torch.cuda.synchronize()
+
+    for replay, rate in enumerate((0.5, 0.05, 0.97, 1.0, 0.0)):
+        case = first if replay == 0 else make(rate)
+        for s, t in zip(static, case):
+            s.copy_(t)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outputs]
+        eager = run(*[t.to(dev) for t in case])   # eager work between replays
+        torch.cuda.synchronize()
+        assert int(got[3]) == int((case[1] != -100).sum()), replay
+        for name, a, b in zip(("weighted_sum", "grad_hidden", "grad_weight", "count"), got, eager):
+            assert torch.equal(a, b), (replay, rate, name)
+        # the synchronising path (exact launch sizes) computes the same sum
+        hidden, labels, weights = (t.to(dev) for t in case)
+        idx, m = native.compact_rows(labels, -100)
+        _, _, _, total = native.masked_loss_forward(
+            native.gather_rows(hidden, idx), weight, None, native.gather_rows(labels, idx),
+            native.gather_rows(weights, idx), row_idx=idx if m < n else None, n_out=n,
+            want_losses=False, want_sum=True, **kw)
+        assert torch.equal(total, got[0]), (replay, rate)

@@ -1,0 +1,253 @@
+"""GPU parity of the callers around the operator: the masked-token loss method
+(nemotron/model.py:2046-2151), the per-token variant (:1866-1902) and the
+output head's ``parallel_cross_entropy`` (tensor_parallel/layers.py:326-350),
+against the oracle on the scaled benchmark configurations.
+
+Bars as everywhere: loss within 1e-3 relative, gradients within 2e-2 relative
+max-norm (bf16 inputs).  All three compaction modes of the device path are
+covered; in "device" mode nothing reads the row count back to the host.
+"""
+
+import pytest
+import torch
+from torch import nn
+
+import linear_ce_oracle as oracle
+from turbo_dllm_amd import chunked_linear_ce_native as native
+from turbo_dllm_amd import workloads
+from turbo_dllm_amd.layers import VocabParallelLinear
+from turbo_dllm_amd.loss import (masked_token_loss, native_token_cross_entropy,
+                                 zero_loss_with_module_parameters)
+from turbo_dllm_amd.tiled_linear_cross_entropy import (COMPACTION_MODES, compaction_mode,
+                                                       tiled_linear_cross_entropy)
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-3
+GRAD_REL_MAX = 2e-2
+
+
+def say(*parts):
+    print("[case]", *parts, flush=True)
+
+
+def make_head(weight, bias, dev):
+    v, h = weight.shape
+    head = VocabParallelLinear(h, v, bias=bias is not None)
+    head = head.to(device=dev, dtype=weight.dtype)
+    with torch.no_grad():
+        head.weight.copy_(weight.to(dev))
+        if bias is not None:
+            head.bias.copy_(bias.to(dev))
+    return head
+
+
+def check_masked_loss(dev, wl, *, mode, multiplier=None, exclude=None, bias=None, count=None,
+                      scale=1.0, head_kind="vocab_parallel"):
+    gen = torch.Generator().manual_seed(wl.seed + 100)
+    labels = wl.labels.clone()
+    if exclude is not None:
+        labels[labels == exclude] = (exclude + 1) % wl.weight.shape[0]
+    weights = torch.rand(labels.shape, generator=gen) + 0.25
+    count = float((labels != -100).sum()) if count is None else count
+    if head_kind == "vocab_parallel":
+        head = make_head(wl.weight, bias, dev)
+    else:
+        head = nn.Linear(wl.weight.shape[1], wl.weight.shape[0], bias=bias is not None)
+        head = head.to(device=dev, dtype=wl.weight.dtype)
+        with torch.no_grad():
+            head.weight.copy_(wl.weight.to(dev))
+            if bias is not None:
+                head.bias.copy_(bias.to(dev))
+    hidden = wl.hidden.to(dev).requires_grad_(True)
+    with compaction_mode(mode):
+        loss = masked_token_loss(
+            hidden, labels.to(dev), weights.to(dev), head, valid_token_count=count,
+            mask_token_id=exclude, exclude_mask_token=exclude is not None,
+            output_multiplier=multiplier, logit_softcap=wl.logit_softcap, loss_scale=scale)
+        loss.backward()
+    torch.cuda.synchronize()
+    kw = dict(bias=bias, exclude_index=exclude, output_multiplier=multiplier,
+              logit_softcap=wl.logit_softcap, loss_scale=scale, dtype=torch.float32)
+    ref = oracle.masked_token_loss(wl.hidden, wl.weight, labels, weights, count, **kw)
+    rdh, rdw, rdb = oracle.masked_token_loss_grads(wl.hidden, wl.weight, labels, weights, count,
+                                                   **kw)
+    assert loss.dtype == torch.float32 and loss.dim() == 0
+    rel = abs(float(loss.detach()) - float(ref)) / max(abs(float(ref)), 1e-12)
+    err_h = oracle.relative_max_error(hidden.grad.cpu(), rdh)
+    err_w = oracle.relative_max_error(head.weight.grad.cpu(), rdw)
+    say(f"  loss {float(loss.detach()):.7f} oracle {float(ref):.7f} rel {rel:.2e}  dH {err_h:.2e}  "
+        f"dW {err_w:.2e}")
+    assert rel <= LOSS_RTOL and err_h <= GRAD_REL_MAX and err_w <= GRAD_REL_MAX
+    ignored = torch.nonzero(labels.reshape(-1) == -100).flatten()
+    assert torch.count_nonzero(hidden.grad.cpu().reshape(-1, hidden.shape[-1])[ignored]) == 0
+    if bias is not None:
+        assert oracle.relative_max_error(head.bias.grad.cpu(), rdb) <= GRAD_REL_MAX
+
+
+@pytest.mark.parametrize("mode", COMPACTION_MODES)
+@pytest.mark.parametrize("name", ["block_diffusion_shard", "gemma_softcap_head"])
+def test_masked_token_loss_on_scaled_configurations(gpu_device, name, mode):
+    wl = workloads.CONFIGS[name](seed=5, scale=16)
+    say("masked_token_loss", name, mode, "N", wl.n_rows, "M", wl.n_loss_rows)
+    check_masked_loss(gpu_device, wl, mode=mode, multiplier=0.5, exclude=7, count=wl.n_rows / 3.0,
+                      scale=4.0)
+
+
+@pytest.mark.parametrize("mode", ["sync", "device"])
+def test_masked_token_loss_with_bias_and_plain_linear_head(gpu_device, mode):
+    wl = workloads.small_head(seed=6, scale=8)
+    bias = (torch.randn(wl.weight.shape[0], generator=torch.Generator().manual_seed(9)) * 0.5
+            ).to(wl.weight.dtype)
+    say("masked_token_loss bias", mode)
+    check_masked_loss(gpu_device, wl, mode=mode, multiplier=2.0, bias=bias, head_kind="linear")
+    check_masked_loss(gpu_device, wl, mode=mode, multiplier=None, bias=bias)
+
+
+@pytest.mark.parametrize("dtype,h,v", [(torch.float32, 33, 517), (torch.bfloat16, 72, 1025),
+                                       (torch.float16, 128, 2048)])
+@pytest.mark.parametrize("mode", ["sync", "device"])
+def test_masked_token_loss_on_every_engine(gpu_device, dtype, h, v, mode):
+    # float32 / odd hidden sizes use the generic and register-staged engines and the
+    # transposed-copy gradient path; all of them must honour the device row count
+    gen = torch.Generator().manual_seed(21)
+    n = 300
+    hidden = torch.randn(n, h, generator=gen).to(dtype)
+    weight = (torch.randn(v, h, generator=gen) * 0.2).to(dtype)
+    labels = torch.randint(0, v, (n,), generator=gen)
+    labels[torch.rand(n, generator=gen) < 0.6] = -100
+    wl = workloads.Workload("engine_case", hidden, weight, labels, seed=21)
+    say("masked_token_loss engines", dtype, h, v, mode, "M", wl.n_loss_rows)
+    check_masked_loss(gpu_device, wl, mode=mode, multiplier=1.5)
+
+
+@pytest.mark.parametrize("mode", ["sync", "device"])
+def test_empty_rank_keeps_its_graph(gpu_device, mode):
+    """No supervised token: the loss is an exact zero that still reaches the
+    hidden states and the head (core/models/loss.py:13-31)."""
+    dev = gpu_device
+    say("masked_token_loss without loss-bearing rows", mode)
+    wl = workloads.small_head(seed=7, scale=16)
+    head = make_head(wl.weight, None, dev)
+    hidden = wl.hidden.to(dev).requires_grad_(True)
+    labels = torch.full(wl.labels.shape, -100, device=dev)
+    with compaction_mode(mode):
+        loss = masked_token_loss(hidden, labels, torch.ones(labels.shape, device=dev), head,
+                                 valid_token_count=1.0, output_multiplier=0.5)
+        loss.backward()
+    torch.cuda.synchronize()
+    assert float(loss) == 0.0
+    assert hidden.grad is not None and torch.count_nonzero(hidden.grad) == 0
+    assert head.weight.grad is not None and torch.count_nonzero(head.weight.grad) == 0
+    zero = zero_loss_with_module_parameters(hidden, head)
+    assert float(zero) == 0.0 and zero.requires_grad
+
+
+@pytest.mark.parametrize("name", ["block_diffusion_shard", "gemma_softcap_head"])
+def test_parallel_cross_entropy_of_the_output_head(gpu_device, name):
+    """VocabParallelLinear.parallel_cross_entropy (TP=1): reduction "none" by
+    default, dtype = x.dtype, vocab-first weight."""
+    dev = gpu_device
+    wl = workloads.CONFIGS[name](seed=8, scale=16)
+    say("parallel_cross_entropy", name, "N", wl.n_rows, "M", wl.n_loss_rows)
+    bias = (torch.randn(wl.weight.shape[0], generator=torch.Generator().manual_seed(3)) * 0.3
+            ).to(wl.weight.dtype)
+    head = make_head(wl.weight, bias, dev)
+    x = wl.hidden.to(dev).requires_grad_(True)
+    gen = torch.Generator().manual_seed(4)
+    go = torch.rand(wl.labels.shape, generator=gen)
+    losses = head.parallel_cross_entropy(x, wl.labels.to(dev), exclude_index=11,
+                                         logit_softcap=wl.logit_softcap)
+    assert losses.shape == wl.labels.shape and losses.dtype == torch.float32
+    losses.backward(go.to(dev))
+    torch.cuda.synchronize()
+    labels = wl.labels.clone()
+    ref = oracle.dense_linear_ce(wl.hidden, wl.weight, labels, bias=bias, reduction="none",
+                                 exclude_index=11, logit_softcap=wl.logit_softcap,
+                                 dtype=torch.float32)
+    # rows labelled with the excluded column are outside the dense expression
+    ok = labels != 11
+    torch.testing.assert_close(losses.cpu()[ok], ref[ok], rtol=LOSS_RTOL, atol=1e-4)
+    rdh, rdw, rdb = oracle.dense_linear_ce_grads(wl.hidden, wl.weight, labels, go, bias=bias,
+                                                 reduction="none", exclude_index=11,
+                                                 logit_softcap=wl.logit_softcap,
+                                                 dtype=torch.float32)
+    assert oracle.relative_max_error(x.grad.cpu(), rdh) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(head.weight.grad.cpu(), rdw) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(head.bias.grad.cpu(), rdb) <= GRAD_REL_MAX
+    mean = head.parallel_cross_entropy(x.detach(), wl.labels.to(dev), reduction="mean",
+                                       logit_softcap=wl.logit_softcap)
+    ref_mean = oracle.dense_linear_ce(wl.hidden, wl.weight, labels, bias=bias, reduction="mean",
+                                      logit_softcap=wl.logit_softcap, dtype=torch.float32)
+    assert abs(float(mean) - float(ref_mean)) <= LOSS_RTOL * abs(float(ref_mean))
+
+
+def test_native_token_cross_entropy_folds_the_multiplier(gpu_device):
+    dev = gpu_device
+    wl = workloads.gemma_softcap_head(seed=9, scale=32)
+    keep = torch.nonzero(wl.labels != -100).flatten()
+    hidden, labels = wl.hidden[keep], wl.labels[keep]          # callers compact first
+    say("native_token_cross_entropy", "M", labels.numel())
+    head = make_head(wl.weight, None, dev)
+    x = hidden.to(dev).requires_grad_(True)
+    losses = native_token_cross_entropy(x, labels.to(dev), head, output_multiplier=0.75,
+                                        logit_softcap=wl.logit_softcap)
+    go = torch.rand(labels.shape, generator=torch.Generator().manual_seed(5))
+    losses.backward(go.to(dev))
+    torch.cuda.synchronize()
+    ref = oracle.dense_linear_ce(hidden.float() * 0.75, wl.weight, labels, reduction="none",
+                                 logit_softcap=wl.logit_softcap, dtype=torch.float32)
+    torch.testing.assert_close(losses.cpu(), ref, rtol=LOSS_RTOL, atol=1e-4)
+    rdh, rdw, _ = oracle.masked_token_loss_grads(hidden, wl.weight, labels, go, 1.0,
+                                                 output_multiplier=0.75,
+                                                 logit_softcap=wl.logit_softcap,
+                                                 dtype=torch.float32)
+    assert oracle.relative_max_error(x.grad.cpu(), rdh) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(head.weight.grad.cpu(), rdw) <= GRAD_REL_MAX
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum", "none"])
+@pytest.mark.parametrize("mode", ["device", "none"])
+def test_loss_api_compaction_modes_agree_with_the_oracle(gpu_device, mode, reduction):
+    """tiled_linear_cross_entropy without a host read-back of the row count
+    ("device") and without compaction ("none")."""
+    dev = gpu_device
+    wl = workloads.qwen3_8b_head(seed=10, scale=16, h=512)
+    say("loss API", mode, reduction, "N", wl.n_rows, "M", wl.n_loss_rows)
+    hidden = wl.hidden.to(dev).requires_grad_(True)
+    weight = wl.weight.to(dev).requires_grad_(True)
+    go = None
+    if reduction == "none":
+        go = torch.rand(wl.labels.shape, generator=torch.Generator().manual_seed(6))
+    with compaction_mode(mode):
+        loss = tiled_linear_cross_entropy(hidden, weight, wl.labels.to(dev), reduction=reduction,
+                                          dtype=torch.bfloat16, weight_layout="vocab_first")
+        loss.backward(None if go is None else go.to(dev))
+    torch.cuda.synchronize()
+    ref = oracle.dense_linear_ce(wl.hidden, wl.weight, wl.labels, reduction=reduction,
+                                 dtype=torch.float32)
+    torch.testing.assert_close(loss.cpu(), ref, rtol=LOSS_RTOL, atol=1e-4)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(wl.hidden, wl.weight, wl.labels, go,
+                                               reduction=reduction, dtype=torch.float32)
+    assert oracle.relative_max_error(hidden.grad.cpu(), rdh) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(weight.grad.cpu(), rdw) <= GRAD_REL_MAX
+
+
+def test_device_row_count_forward_is_bit_equal_to_the_exact_plan(gpu_device):
+    """With the count on the device the kernels re-derive the exact plan, so
+    per-token losses equal those of the synchronising path bit for bit."""
+    dev = gpu_device
+    wl = workloads.block_diffusion_shard(seed=11, scale=16, h=256)
+    say("device row count vs exact plan", "N", wl.n_rows, "M", wl.n_loss_rows)
+    hidden, weight, labels = wl.hidden.to(dev), wl.weight.to(dev), wl.labels.to(dev)
+    outs = {}
+    for mode in ("sync", "device"):
+        with compaction_mode(mode):
+            outs[mode] = tiled_linear_cross_entropy(hidden, weight, labels, reduction="none",
+                                                    dtype=torch.bfloat16,
+                                                    weight_layout="vocab_first")
+    torch.cuda.synchronize()
+    assert torch.equal(outs["sync"], outs["device"])
+    idx, count = native.compact_rows_device(labels, -100)
+    assert int(count) == wl.n_loss_rows
+    assert idx[: wl.n_loss_rows].cpu().tolist() == oracle.compact_rows(wl.labels.numpy()).tolist()

@@ -345,3 +345,108 @@ def test_ce_topk_oracle_orders_ties_by_id():
                           dtype=torch.float64)
     _, _, vals, ids, _ = oracle.dense_ce_topk(hidden, weight, torch.tensor([0]), 4)
     assert ids.tolist() == [[1, 3, 0, 2]] and vals.tolist() == [[3.0, 3.0, 2.0, 2.0]]
+
+
+def test_rounded_logit_gradient_brute_force():
+    """round_grad_logits pinned exactly: every logit gradient is formed with
+    Python floats, rounded element by element to bfloat16 (torch's scalar
+    conversion, a routine the oracle does not use), and contracted by loops."""
+    torch.manual_seed(12)
+    n, h, v = 5, 4, 7
+    hidden = torch.randn(n, h).bfloat16()
+    weight = (torch.randn(v, h) * 0.5).bfloat16()
+    labels = torch.tensor([3, -100, 0, 6, 2])
+    valid = [y for y in labels.tolist() if y != -100]
+    dh = [[0.0] * h for _ in range(n)]
+    dw = [[0.0] * h for _ in range(v)]
+    for r in range(n):
+        y = int(labels[r])
+        if y == -100:
+            continue
+        z = [sum(float(hidden[r, k]) * float(weight[c, k]) for k in range(h)) for c in range(v)]
+        zmax = max(z)
+        denom = sum(math.exp(x - zmax) for x in z)
+        for c in range(v):
+            g = (math.exp(z[c] - zmax) / denom - (1.0 if c == y else 0.0)) / len(valid)
+            g = float(torch.tensor(g, dtype=torch.float64).to(torch.bfloat16))   # the rounding point
+            for k in range(h):
+                dh[r][k] += g * float(weight[c, k])
+                dw[c][k] += g * float(hidden[r, k])
+    got_dh, got_dw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, reduction="mean",
+                                                     round_grad_logits=torch.bfloat16)
+    torch.testing.assert_close(got_dh, torch.tensor(dh, dtype=torch.float64), atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(got_dw, torch.tensor(dw, dtype=torch.float64), atol=1e-12, rtol=1e-10)
+    # rounding after the contraction instead (a wrong rounding point) is not the same thing
+    exact = oracle.dense_linear_ce_grads(hidden, weight, labels, reduction="mean")
+    assert not torch.equal(got_dh, exact[0].bfloat16().double())
+
+
+@pytest.mark.parametrize("softcap", [None, 5.0])
+def test_dim_first_head_matches_library_cross_entropy_and_autograd(softcap):
+    """weight_dim_first=True pinned against F.cross_entropy(hidden @ weight) and
+    autograd through it (the [H, V] head multiplies without a transpose)."""
+    torch.manual_seed(13)
+    n, h, v = 9, 6, 11
+    hidden = torch.randn(n, h, dtype=torch.float64, requires_grad=True)
+    weight = (torch.randn(h, v, dtype=torch.float64) * 0.7).requires_grad_(True)
+    bias = torch.randn(v, dtype=torch.float64, requires_grad=True)
+    labels = torch.randint(0, v, (n,))
+    labels[2] = -100
+    logits = hidden @ weight + bias
+    if softcap:
+        logits = torch.tanh(logits / softcap) * softcap
+    ref = F.cross_entropy(logits, labels, ignore_index=-100, reduction="sum")
+    ref.backward()
+    got = oracle.dense_linear_ce(hidden.detach(), weight.detach(), labels, bias=bias.detach(),
+                                 reduction="sum", logit_softcap=softcap, weight_dim_first=True)
+    torch.testing.assert_close(got, ref.detach(), atol=1e-12, rtol=1e-12)
+    dh, dw, db = oracle.dense_linear_ce_grads(hidden.detach(), weight.detach(), labels,
+                                              bias=bias.detach(), reduction="sum",
+                                              logit_softcap=softcap, weight_dim_first=True)
+    assert dw.shape == weight.shape
+    torch.testing.assert_close(dh, hidden.grad, atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(dw, weight.grad, atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(db, bias.grad, atol=1e-12, rtol=1e-10)
+
+
+@pytest.mark.parametrize("multiplier,softcap,exclude", [(None, None, None), (0.25, None, 4),
+                                                        (3.0, 8.0, None), (0.5, 6.0, 2)])
+def test_masked_token_loss_oracle_matches_library_expression(multiplier, softcap, exclude):
+    """The loss-method restatement against the sequence of library calls the
+    reference makes (nemotron/model.py:2084-2151: scaled hidden states, logits,
+    soft cap, -inf on the mask token, F.cross_entropy(reduction='none'), weights,
+    / valid_token_count * scale) and autograd through it."""
+    torch.manual_seed(14)
+    n, h, v = 12, 5, 9
+    hidden = torch.randn(n, h, dtype=torch.float64, requires_grad=True)
+    weight = (torch.randn(v, h, dtype=torch.float64) * 0.6).requires_grad_(True)
+    bias = torch.randn(v, dtype=torch.float64, requires_grad=True)
+    labels = torch.randint(0, v, (n,))
+    if exclude is not None:
+        labels[labels == exclude] = (exclude + 1) % v
+    labels[[1, 7]] = -100
+    weights = torch.rand(n, dtype=torch.float64) + 0.1
+    count, scale = 7.0, 2.0
+    rows = torch.nonzero(labels != -100).flatten()
+    active = hidden.index_select(0, rows)
+    if multiplier is not None:
+        active = active * multiplier
+    logits = active @ weight.t() + bias
+    if softcap:
+        logits = torch.tanh(logits / softcap) * softcap
+    if exclude is not None:
+        logits = logits.clone()
+        logits[:, exclude] = -float("inf")
+    token_losses = F.cross_entropy(logits, labels[rows], ignore_index=-100, reduction="none")
+    ref = (token_losses * weights[rows]).sum() / count * scale
+    ref.backward()
+    kw = dict(bias=bias.detach(), exclude_index=exclude, output_multiplier=multiplier,
+              logit_softcap=softcap, loss_scale=scale)
+    got = oracle.masked_token_loss(hidden.detach(), weight.detach(), labels, weights, count, **kw)
+    torch.testing.assert_close(got, ref.detach(), atol=1e-12, rtol=1e-12)
+    dh, dw, db = oracle.masked_token_loss_grads(hidden.detach(), weight.detach(), labels, weights,
+                                                count, **kw)
+    torch.testing.assert_close(dh, hidden.grad, atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(dw, weight.grad, atol=1e-12, rtol=1e-10)
+    torch.testing.assert_close(db, bias.grad, atol=1e-12, rtol=1e-10)
+    assert torch.count_nonzero(dh[[1, 7]]) == 0

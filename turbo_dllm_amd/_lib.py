@@ -33,6 +33,14 @@ SIGNATURES = {
     "tlce_gather_rows": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "tlce_scatter_rows": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "tlce_fill_zero": (c_int, [c_void_p, c_int64, c_void_p]),
+    "tlce_gather_loss_rows": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden labels weights row_idx count
+            c_int64, c_int64, c_int64, c_int64,                 # capacity padded_rows row_bytes ignore
+            c_void_p, c_void_p, c_void_p, c_void_p,             # hidden_dst labels_dst weights_dst stream
+        ],
+    ),
     "tlce_forward_workspace_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int]),
     "tlce_forward": (
         c_int,
@@ -65,6 +73,32 @@ SIGNATURES = {
             c_void_p, c_void_p, c_void_p,                       # lse valid_count grad_output
             c_int64, c_int64, c_int64, c_int64, c_int,          # m n_out h v dtype
             c_int, c_int64, c_int64, c_float,                   # reduction ignore exclude softcap
+            c_void_p, c_void_p, c_void_p,                       # grad_hidden grad_weight grad_bias
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
+    "tlce_masked_loss_forward_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int, c_int]
+    ),
+    "tlce_masked_loss_forward": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden weight bias labels weights
+            c_void_p, c_void_p,                                 # row_idx row_count
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m n_out h v dtype
+            c_int64, c_int64, c_float, c_float,                 # ignore exclude softcap multiplier
+            c_void_p, c_void_p, c_void_p, c_void_p,             # losses lse valid_count weighted_sum
+            c_void_p, c_int64, c_void_p,                        # workspace bytes stream
+        ],
+    ),
+    "tlce_masked_loss_backward": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden weight bias labels weights
+            c_void_p, c_void_p,                                 # row_idx row_count
+            c_void_p, c_void_p, c_void_p,                       # lse valid_count grad_output
+            c_int64, c_int64, c_int64, c_int64, c_int, c_int,   # m n_out h v dtype reduction
+            c_int64, c_int64, c_float, c_float,                 # ignore exclude softcap multiplier
             c_void_p, c_void_p, c_void_p,                       # grad_hidden grad_weight grad_bias
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],

@@ -117,6 +117,69 @@ def compact_rows(labels: torch.Tensor, ignore_index: int) -> tuple[torch.Tensor,
     return row_idx[:m], m
 
 
+def compact_rows_device(labels: torch.Tensor, ignore_index: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """As ``compact_rows`` without the host read-back: returns the index buffer
+    at full length ``n`` (only its first ``count`` entries are defined) and the
+    count as a device int64 tensor of one element.  Nothing here synchronises,
+    so the call can be recorded into a HIP graph."""
+    device = _require_device(labels)
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    n = labels.numel()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        row_idx = torch.empty(max(n, 1), dtype=torch.long, device=device)
+        count = torch.empty(1, dtype=torch.long, device=device)
+        ws = _workspace(lib.tlce_compact_workspace_bytes(n), device)
+        _lib.check(
+            lib.tlce_compact_rows(
+                _ptr(labels), n, int(ignore_index), row_idx.data_ptr(), count.data_ptr(),
+                ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_compact_rows",
+        )
+    return row_idx[:n], count
+
+
+def gather_loss_rows(
+    hidden: torch.Tensor,
+    labels: torch.Tensor,
+    weights: torch.Tensor | None,
+    row_idx: torch.Tensor,
+    row_count: torch.Tensor,
+    ignore_index: int,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
+    """Hidden rows, labels and (optional) float32 loss weights of the first
+    ``row_count`` positions in ``row_idx``, gathered in one launch with the
+    count read on the device.  The outputs have ``round_up(n, 64)`` rows; rows
+    from the count up to the next multiple of 64 are zero / ignored / weight 0."""
+    device = _require_device(hidden, labels, weights, row_idx, row_count)
+    hidden = hidden.contiguous()
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    n, h = hidden.shape
+    if labels.numel() != n or row_idx.numel() != n:
+        raise RuntimeError("gather_loss_rows: hidden, labels and row_idx lengths differ")
+    if weights is not None:
+        weights = weights.reshape(-1).to(torch.float32).contiguous()
+        if weights.numel() != n:
+            raise RuntimeError("gather_loss_rows: weights length differs")
+    padded = (n + 63) // 64 * 64
+    row_bytes = h * hidden.element_size()
+    with torch.cuda.device(device):
+        rows = torch.empty((padded, h), dtype=hidden.dtype, device=device)
+        targets = torch.empty(padded, dtype=torch.long, device=device)
+        w = None if weights is None else torch.empty(padded, dtype=torch.float32, device=device)
+        if n:
+            _lib.check(
+                _lib.library().tlce_gather_loss_rows(
+                    hidden.data_ptr(), labels.data_ptr(), _ptr(weights), row_idx.data_ptr(),
+                    row_count.data_ptr(), n, padded, row_bytes, int(ignore_index),
+                    rows.data_ptr(), targets.data_ptr(), _ptr(w), _stream(device),
+                ),
+                "tlce_gather_loss_rows",
+            )
+    return rows, targets, w
+
+
 def gather_rows(src: torch.Tensor, row_idx: torch.Tensor) -> torch.Tensor:
     """``src.index_select(0, row_idx)`` for a contiguous ``src`` (any trailing shape)."""
     device = _require_device(src, row_idx)
@@ -344,6 +407,159 @@ def backward_frozen_weight(
         logit_softcap=logit_softcap, weight_dim_first=weight_dim_first,
         compute_weight_grad=False, row_idx=row_idx, n_out=n_out,
     )
+
+
+# ---------------------------------------------------------- masked-token loss --
+def masked_loss_forward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    labels: torch.Tensor,
+    token_weights: torch.Tensor | None,
+    *,
+    m: int | None = None,
+    row_idx: torch.Tensor | None = None,
+    row_count: torch.Tensor | None = None,
+    n_out: int | None = None,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+    logit_multiplier: float = 1.0,
+    want_losses: bool = True,
+    want_sum: bool = True,
+) -> tuple[torch.Tensor | None, torch.Tensor, torch.Tensor, torch.Tensor | None]:
+    """The forward with the loss method's arithmetic folded in
+    (distributed_block_diffusion_loss, nemotron/model.py:2084-2151): logits
+    scaled by ``logit_multiplier`` instead of a scaled copy of ``hidden``, and
+    ``weighted_sum = sum_r token_weights[r] * loss_r`` formed on the device.
+
+    ``hidden`` [>= m, H] (vocab-first ``weight`` [V, H]); ``m`` defaults to
+    ``hidden.shape[0]``.  With ``row_count`` (device int64 [1]) ``m`` is only the
+    capacity: rows past the count carry no loss and the call never synchronises;
+    ``hidden`` must then hold ``round_up(m, 64)`` rows (``gather_loss_rows``
+    provides them).  Returns ``(losses [n_out] | None, lse [m], valid_count [1],
+    weighted_sum [1] | None)``, all float32.
+    """
+    device = _require_device(hidden, weight, bias, labels, token_weights, row_idx, row_count)
+    if hidden.dim() != 2 or weight.dim() != 2 or weight.shape[1] != hidden.shape[1]:
+        raise RuntimeError("masked loss expects hidden [N, D] and weight [V, D]")
+    if weight.dtype != hidden.dtype:
+        raise RuntimeError("native linear CE expects hidden and weight of one dtype")
+    if not (want_losses or want_sum):
+        raise RuntimeError("masked loss: nothing to compute")
+    hidden = hidden.contiguous()
+    weight = weight.contiguous()
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    h = hidden.shape[1]
+    v = weight.shape[0]
+    m = hidden.shape[0] if m is None else int(m)
+    need_rows = (m + 63) // 64 * 64 if row_count is not None else m
+    if hidden.shape[0] < need_rows or labels.numel() < m:
+        raise RuntimeError("masked loss: hidden / labels hold fewer rows than m")
+    n_out = m if n_out is None else int(n_out)
+    bias32 = None if bias is None else bias.to(torch.float32).contiguous()
+    if token_weights is not None:
+        token_weights = token_weights.reshape(-1).to(torch.float32).contiguous()
+        if token_weights.numel() < m:
+            raise RuntimeError("masked loss: token_weights holds fewer entries than m")
+    lib = _lib.library()
+    code = _dtype_code(hidden)
+    with torch.cuda.device(device):
+        losses = torch.empty(n_out, dtype=torch.float32, device=device) if want_losses else None
+        lse = torch.empty(m, dtype=torch.float32, device=device)
+        valid_count = torch.empty(1, dtype=torch.float32, device=device)
+        weighted_sum = torch.empty(1, dtype=torch.float32, device=device) if want_sum else None
+        ws = _workspace(
+            lib.tlce_masked_loss_forward_workspace_bytes(m, h, v, code, int(row_count is not None)),
+            device,
+        )
+        _lib.check(
+            lib.tlce_masked_loss_forward(
+                _ptr(hidden), _ptr(weight), _ptr(bias32), _ptr(labels), _ptr(token_weights),
+                _ptr(row_idx), _ptr(row_count), m, n_out, h, v, code,
+                int(ignore_index), int(exclude_index), float(logit_softcap),
+                float(logit_multiplier),
+                _ptr(losses), _ptr(lse), valid_count.data_ptr(), _ptr(weighted_sum),
+                ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_masked_loss_forward",
+        )
+    return losses, lse, valid_count, weighted_sum
+
+
+def masked_loss_backward(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: torch.Tensor | None,
+    labels: torch.Tensor,
+    token_weights: torch.Tensor | None,
+    lse: torch.Tensor,
+    valid_count: torch.Tensor | None,
+    grad_output: torch.Tensor,
+    *,
+    reduction: str = "sum",
+    m: int | None = None,
+    row_idx: torch.Tensor | None = None,
+    row_count: torch.Tensor | None = None,
+    n_out: int | None = None,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+    logit_multiplier: float = 1.0,
+    compute_weight_grad: bool = True,
+) -> tuple[torch.Tensor, torch.Tensor | None, torch.Tensor | None]:
+    """Gradients of ``masked_loss_forward``.  ``reduction="sum"`` with
+    ``grad_output`` [1] is the gradient of ``weighted_sum``; "none" / "mean" take
+    the gradient of the per-token losses / of their mean, as ``backward`` does,
+    with ``token_weights`` applied on top.  Returns ``(grad_hidden [n_out, H],
+    grad_weight | None, grad_bias | None)`` in the input dtypes."""
+    device = _require_device(hidden, weight, bias, labels, token_weights, lse, valid_count,
+                             grad_output, row_idx, row_count)
+    hidden = hidden.contiguous()
+    weight = weight.contiguous()
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    h = hidden.shape[1]
+    v = weight.shape[0]
+    m = hidden.shape[0] if m is None else int(m)
+    n_out = m if n_out is None else int(n_out)
+    code = _dtype_code(hidden)
+    reduction_code = _reduction_code(reduction)
+    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
+    expected = n_out if reduction_code == _lib.REDUCTION_NONE else 1
+    if grad_output.numel() != expected:
+        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected {expected}")
+    bias32 = None if bias is None else bias.to(torch.float32).contiguous()
+    if token_weights is not None:
+        token_weights = token_weights.reshape(-1).to(torch.float32).contiguous()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        grad_hidden = torch.empty((n_out, h), dtype=hidden.dtype, device=device)
+        grad_weight = (
+            torch.empty((v, h), dtype=weight.dtype, device=device) if compute_weight_grad else None
+        )
+        grad_bias32 = (
+            torch.empty(v, dtype=torch.float32, device=device) if bias is not None else None
+        )
+        ws = _workspace(
+            lib.tlce_backward_workspace_bytes(
+                m, h, v, code, int(compute_weight_grad), int(bias is not None), PANEL_BYTES
+            ),
+            device,
+        )
+        _lib.check(
+            lib.tlce_masked_loss_backward(
+                _ptr(hidden), _ptr(weight), _ptr(bias32), _ptr(labels), _ptr(token_weights),
+                _ptr(row_idx), _ptr(row_count), _ptr(lse), _ptr(valid_count), _ptr(grad_output),
+                m, n_out, h, v, code, reduction_code,
+                int(ignore_index), int(exclude_index), float(logit_softcap),
+                float(logit_multiplier),
+                _ptr(grad_hidden), _ptr(grad_weight), _ptr(grad_bias32),
+                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_masked_loss_backward",
+        )
+    grad_bias = None if grad_bias32 is None else grad_bias32.to(bias.dtype)
+    return grad_hidden, grad_weight, grad_bias
 
 
 # ------------------------------------------------------------ vocabulary shards --

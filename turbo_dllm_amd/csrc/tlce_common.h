@@ -45,6 +45,17 @@ static inline int64_t align256(int64_t x) { return round_up(x, 256); }
 
 static inline int dtype_bytes(int dtype) { return dtype == TLCE_DTYPE_F32 ? 4 : 2; }
 
+// Forward launch shape: token tiles x vocabulary splits workgroups, at most (and
+// close to) four whole waves of 256 workgroups on a 256-CU MI355X.  Shared by
+// the host plan and by the kernels that derive the plan from a row count that
+// only the device knows.
+constexpr int kTargetWorkgroups = 1024;
+__host__ __device__ static inline int forward_vocab_splits(int n_ttiles, int n_vtiles) {
+  const int want = n_ttiles > 0 ? kTargetWorkgroups / n_ttiles : kTargetWorkgroups;
+  const int s = want < 1 ? 1 : want;
+  return s < n_vtiles ? s : n_vtiles;
+}
+
 constexpr int kXcds = 8;  // MI355X: 8 accelerator dies, workgroups dealt round-robin
 
 // ------------------------------------------------------------- device -------
@@ -57,6 +68,25 @@ constexpr int kXcds = 8;  // MI355X: 8 accelerator dies, workgroups dealt round-
 __device__ __forceinline__ int xcd_logical_block(int bid, int nblocks) {
   const int per = nblocks / kXcds;
   return (bid % kXcds) * per + (bid / kXcds);
+}
+
+// Rows of a call whose row count lives on the device: `m` is then the
+// capacity the launch was sized for and *m_dev (clamped to [0, m]) the real
+// count.  m_dev == null: m itself.
+__device__ __forceinline__ int effective_rows(int m, const int64_t* m_dev) {
+  if (m_dev == nullptr) return m;
+  const int64_t c = *m_dev;
+  return c < 0 ? 0 : (c < (int64_t)m ? (int)c : m);
+}
+
+// Logical block id when only the first `tiles` of the launched workgroups have
+// work (the launch was sized for more rows than there are): the same mapping a
+// launch of round_up(tiles, 8) workgroups would get; -1 for the others.
+__device__ __forceinline__ int xcd_logical_block_of(int bid, int tiles) {
+  const int total = (tiles + kXcds - 1) / kXcds * kXcds;
+  if (bid >= total) return -1;
+  const int logical = xcd_logical_block(bid, total);
+  return logical < tiles ? logical : -1;
 }
 
 // Grouped tile order: consecutive logical ids walk `group` tiles along i, then

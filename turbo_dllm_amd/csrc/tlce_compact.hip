@@ -112,6 +112,44 @@ __global__ __launch_bounds__(256) void scatter_rows_kernel(const V* __restrict__
   }
 }
 
+// Gather of everything the masked-token loss needs from its loss-bearing rows in
+// one launch, with the row count read on the device: for r < *row_count the
+// hidden row, label and loss weight of position row_idx[r]; the rows from
+// *row_count up to the next multiple of 64 (inside the destination's
+// padded_rows) become zero rows with the ignore label and weight 0, so that a
+// contraction over whole 64-row slabs of the gathered rows never meets
+// uninitialised memory.  One workgroup per destination row.
+template <typename V>
+__global__ __launch_bounds__(256) void gather_loss_rows_kernel(
+    const V* __restrict__ hidden_src, const int64_t* __restrict__ labels_src,
+    const float* __restrict__ weights_src, const int64_t* __restrict__ row_idx,
+    const int64_t* __restrict__ row_count, int64_t padded_rows, int vecs_per_row,
+    int64_t ignore, V* __restrict__ hidden_dst, int64_t* __restrict__ labels_dst,
+    float* __restrict__ weights_dst) {
+  const int64_t count = *row_count;
+  const int64_t fill_end = min(padded_rows, (count + 63) / 64 * 64);
+  for (int64_t r = blockIdx.x; r < fill_end; r += gridDim.x) {
+    V* dst = hidden_dst + r * vecs_per_row;
+    if (r < count) {
+      const int64_t s = row_idx[r];
+      const V* src = hidden_src + s * vecs_per_row;
+      for (int c = threadIdx.x; c < vecs_per_row; c += 256) dst[c] = src[c];
+      if (threadIdx.x == 0) {
+        labels_dst[r] = labels_src[s];
+        if (weights_dst != nullptr) weights_dst[r] = weights_src[s];
+      }
+    } else {
+      V z;
+      memset(&z, 0, sizeof(V));
+      for (int c = threadIdx.x; c < vecs_per_row; c += 256) dst[c] = z;
+      if (threadIdx.x == 0) {
+        labels_dst[r] = ignore;
+        if (weights_dst != nullptr) weights_dst[r] = 0.0f;
+      }
+    }
+  }
+}
+
 static int pick_vector_bytes(const void* a, const void* b, int64_t row_bytes) {
   const uintptr_t bits = (uintptr_t)a | (uintptr_t)b | (uintptr_t)row_bytes;
   if ((bits & 15) == 0) return 16;
@@ -200,4 +238,39 @@ extern "C" int tlce_gather_rows(const void* src, const int64_t* row_idx, int64_t
 extern "C" int tlce_scatter_rows(const void* src, const int64_t* row_idx, int64_t m,
                                  int64_t row_bytes, void* dst, void* stream) {
   return move_rows<false>(src, row_idx, m, row_bytes, dst, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlce_gather_loss_rows(const void* hidden_src, const int64_t* labels_src,
+                                     const float* weights_src, const int64_t* row_idx,
+                                     const int64_t* row_count, int64_t capacity,
+                                     int64_t padded_rows, int64_t row_bytes,
+                                     int64_t ignore_index, void* hidden_dst,
+                                     int64_t* labels_dst, float* weights_dst, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  TLCE_REQUIRE(capacity >= 0 && padded_rows >= capacity && row_bytes > 0,
+               "gather_loss_rows: bad sizes");
+  if (capacity == 0) return 0;
+  TLCE_REQUIRE(hidden_src && labels_src && row_idx && row_count && hidden_dst && labels_dst,
+               "gather_loss_rows: null pointer");
+  TLCE_REQUIRE((weights_src == nullptr) == (weights_dst == nullptr),
+               "gather_loss_rows: weights source and destination go together");
+  const int vb = pick_vector_bytes(hidden_src, hidden_dst, row_bytes);
+  const int64_t vpr = row_bytes / vb;
+  TLCE_REQUIRE(vpr <= INT32_MAX, "gather_loss_rows: row too long");
+  const int grid = (int)std::min<int64_t>(padded_rows, 256 * 32);
+#define TLCE_GATHER(V)                                                                      \
+  gather_loss_rows_kernel<V><<<grid, 256, 0, stream>>>(                                     \
+      static_cast<const V*>(hidden_src), labels_src, weights_src, row_idx, row_count,       \
+      padded_rows, (int)vpr, ignore_index, static_cast<V*>(hidden_dst), labels_dst,         \
+      weights_dst)
+  switch (vb) {
+    case 16: TLCE_GATHER(uint4); break;
+    case 8: TLCE_GATHER(uint2); break;
+    case 4: TLCE_GATHER(uint32_t); break;
+    case 2: TLCE_GATHER(uint16_t); break;
+    default: TLCE_GATHER(uint8_t); break;
+  }
+#undef TLCE_GATHER
+  TLCE_LAUNCH_CHECK();
+  return 0;
 }

@@ -74,7 +74,6 @@ struct ScopedTimer {
 };
 
 constexpr int64_t kDefaultPanelBytes = 1ll << 30;
-constexpr int kTargetWorkgroups = 1024;  // 4 per CU on a 256-CU MI355X
 
 struct Plan {
   int engine;   // 2 = direct-to-LDS MFMA, 1 = register-staged MFMA, 0 = generic
@@ -114,8 +113,7 @@ inline Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_gr
   p.n_htiles = (int)ceil_div(h, p.tile);
   // forward: token tiles x vocabulary splits workgroups, at most (and close to)
   // four whole waves of 256 workgroups
-  p.nsplit = (int)std::min<int64_t>(
-      p.n_vtiles, std::max<int64_t>(1, kTargetWorkgroups / p.n_ttiles));
+  p.nsplit = forward_vocab_splits(p.n_ttiles, p.n_vtiles);
   if (panel_bytes <= 0) panel_bytes = kDefaultPanelBytes;
   const int64_t col_bytes = p.mp * dtype_bytes(dtype) * ((weight_grad && !p.kmajor) ? 2 : 1);
   int64_t tiles_per_panel = std::max<int64_t>(1, panel_bytes / col_bytes / p.tile);
@@ -150,15 +148,34 @@ inline Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_gr
   return p;
 }
 
-struct ForwardLayout {
-  int64_t part_max, part_sum, total;
+// What the masked-token loss adds to the plain operator
+// (distributed_block_diffusion_loss, nemotron/model.py:2084-2151): the output
+// multiplier applied to the logits instead of to a copy of the hidden states,
+// per-row loss weights, the weighted loss sum, and a row count that stays on
+// the device (row_count != null: m is the capacity every launch is sized for).
+struct RowOptions {
+  float logit_scale = 1.0f;
+  const float* token_weights = nullptr;   // [m] float32, compacted order
+  const int64_t* row_count = nullptr;     // device int64
+  float* weighted_sum = nullptr;          // forward: [1] float32 out
 };
-inline ForwardLayout forward_layout(const Plan& p) {
+
+struct ForwardLayout {
+  int64_t part_max, part_sum, weighted, total;
+};
+// dynamic_rows: the partials must fit whatever plan the kernels derive from a
+// device-side row count <= m (at most kTargetWorkgroups tiles, or one split of
+// all token tiles); weighted: room for the per-row weighted losses.
+inline ForwardLayout forward_layout(const Plan& p, bool dynamic_rows = false,
+                                    bool weighted = false) {
   ForwardLayout l;
-  const int64_t part = align256((int64_t)p.nsplit * p.mp * 4);
+  int64_t floats = (int64_t)p.nsplit * p.mp;
+  if (dynamic_rows) floats = std::max<int64_t>((int64_t)kTargetWorkgroups * p.tile, p.mp);
+  const int64_t part = align256(floats * 4);
   l.part_max = 0;
   l.part_sum = part;
-  l.total = 2 * part;
+  l.weighted = 2 * part;
+  l.total = 2 * part + (weighted ? align256(p.mp * 4) : 0);
   return l;
 }
 
@@ -226,7 +243,13 @@ int launch_forward_variant(const Plan& p, const ForwardArgs& a, hipStream_t stre
   static LdsOptIn lds;
   if (int rc = enable_large_lds(lce_forward_stats_kernel<E, kSoftcap, kBias>, E::kSmemBytes, lds))
     return rc;
-  const int grid = xcd_grid((int64_t)p.n_ttiles * p.nsplit);
+  // with a device-side row count: the most tiles any row count <= m can plan
+  const int64_t tiles =
+      a.m_dev == nullptr
+          ? (int64_t)p.n_ttiles * p.nsplit
+          : std::min<int64_t>((int64_t)p.n_ttiles * p.n_vtiles,
+                              std::max<int64_t>(kTargetWorkgroups, p.n_ttiles));
+  const int grid = xcd_grid(tiles);
   ScopedTimer timer(kClassForwardStats, stream);
   lce_forward_stats_kernel<E, kSoftcap, kBias><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
@@ -281,12 +304,13 @@ int launch_gemm(GemmArgs a, int ksplit, int cls, hipStream_t stream) {
 
 template <typename T>
 int launch_transpose(const T* in, int64_t ld_in, int64_t rows, int64_t cols, T* out,
-                     int64_t ld_out, int64_t out_cols, hipStream_t stream) {
+                     int64_t ld_out, int64_t out_cols, hipStream_t stream,
+                     const int64_t* rows_dev = nullptr) {
   dim3 grid((unsigned)ceil_div(cols, 64), (unsigned)ceil_div(out_cols, 64), 1);
   TLCE_REQUIRE(grid.y <= 65535, "transpose: too many row tiles");
   ScopedTimer timer(kClassTranspose, stream);
   lce_transpose_pad_kernel<T><<<grid, 256, 0, stream>>>(in, ld_in, (int)rows, (int)cols, out,
-                                                        ld_out, (int)out_cols);
+                                                        ld_out, (int)out_cols, rows_dev);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
@@ -298,6 +322,7 @@ int launch_token_scale(const ScaleArgs& sa, hipStream_t stream);
 int launch_kl_finish(float* losses, const float* tsum, const float* lse, int64_t m,
                      hipStream_t stream);
 int launch_topk_scan(const TopkScanArgs& sa, hipStream_t stream);
+int launch_sum(const float* x, int64_t n, float* out, hipStream_t stream);
 
 // ----------------------------------------------------------------- forward --
 // Outputs of the vocabulary-shard forward (all null for the full-vocabulary one).
@@ -312,13 +337,16 @@ template <class E>
 int forward_impl(const Plan& p, const void* hidden, const void* weight, const float* bias,
                  const int64_t* labels, const int64_t* row_idx, int64_t m, int64_t h, int64_t v,
                  int64_t ignore, int64_t exclude, float softcap, float* losses, float* lse,
-                 float* valid_count, const ShardStats& shard, char* ws, hipStream_t stream) {
+                 float* valid_count, const ShardStats& shard, char* ws, hipStream_t stream,
+                 const RowOptions& opt) {
   using T = typename E::T;
-  const ForwardLayout l = forward_layout(p);
+  const bool dynamic = opt.row_count != nullptr;
+  const ForwardLayout l = forward_layout(p, dynamic, opt.weighted_sum != nullptr);
   ForwardArgs fa;
   fa.hidden = hidden; fa.weight = weight; fa.bias = bias;
   fa.m = (int)m; fa.h = (int)h; fa.v = (int)v;
   fa.exclude = exclude - shard.vocab_start; fa.softcap = softcap;
+  fa.logit_scale = opt.logit_scale; fa.m_dev = opt.row_count;
   fa.n_ttiles = p.n_ttiles; fa.n_vtiles = p.n_vtiles; fa.nsplit = p.nsplit;
   fa.part_max = reinterpret_cast<float*>(ws + l.part_max);
   fa.part_sum = reinterpret_cast<float*>(ws + l.part_sum);
@@ -336,11 +364,19 @@ int forward_impl(const Plan& p, const void* hidden, const void* weight, const fl
   ca.label_offset = shard.vocab_start;
   ca.local_max = shard.local_max; ca.local_sum = shard.local_sum;
   ca.target_logits = shard.target_logits;
+  ca.logit_scale = opt.logit_scale; ca.token_weights = opt.token_weights;
+  ca.n_vtiles = p.n_vtiles; ca.tile = p.tile; ca.m_dev = opt.row_count;
+  float* weighted = reinterpret_cast<float*>(ws + l.weighted);
+  if (opt.weighted_sum != nullptr) {
+    ca.weighted = weighted;
+    ca.weighted_rows = (int)m;
+  }
   {
     ScopedTimer timer(kClassCombine, stream);
     lce_combine_loss_kernel<T><<<(int)ceil_div(m, kCombineRowsPerBlock), 256, 0, stream>>>(ca);
   }
   TLCE_LAUNCH_CHECK();
+  if (opt.weighted_sum != nullptr) return launch_sum(weighted, m, opt.weighted_sum, stream);
   return 0;
 }
 
@@ -355,7 +391,8 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
                        const void* weight, const int64_t* row_idx, int64_t m, int64_t n_out,
                        int64_t h, int64_t v, int dtype, void* grad_hidden, void* grad_weight,
                        char* ws, hipStream_t stream, Producer&& produce,
-                       const std::function<int(float*)>& before_cast = nullptr) {
+                       const std::function<int(float*)>& before_cast = nullptr,
+                       const int64_t* m_dev = nullptr) {
   using T = typename E::T;
   const bool weight_grad = grad_weight != nullptr;
   float* acc32 = reinterpret_cast<float*>(ws + l.acc32);
@@ -372,9 +409,10 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     // K-contiguous copies for engines that cannot read K-major operands
     if (int rc = launch_transpose<T>(weight_t, h, v, h, wt, p.vp, p.vp, stream)) return rc;
     if (weight_grad) {
-      if (int rc = launch_transpose<T>(hidden_t, h, m, h, ht, p.mp, p.mp, stream)) return rc;
+      if (int rc = launch_transpose<T>(hidden_t, h, m, h, ht, p.mp, p.mp, stream, m_dev))
+        return rc;
     }
-  } else if (weight_grad && m64 != m) {
+  } else if (weight_grad && m64 != m && m_dev == nullptr) {
     // whole 64-row K slabs must exist: pad hidden with zero rows
     TLCE_HIP(hipMemcpyAsync(ht, hidden_t, (size_t)(m * h * sizeof(T)), hipMemcpyDeviceToDevice,
                             stream));
@@ -395,7 +433,9 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     dh.c = acc32; dh.ldc = h; dh.c_rows = (int)p.mp; dh.c_cols = (int)h;
     dh.c_split_stride = p.mp * h;
     dh.mode = (panel == 0) ? kStoreF32 : kAddF32;
+    dh.m_dev = m_dev; dh.m_role = kRowsFollow;
     GemmArgs dw;
+    dw.m_dev = m_dev; dw.m_role = kKFollows; dw.m_round = p.bk;
     dw.k_per_split = 0;
     dw.ni = p.n_htiles; dw.nj = (int)(width / p.tile);
     dw.c = weight_grad ? static_cast<T*>(grad_weight) + v0 * h : nullptr; dw.ldc = h;
@@ -434,13 +474,14 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
   if (before_cast) {
     if (int rc = before_cast(acc32)) return rc;   // extra float32 terms of grad_hidden
   }
-  if (row_idx != nullptr) {
+  if (row_idx != nullptr || m_dev != nullptr) {
     if (int rc = fill_zero(grad_hidden, n_out * h * dtype_bytes(dtype), stream)) return rc;
   }
   {
     ScopedTimer timer(kClassOther, stream);
     lce_finalize_grad_hidden_kernel<T><<<(int)m, 256, 0, stream>>>(
-        acc32, p.dh_ksplit, p.mp * h, row_idx, (int)m, (int)h, static_cast<T*>(grad_hidden));
+        acc32, p.dh_ksplit, p.mp * h, row_idx, (int)m, (int)h, static_cast<T*>(grad_hidden),
+        m_dev);
   }
   TLCE_LAUNCH_CHECK();
   return 0;
@@ -456,13 +497,16 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
                   int64_t h, int64_t v, int dtype, int reduction, int64_t ignore, int64_t exclude,
                   float softcap, int64_t vocab_start, void* grad_hidden, void* grad_weight,
                   float* grad_bias, char* ws, hipStream_t stream,
-                  float probabilities_scale = 0.0f) {
+                  float probabilities_scale, const RowOptions& opt) {
   const BackwardLayout l = backward_layout(p, m, h, dtype, grad_weight != nullptr);
   float* scale = reinterpret_cast<float*>(ws + l.scale);
   ScaleArgs sa;
   sa.labels = labels; sa.row_idx = row_idx; sa.grad_output = grad_output;
   sa.valid_count = valid_count; sa.m = (int)m; sa.mp = (int)p.mp; sa.reduction = reduction;
-  sa.ignore = ignore; sa.scale = scale; sa.constant = probabilities_scale; sa.multiplier = 1.0f;
+  sa.ignore = ignore; sa.scale = scale; sa.constant = probabilities_scale;
+  // the gradient with respect to the raw dot products carries the logit multiplier
+  sa.multiplier = opt.logit_scale;
+  sa.token_weights = opt.token_weights; sa.m_dev = opt.row_count;
   if (int rc = launch_token_scale(sa, stream)) return rc;
   if (grad_bias != nullptr) {
     if (int rc = fill_zero(grad_bias, v * 4, stream)) return rc;
@@ -476,7 +520,7 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     ga.label_offset = vocab_start;
     ga.probabilities = (labels == nullptr) ? 1 : 0;
     ga.cap_grad = (labels == nullptr) ? 0 : 1;
-    ga.logit_scale = 1.0f;
+    ga.logit_scale = opt.logit_scale; ga.m_dev = opt.row_count;
     ga.v0 = (int)v0;
     ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
     ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
@@ -484,7 +528,7 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     return launch_grad_logits<E>(ga, stream);
   };
   return panel_contractions<E>(p, l, hidden, weight, row_idx, m, n_out, h, v, dtype, grad_hidden,
-                               grad_weight, ws, stream, produce);
+                               grad_weight, ws, stream, produce, nullptr, opt.row_count);
 }
 
 // -------------------------------------------------------------- frozen KL ----
@@ -571,7 +615,7 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
   // teacher statistics first: its probabilities need the teacher lse
   if (int rc = forward_impl<E>(pt, teacher_hidden, teacher_weight, nullptr, nullptr, nullptr, m,
                                ht, v, 0, -1, softcap, nullptr, teacher_lse, nullptr, ShardStats{},
-                               ws + l.stats, stream))
+                               ws + l.stats, stream, RowOptions{}))
     return rc;
   float* ones = reinterpret_cast<float*>(ws + l.ones);
   float* tsum = reinterpret_cast<float*>(ws + l.tsum);
@@ -798,11 +842,11 @@ int soft_embedding_impl(const Plan& fp, const Plan& bp, const SoftEmbeddingLayou
   float* lse = reinterpret_cast<float*>(ws + l.lse);
   if (int rc = forward_impl<E>(fp, hidden, weight, nullptr, nullptr, nullptr, m, h, v, 0, -1,
                                softcap, nullptr, lse, nullptr, ShardStats{}, ws + l.forward_ws,
-                               stream))
+                               stream, RowOptions{}))
     return rc;
   return backward_impl<E>(bp, hidden, weight, nullptr, nullptr, nullptr, lse, nullptr, nullptr, m,
                           m, h, v, dtype, TLCE_REDUCTION_SUM, 0, -1, softcap, 0, out, nullptr,
-                          nullptr, ws + l.backward_ws, stream, scale);
+                          nullptr, ws + l.backward_ws, stream, scale, RowOptions{});
 }
 
 
@@ -830,11 +874,12 @@ int soft_embedding_impl(const Plan& fp, const Plan& bp, const SoftEmbeddingLayou
 #define TLCE_ENGINE_ENTRY_POINTS(X, E)                                                          \
   X int forward_impl<E>(const Plan&, const void*, const void*, const float*, const int64_t*,    \
                         const int64_t*, int64_t, int64_t, int64_t, int64_t, int64_t, float,     \
-                        float*, float*, float*, const ShardStats&, char*, hipStream_t);         \
+                        float*, float*, float*, const ShardStats&, char*, hipStream_t,          \
+                        const RowOptions&);                                                     \
   X int backward_impl<E>(const Plan&, const void*, const void*, const float*, const int64_t*,   \
                          const int64_t*, const float*, const float*, const float*, int64_t,     \
                          int64_t, int64_t, int64_t, int, int, int64_t, int64_t, float, int64_t, \
-                         void*, void*, float*, char*, hipStream_t, float);                      \
+                         void*, void*, float*, char*, hipStream_t, float, const RowOptions&);   \
   X int soft_embedding_impl<E>(const Plan&, const Plan&, const SoftEmbeddingLayout&,            \
                                const void*, const void*, int64_t, int64_t, int64_t, int, float, \
                                float, void*, char*, hipStream_t);                               \

@@ -26,18 +26,29 @@ struct ForwardArgs {
   int m, h, v;
   int64_t exclude;
   float softcap;
+  float logit_scale = 1.0f;   // logits = cap(logit_scale * hidden . weight^T + bias); > 0
   int n_ttiles, n_vtiles, nsplit;
   float* part_max;      // [nsplit, part_ld]  base-2 running max
   float* part_sum;      // [nsplit, part_ld]
   int part_ld;
+  // Row count known only to the device (null: m is exact).  m is then the
+  // capacity; token tiles, vocabulary splits and part_ld follow the real count
+  // exactly as the host plan would have set them for it.
+  const int64_t* m_dev = nullptr;
 };
 
 template <class E, bool kSoftcap, bool kBias>
 __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
-  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
-  if (logical >= p.n_ttiles * p.nsplit) return;
+  if (p.m_dev != nullptr) {
+    p.m = effective_rows(p.m, p.m_dev);
+    p.n_ttiles = (p.m + E::kTile - 1) / E::kTile;
+    p.nsplit = forward_vocab_splits(p.n_ttiles, p.n_vtiles);
+    p.part_ld = p.n_ttiles * E::kTile;
+  }
+  const int logical = xcd_logical_block_of(blockIdx.x, p.n_ttiles * p.nsplit);
+  if (logical < 0) return;
   int tt, vs;
   grouped_tile(logical, p.n_ttiles, p.nsplit, 4, &tt, &vs);
   const int vt0 = (int)((int64_t)vs * p.n_vtiles / p.nsplit);
@@ -46,7 +57,12 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
   E eng;
   const T* hidden = static_cast<const T*>(p.hidden);
   const T* weight = static_cast<const T*>(p.weight);
-  const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
+  // the logit multiplier is applied where the raw dot product is first touched:
+  // with the bias, else inside the soft cap's argument, else inside the
+  // exponent's scale
+  const float raw_scale = kBias ? 1.0f : p.logit_scale;
+  const float inv_cap = kSoftcap ? raw_scale / p.softcap : 0.0f;
+  const float log2e_scaled = kSoftcap ? TLCE_LOG2E : TLCE_LOG2E * raw_scale;
 
   float run_max[E::kCols], run_sum[E::kCols];
 #pragma unroll
@@ -69,7 +85,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
       for (int i = 0; i < E::kRows; ++i) {
         const float b = p.bias[min(vbase + eng.row(i), p.v - 1)];
 #pragma unroll
-        for (int j = 0; j < E::kCols; ++j) E::set(acc, j, i, E::get(acc, j, i) + b);
+        for (int j = 0; j < E::kCols; ++j)
+          E::set(acc, j, i, fmaf(E::get(acc, j, i), p.logit_scale, b));
       }
     }
     // Only the last vocabulary tile (rows past v) and the tile that holds the
@@ -97,12 +114,12 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
       float tile_max = -INFINITY;
 #pragma unroll
       for (int i = 0; i < E::kRows; ++i) tile_max = fmaxf(tile_max, E::get(acc, j, i));
-      const float new_max = fmaxf(run_max[j], tile_max * TLCE_LOG2E);
+      const float new_max = fmaxf(run_max[j], tile_max * log2e_scaled);
       if (new_max > -INFINITY) {
         float s = run_sum[j] * fast_exp2(run_max[j] - new_max);
 #pragma unroll
         for (int i = 0; i < E::kRows; ++i)
-          s += fast_exp2(fmaf(E::get(acc, j, i), TLCE_LOG2E, -new_max));
+          s += fast_exp2(fmaf(E::get(acc, j, i), log2e_scaled, -new_max));
         run_sum[j] = s;
         run_max[j] = new_max;
       }
@@ -163,6 +180,16 @@ struct CombineArgs {
   float* local_max;
   float* local_sum;
   float* target_logits;
+  // masked-token loss extras: the logit multiplier of the forward kernel, an
+  // optional per-row weight [m] and, when weighted != null, the row's weighted
+  // loss written compactly (weighted[r] = weight[r] * loss[r], 0 for ignored
+  // rows and rows past the device row count) for a deterministic sum afterwards
+  float logit_scale = 1.0f;
+  const float* token_weights = nullptr;
+  float* weighted = nullptr;
+  int weighted_rows = 0;             // entries of `weighted` to define (rows past m get 0)
+  int n_vtiles = 0, tile = 0;        // for the device-side plan when m_dev != null
+  const int64_t* m_dev = nullptr;
 };
 
 // Dot product of two rows of length h by one wave (every lane gets the sum):
@@ -197,10 +224,19 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
   const int wave = threadIdx.x >> 6;
   if (threadIdx.x == 0) block_valid = 0;
   __syncthreads();
+  if (p.m_dev != nullptr) {
+    p.m = effective_rows(p.m, p.m_dev);
+    const int n_ttiles = (p.m + p.tile - 1) / p.tile;
+    p.nsplit = forward_vocab_splits(n_ttiles, p.n_vtiles);
+    p.part_ld = n_ttiles * p.tile;
+  }
   int wave_valid = 0;
   for (int i = 0; i < kCombineRowsPerBlock / 4; ++i) {
     const int r = blockIdx.x * kCombineRowsPerBlock + wave * (kCombineRowsPerBlock / 4) + i;
-    if (r >= p.m) break;
+    if (r >= p.m) {
+      if (p.weighted != nullptr && r < p.weighted_rows && lane == 0) p.weighted[r] = 0.0f;
+      continue;
+    }
     float mx = -INFINITY;
     for (int s = lane; s < p.nsplit; s += 64)
       mx = fmaxf(mx, p.part_max[(int64_t)s * p.part_ld + r]);
@@ -226,7 +262,7 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
     if (has_target) {
       const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
       const T* wrow = static_cast<const T*>(p.weight) + y * (int64_t)p.h;
-      float dot = wave_dot<T>(hrow, wrow, p.h, lane);
+      float dot = wave_dot<T>(hrow, wrow, p.h, lane) * p.logit_scale;
       if (p.bias != nullptr) dot += p.bias[y];
       if (p.softcap > 0.0f) dot = p.softcap * tanhf(dot / p.softcap);
       target = dot;
@@ -239,8 +275,13 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
         p.target_logits[r] = (here && label == p.exclude) ? -INFINITY : target;
       } else {
         p.lse[r] = lse;
-        const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r;
-        p.losses[o] = valid ? (lse - target) : 0.0f;
+        const float loss = valid ? (lse - target) : 0.0f;
+        if (p.losses != nullptr) {
+          const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : (int64_t)r;
+          p.losses[o] = loss;
+        }
+        if (p.weighted != nullptr)
+          p.weighted[r] = (p.token_weights != nullptr) ? loss * p.token_weights[r] : loss;
       }
     }
     wave_valid += valid ? 1 : 0;
@@ -264,6 +305,8 @@ struct ScaleArgs {
   int64_t ignore;
   float constant;   // labels == null: every real row gets this scale
   float multiplier; // applied to every scale
+  const float* token_weights = nullptr;   // optional per-row factor [m] (loss weights)
+  const int64_t* m_dev = nullptr;   // device row count (null: m is exact); rows past it get 0
   float* scale;
 };
 
@@ -288,8 +331,10 @@ struct GradLogitsArgs {
   int probabilities;     // 1: g = softmax * scale (labels may be null; no onehot)
   int cap_grad;          // 1: g carries the soft cap's derivative 1 - tanh^2 (a gradient
                          // with respect to the raw logits), 0: it does not (probabilities)
-  float logit_scale;     // logits = cap(logit_scale * hidden . weight^T); needs bias == null
-                         // unless it is 1.  The caller folds it into `scale` for gradients.
+  float logit_scale;     // logits = cap(logit_scale * hidden . weight^T + bias).  The caller
+                         // folds it into `scale` for gradients.
+  const int64_t* m_dev = nullptr;   // device row count (null: m is exact): m is then the
+                         // capacity and only the token tiles below the real count are produced
   int v0;             // first vocabulary row of the panel
   int n_ttiles, n_ptiles;
   void* g;            // [mp, ldg]
@@ -330,8 +375,12 @@ template <class E, bool kSoftcap, bool kBias>
 __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(GradLogitsArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
-  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
-  if (logical >= p.n_ttiles * p.n_ptiles) return;
+  if (p.m_dev != nullptr) {
+    p.m = effective_rows(p.m, p.m_dev);
+    p.n_ttiles = (p.m + E::kTile - 1) / E::kTile;
+  }
+  const int logical = xcd_logical_block_of(blockIdx.x, p.n_ttiles * p.n_ptiles);
+  if (logical < 0) return;
   int tt, pv;
   grouped_tile(logical, p.n_ttiles, p.n_ptiles, 4, &tt, &pv);
 
@@ -342,8 +391,11 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   const int vbase = p.v0 + pv * E::kTile;
   eng.mainloop_set(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
 
-  const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
-  const float log2e_scaled = TLCE_LOG2E * p.logit_scale;
+  // the bias add applies the logit multiplier itself (z = multiplier * dot + bias)
+  const float raw_scale = kBias ? 1.0f : p.logit_scale;
+  const float inv_cap = kSoftcap ? raw_scale / p.softcap : 0.0f;
+  const float log2e_scaled = TLCE_LOG2E * raw_scale;
+  const float inv_logit_scale = kBias ? 1.0f / p.logit_scale : 1.0f;
   // per owned token column: row of its label inside this tile (-1: none here),
   // lse in base-2 units, and the loss scale (0 for ignored and padding rows,
   // which zeroes their whole column of g without a per-element test)
@@ -368,7 +420,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
     for (int i = 0; i < E::kRows; ++i) {
       const float b = p.bias[min(vbase + eng.row(i), p.v - 1)];
 #pragma unroll
-      for (int j = 0; j < E::kCols; ++j) E::set(acc, j, i, E::get(acc, j, i) + b);
+      for (int j = 0; j < E::kCols; ++j)
+        E::set(acc, j, i, fmaf(E::get(acc, j, i), p.logit_scale, b));
     }
   }
   // workgroup-uniform: rows past v or the excluded column in this tile;
@@ -402,7 +455,9 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   auto add_grad_bias = [&](int row, float row_sum) {
     const int v = vbase + row;
     row_sum = eng.reduce_over_cols(row_sum);
-    if (eng.col_leader() && v < p.v && row_sum != 0.0f) atomicAdd(p.grad_bias + v, row_sum);
+    // g carries the logit multiplier (folded into scale); the bias sits outside it
+    if (eng.col_leader() && v < p.v && row_sum != 0.0f)
+      atomicAdd(p.grad_bias + v, row_sum * inv_logit_scale);
   };
 
   T* g_out = static_cast<T*>(p.g);
@@ -966,14 +1021,30 @@ struct GemmArgs {
   int64_t c_split_stride;  // elements between the outputs of consecutive K splits
   int c_rows, c_cols;
   int mode;
+  // Token count known only to the device (null: the sizes above are exact).
+  // m_role kRowsFollow: the B rows / output rows are tokens (grad_hidden): tiles
+  // along j and c_rows shrink to the real count.  kKFollows: K is the token axis
+  // (grad_weight): k shrinks to the real count rounded up to m_round.
+  const int64_t* m_dev = nullptr;
+  int m_role = 0, m_round = 1;
 };
+enum { kRowsFollow = 1, kKFollows = 2 };
 
 template <class E, bool kAKMajor, bool kBKMajor>
 __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
-  const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
-  if (logical >= p.ni * p.nj) return;
+  if (p.m_dev != nullptr) {
+    if (p.m_role == kRowsFollow) {
+      p.c_rows = effective_rows(p.c_rows, p.m_dev);
+      p.nj = (p.c_rows + E::kTile - 1) / E::kTile;
+    } else if (p.m_role == kKFollows) {
+      const int rows = effective_rows(p.k, p.m_dev);
+      p.k = (rows + p.m_round - 1) / p.m_round * p.m_round;
+    }
+  }
+  const int logical = xcd_logical_block_of(blockIdx.x, p.ni * p.nj);
+  if (logical < 0) return;
   int ti, tj;
   grouped_tile(logical, p.ni, p.nj, 4, &ti, &tj);
   // each K split owns its own output slab: no atomics, reproducible sums; a
@@ -1046,8 +1117,10 @@ template <typename T>
 __global__ __launch_bounds__(256) void lce_transpose_pad_kernel(const T* __restrict__ in,
                                                                 int64_t ld_in, int rows, int cols,
                                                                 T* __restrict__ out,
-                                                                int64_t ld_out, int out_cols) {
+                                                                int64_t ld_out, int out_cols,
+                                                                const int64_t* rows_dev) {
   __shared__ T tile[64][66];
+  rows = effective_rows(rows, rows_dev);   // rows past a device-side count read as zero
   const int tx = threadIdx.x & 63;
   const int ty = threadIdx.x >> 6;
   const int c0 = blockIdx.x * 64;
@@ -1075,9 +1148,10 @@ __global__ __launch_bounds__(256) void lce_transpose_pad_kernel(const T* __restr
 template <typename T>
 __global__ __launch_bounds__(256) void lce_finalize_grad_hidden_kernel(
     const float* __restrict__ acc32, int n_splits, int64_t split_stride,
-    const int64_t* __restrict__ row_idx, int m, int h, T* __restrict__ out) {
+    const int64_t* __restrict__ row_idx, int m, int h, T* __restrict__ out,
+    const int64_t* __restrict__ m_dev) {
   const int r = blockIdx.x;
-  if (r >= m) return;
+  if (r >= effective_rows(m, m_dev)) return;
   const int64_t o = (row_idx != nullptr) ? row_idx[r] : (int64_t)r;
   const float* src = acc32 + (int64_t)r * h;
   T* dst = out + o * h;

@@ -57,6 +57,13 @@ int launch_topk_scan(const TopkScanArgs& sa, hipStream_t stream) {
   return 0;
 }
 
+int launch_sum(const float* x, int64_t n, float* out, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_sum_kernel<<<1, 1024, 0, stream>>>(x, (int)n, out);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaDirect4Engine<__bf16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaDirect4Engine<_Float16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaEngine<__bf16>)
@@ -128,29 +135,35 @@ int forward_entry(const void* hidden, const void* weight, const float* bias,
                   int64_t h, int64_t v, int dtype, int64_t ignore_index, int64_t exclude_index,
                   float logit_softcap, float* losses, float* lse, float* valid_count,
                   const ShardStats& shard, void* workspace, int64_t workspace_bytes,
-                  hipStream_t stream) {
+                  hipStream_t stream, const RowOptions& opt = RowOptions{}) {
   const bool local = shard.local_max != nullptr;
+  const bool fused = opt.weighted_sum != nullptr;   // the masked-token loss entry point
   if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
   TLCE_REQUIRE(valid_count != nullptr, "forward: valid_count is null");
+  TLCE_REQUIRE(opt.logit_scale > 0.0f, "forward: the logit multiplier must be positive");
   TLCE_REQUIRE(n_out >= m, "forward: n_out=%lld < m=%lld", (long long)n_out, (long long)m);
   TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
                "forward: n_out != m without row_idx");
   if (int rc = fill_zero(valid_count, 4, stream)) return rc;
-  if (!local && (row_idx != nullptr || m == 0)) {
-    TLCE_REQUIRE(losses != nullptr || n_out == 0, "forward: losses is null");
+  TLCE_REQUIRE(local || fused || losses != nullptr || n_out == 0, "forward: losses is null");
+  if (!local && losses != nullptr && (row_idx != nullptr || m == 0 || opt.row_count != nullptr)) {
     if (int rc = fill_zero(losses, n_out * 4, stream)) return rc;
   }
+  if (fused && m == 0) {
+    if (int rc = fill_zero(opt.weighted_sum, 4, stream)) return rc;
+  }
   if (m == 0) return 0;
-  TLCE_REQUIRE(labels && workspace && (local || (losses && lse)), "forward: null pointer");
+  TLCE_REQUIRE(labels && workspace && (local || ((losses || fused) && lse)),
+               "forward: null pointer");
   const Plan p = make_plan(m, h, v, dtype, false, 0);
-  TLCE_REQUIRE(workspace_bytes >= forward_layout(p).total,
-               "forward: workspace too small (%lld < %lld)", (long long)workspace_bytes,
-               (long long)forward_layout(p).total);
+  const int64_t need = forward_layout(p, opt.row_count != nullptr, fused).total;
+  TLCE_REQUIRE(workspace_bytes >= need, "forward: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
   TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0, "forward: workspace must be 256-byte aligned");
   TLCE_DISPATCH(p, dtype,
                 forward_impl<E>(p, hidden, weight, bias, labels, row_idx, m, h, v, ignore_index,
                                 exclude_index, logit_softcap, losses, lse, valid_count, shard,
-                                static_cast<char*>(workspace), stream));
+                                static_cast<char*>(workspace), stream, opt));
 }
 
 }  // namespace
@@ -257,8 +270,10 @@ int backward_entry(const void* hidden, const void* weight, const float* bias,
                    int64_t h, int64_t v, int dtype, int reduction_code, int64_t vocab_start,
                    int64_t ignore_index, int64_t exclude_index, float logit_softcap,
                    void* grad_hidden, void* grad_weight, float* grad_bias, int64_t panel_bytes,
-                   void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+                   void* workspace, int64_t workspace_bytes, hipStream_t stream,
+                   const RowOptions& opt = RowOptions{}) {
   if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  TLCE_REQUIRE(opt.logit_scale > 0.0f, "backward: the logit multiplier must be positive");
   TLCE_REQUIRE(reduction_code >= TLCE_REDUCTION_NONE && reduction_code <= TLCE_REDUCTION_MEAN,
                "backward: bad reduction code %d", reduction_code);
   TLCE_REQUIRE(n_out >= m, "backward: n_out=%lld < m=%lld", (long long)n_out, (long long)m);
@@ -275,7 +290,9 @@ int backward_entry(const void* hidden, const void* weight, const float* bias,
     if (bias != nullptr) return fill_zero(grad_bias, v * 4, stream);
     return 0;
   }
-  TLCE_REQUIRE(labels && lse && valid_count && grad_output && workspace, "backward: null pointer");
+  TLCE_REQUIRE(labels && lse && grad_output && workspace, "backward: null pointer");
+  TLCE_REQUIRE(valid_count != nullptr || reduction_code != TLCE_REDUCTION_MEAN,
+               "backward: the mean reduction needs valid_count");
   TLCE_REQUIRE(((uintptr_t)grad_hidden & 15) == 0 && ((uintptr_t)grad_weight & 15) == 0,
                "backward: gradients must be 16-byte aligned");
   const Plan p = make_plan(m, h, v, dtype, grad_weight != nullptr, panel_bytes);
@@ -288,7 +305,7 @@ int backward_entry(const void* hidden, const void* weight, const float* bias,
                                  grad_output, m, n_out, h, v, dtype, reduction_code, ignore_index,
                                  exclude_index, logit_softcap, vocab_start, grad_hidden,
                                  grad_weight, (bias != nullptr) ? grad_bias : nullptr,
-                                 static_cast<char*>(workspace), stream));
+                                 static_cast<char*>(workspace), stream, 0.0f, opt));
 }
 
 }  // namespace
@@ -320,6 +337,56 @@ extern "C" int tlce_backward_local(const void* hidden, const void* weight, const
                         ignore_index, exclude_index, logit_softcap, grad_hidden, grad_weight,
                         grad_bias, panel_bytes, workspace, workspace_bytes,
                         static_cast<hipStream_t>(stream));
+}
+
+// --------------------------------------------------------- masked-token loss --
+extern "C" int64_t tlce_masked_loss_forward_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                                            int dtype, int dynamic_rows) {
+  if (m < 0 || h <= 0 || v <= 0) return -1;
+  return forward_layout(make_plan(m, h, v, dtype, false, 0), dynamic_rows != 0, true).total;
+}
+
+extern "C" int tlce_masked_loss_forward(const void* hidden, const void* weight, const float* bias,
+                                        const int64_t* labels, const float* token_weights,
+                                        const int64_t* row_idx, const int64_t* row_count,
+                                        int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                                        int64_t ignore_index, int64_t exclude_index,
+                                        float logit_softcap, float logit_multiplier,
+                                        float* losses, float* lse, float* valid_count,
+                                        float* weighted_sum, void* workspace,
+                                        int64_t workspace_bytes, void* stream) {
+  TLCE_REQUIRE(weighted_sum != nullptr || losses != nullptr || n_out == 0,
+               "masked_loss_forward: neither weighted_sum nor losses given");
+  RowOptions opt;
+  opt.logit_scale = logit_multiplier;
+  opt.token_weights = token_weights;
+  opt.row_count = row_count;
+  opt.weighted_sum = weighted_sum;
+  return forward_entry(hidden, weight, bias, labels, row_idx, m, n_out, h, v, dtype, ignore_index,
+                       exclude_index, logit_softcap, losses, lse, valid_count, ShardStats{},
+                       workspace, workspace_bytes, static_cast<hipStream_t>(stream), opt);
+}
+
+extern "C" int tlce_masked_loss_backward(const void* hidden, const void* weight, const float* bias,
+                                         const int64_t* labels, const float* token_weights,
+                                         const int64_t* row_idx, const int64_t* row_count,
+                                         const float* lse, const float* valid_count,
+                                         const float* grad_output, int64_t m, int64_t n_out,
+                                         int64_t h, int64_t v, int dtype, int reduction_code,
+                                         int64_t ignore_index, int64_t exclude_index,
+                                         float logit_softcap, float logit_multiplier,
+                                         void* grad_hidden, void* grad_weight, float* grad_bias,
+                                         int64_t panel_bytes, void* workspace,
+                                         int64_t workspace_bytes, void* stream) {
+  RowOptions opt;
+  opt.logit_scale = logit_multiplier;
+  opt.token_weights = token_weights;
+  opt.row_count = row_count;
+  // d(sum_r w_r loss_r) / d loss_r = w_r: the sum reduction with per-row weights
+  return backward_entry(hidden, weight, bias, labels, row_idx, lse, valid_count, grad_output, m,
+                        n_out, h, v, dtype, reduction_code, 0, ignore_index, exclude_index,
+                        logit_softcap, grad_hidden, grad_weight, grad_bias, panel_bytes, workspace,
+                        workspace_bytes, static_cast<hipStream_t>(stream), opt);
 }
 
 // ---------------------------------------------------------- soft embedding --

@@ -11,6 +11,7 @@ namespace tlce {
 __global__ __launch_bounds__(256) void lce_token_scale_kernel(ScaleArgs p) {
   const int r = blockIdx.x * 256 + threadIdx.x;
   if (r >= p.mp) return;
+  p.m = effective_rows(p.m, p.m_dev);
   float s = 0.0f;
   if (p.labels == nullptr) {
     // no labels: every real row gets grad_output[r] (per-row objectives) or the constant
@@ -24,7 +25,24 @@ __global__ __launch_bounds__(256) void lce_token_scale_kernel(ScaleArgs p) {
       s = p.grad_output[0] / p.valid_count[0];
     }
   }
+  if (p.token_weights != nullptr && r < p.m) s *= p.token_weights[r];
   p.scale[r] = s * p.multiplier;
+}
+
+// out[0] = sum of x[0..n) in a fixed order (one workgroup, pairwise tree): the
+// weighted loss sum of the masked-token loss, reproducible run to run.
+__global__ __launch_bounds__(1024) void lce_sum_kernel(const float* __restrict__ x, int n,
+                                                       float* __restrict__ out) {
+  __shared__ float part[1024];
+  float s = 0.0f;
+  for (int i = threadIdx.x; i < n; i += 1024) s += x[i];
+  part[threadIdx.x] = s;
+  __syncthreads();
+  for (int o = 512; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[0] = part[0];
 }
 
 // losses[r] = losses[r] + tsum[r] * lse_draft[r] + 1  (see lce_kl_panel_kernel)

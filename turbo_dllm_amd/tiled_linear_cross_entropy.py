@@ -22,9 +22,47 @@ from the softmax outright, also under a soft cap
 
 from __future__ import annotations
 
+import contextlib
 from typing import Optional
 
 import torch
+
+# How the device path deals with rows whose label is ``ignore_index``:
+#   "sync"   (default) compact them away on the device and read the count of
+#            loss-bearing rows back once, so every launch is sized exactly (the
+#            one host synchronisation the reference's call sites incur as well,
+#            nemotron/model.py:4244-4248);
+#   "device" compact them away without any host read-back: launches are sized
+#            for all rows and the kernels take the count from device memory, so
+#            the whole loss (forward and backward) can be recorded into a HIP
+#            graph;
+#   "none"   no compaction: the caller has compacted already (the reference's
+#            call sites do) or accepts GEMM work on ignored rows; the kernels
+#            zero their loss and gradient like the reference operator.
+COMPACTION_MODES = ("sync", "device", "none")
+_compaction_mode = "sync"
+
+
+def set_compaction_mode(mode: str) -> str:
+    """Selects how the device path handles ignored rows; returns the old mode."""
+    global _compaction_mode
+    if mode not in COMPACTION_MODES:
+        raise ValueError(f"compaction mode must be one of {COMPACTION_MODES}")
+    old, _compaction_mode = _compaction_mode, mode
+    return old
+
+
+def get_compaction_mode() -> str:
+    return _compaction_mode
+
+
+@contextlib.contextmanager
+def compaction_mode(mode: str):
+    old = set_compaction_mode(mode)
+    try:
+        yield
+    finally:
+        set_compaction_mode(old)
 
 
 def _canonical_dtype(dtype: torch.dtype | str) -> torch.dtype:
@@ -240,26 +278,42 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
 
     hidden_flat = hidden.reshape(-1, hidden.shape[-1]).contiguous()
     labels_flat = labels.reshape(-1).to(torch.long).contiguous()
-    weight = weight.contiguous()
+    # the kernels read the head as [V, H]: a [H, V] head is re-laid once here and
+    # the copy is kept for the backward
+    weight_vf = weight.t().contiguous() if weight_dim_first else weight.contiguous()
     if bias is not None:
         bias = bias.contiguous()
     n = hidden_flat.shape[0]
+    mode = _compaction_mode
 
-    row_idx, m = native.compact_rows(labels_flat, ignore_index)
-    if m == n:
-        row_idx = None
-        rows, targets = hidden_flat, labels_flat
+    row_idx = row_count = None
+    rows, targets, m = hidden_flat, labels_flat, n
+    if mode == "sync":
+        row_idx, m = native.compact_rows(labels_flat, ignore_index)
+        if m == n:
+            row_idx = None
+        else:
+            rows = native.gather_rows(hidden_flat, row_idx)
+            targets = native.gather_rows(labels_flat, row_idx)
+    elif mode == "device" and n > 0:
+        row_idx, row_count = native.compact_rows_device(labels_flat, ignore_index)
+        rows, targets, _ = native.gather_loss_rows(hidden_flat, labels_flat, None, row_idx,
+                                                   row_count, ignore_index)
+
+    if row_count is None:
+        losses, lse, valid_count = native.forward(
+            rows, weight_vf, bias, targets,
+            row_block_size=0, ignore_index=ignore_index, exclude_index=exclude_index,
+            logit_softcap=float(logit_softcap), compute_dtype=compute_dtype,
+            weight_dim_first=False, row_idx=row_idx, n_out=n,
+        )
     else:
-        rows = native.gather_rows(hidden_flat, row_idx)
-        targets = native.gather_rows(labels_flat, row_idx)
-
-    losses, lse, valid_count = native.forward(
-        rows, weight, bias, targets,
-        row_block_size=0, ignore_index=ignore_index, exclude_index=exclude_index,
-        logit_softcap=float(logit_softcap), compute_dtype=compute_dtype,
-        weight_dim_first=weight_dim_first, row_idx=row_idx, n_out=n,
-    )
-    ctx.save_for_backward(rows, weight, bias, targets, lse, valid_count, row_idx)
+        losses, lse, valid_count, _ = native.masked_loss_forward(
+            rows, weight_vf, bias, targets, None, m=n, row_idx=row_idx, row_count=row_count,
+            n_out=n, ignore_index=ignore_index, exclude_index=exclude_index,
+            logit_softcap=float(logit_softcap), want_losses=True, want_sum=False,
+        )
+    ctx.save_for_backward(rows, weight_vf, bias, targets, lse, valid_count, row_idx, row_count)
     ctx.hidden_shape = hidden.shape
     ctx.n_rows = n
     ctx.reduction = reduction
@@ -278,15 +332,25 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
 def _device_backward(ctx, grad_output, frozen: bool):
     from . import chunked_linear_ce_native as native
 
-    rows, weight, bias, targets, lse, valid_count, row_idx = ctx.saved_tensors
-    call = native.backward_frozen_weight if frozen else native.backward
-    grad_hidden, grad_weight, grad_bias = call(
-        rows, weight, bias, targets, lse, valid_count, grad_output,
-        row_block_size=0, reduction=ctx.reduction, ignore_index=ctx.ignore_index,
-        exclude_index=ctx.exclude_index, logit_softcap=ctx.logit_softcap,
-        compute_dtype=ctx.compute_dtype, weight_dim_first=ctx.weight_dim_first,
-        row_idx=row_idx, n_out=ctx.n_rows,
-    )
+    rows, weight_vf, bias, targets, lse, valid_count, row_idx, row_count = ctx.saved_tensors
+    if row_count is None:
+        call = native.backward_frozen_weight if frozen else native.backward
+        grad_hidden, grad_weight, grad_bias = call(
+            rows, weight_vf, bias, targets, lse, valid_count, grad_output,
+            row_block_size=0, reduction=ctx.reduction, ignore_index=ctx.ignore_index,
+            exclude_index=ctx.exclude_index, logit_softcap=ctx.logit_softcap,
+            compute_dtype=ctx.compute_dtype, weight_dim_first=False,
+            row_idx=row_idx, n_out=ctx.n_rows,
+        )
+    else:
+        grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(
+            rows, weight_vf, bias, targets, None, lse, valid_count, grad_output,
+            reduction=ctx.reduction, m=ctx.n_rows, row_idx=row_idx, row_count=row_count,
+            n_out=ctx.n_rows, ignore_index=ctx.ignore_index, exclude_index=ctx.exclude_index,
+            logit_softcap=ctx.logit_softcap, compute_weight_grad=not frozen,
+        )
+    if not frozen and ctx.weight_dim_first:
+        grad_weight = grad_weight.t().contiguous()
     return (
         grad_hidden.reshape(ctx.hidden_shape),
         None if frozen else grad_weight,
