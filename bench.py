@@ -35,33 +35,98 @@ def build_workload(name: str, seed: int):
     return workloads.CONFIGS[name](seed=seed)
 
 
-def cpu_baseline(wl, sample_rows: int):
-    """Oracle (unfused float32 path + analytic gradients) on the first
-    ``sample_rows`` loss-bearing rows, all host threads."""
+def _median(values):
+    values = sorted(values)
+    return values[len(values) // 2]
+
+
+def _time_cpu_paths(hidden, weight, labels, softcap, iterations, warmup):
+    """Median seconds (forward, backward) of the two CPU paths on the given rows:
+    the float32 oracle (unfused matmul -> log-softmax -> masked NLL, analytic
+    gradients) and this package's host implementation of the loss API
+    (vocabulary tiles of 8192, autograd backward)."""
     import torch
 
     sys.path.insert(0, str(REPO_ROOT / "oracle"))
     import linear_ce_oracle as oracle
+    from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+
+    h32, w32 = hidden.float(), weight.float()
+    unfused, tiled = [], []
+    for it in range(warmup + iterations):
+        t0 = time.perf_counter()
+        oracle.dense_linear_ce(h32, w32, labels, logit_softcap=softcap, dtype=torch.float32)
+        t1 = time.perf_counter()
+        oracle.dense_linear_ce_grads(h32, w32, labels, logit_softcap=softcap, dtype=torch.float32)
+        t2 = time.perf_counter()
+        h = hidden.clone().requires_grad_(True)
+        w = weight.clone().requires_grad_(True)
+        t3 = time.perf_counter()
+        loss = tiled_linear_cross_entropy(h, w, labels, vocab_block_size=8192,
+                                          logit_softcap=softcap, dtype=torch.float32,
+                                          weight_layout="vocab_first")
+        t4 = time.perf_counter()
+        loss.backward()
+        t5 = time.perf_counter()
+        if it >= warmup:
+            unfused.append((t1 - t0, t2 - t1))
+            tiled.append((t4 - t3, t5 - t4))
+
+    def summary(samples, rows):
+        fwd = _median([a for a, _ in samples])
+        bwd = _median([b for _, b in samples])
+        both = _median([a + b for a, b in samples])
+        return {"forward_s": fwd, "backward_s": bwd, "forward_backward_s": both,
+                "tokens_per_s": rows / both}
+
+    rows = int((labels != -100).sum())
+    return summary(unfused, rows), summary(tiled, rows)
+
+
+def cpu_baseline(wl, sample_rows: int, iterations: int = 5, warmup: int = 2):
+    """The CPU paths timed on this box's host cores beside the GPU kernels.
+
+    ``value`` is the float32 oracle's forward+backward throughput on the first
+    ``sample_rows`` loss-bearing rows of the workload at its full H and V (rows
+    are independent, so tokens/s carries over to the whole batch up to the
+    fixed cost of the [V, H] weight gradient, which the slice pays in full:
+    the figure is an extrapolation that favours neither side much).  Also
+    reported: this package's host implementation of the loss API on the same
+    rows, and both paths on the small-head configuration at its full size
+    (2048 rows, H=1024, V=32000).  Two warm-up and ``iterations`` timed passes
+    each, medians."""
+    import torch
+
+    from turbo_dllm_amd import workloads
 
     keep = torch.nonzero(wl.labels != -100).flatten()[:sample_rows]
-    hidden = wl.hidden.index_select(0, keep).float()
+    hidden = wl.hidden.index_select(0, keep)
     labels = wl.labels.index_select(0, keep)
-    weight = wl.weight.float()
     cores = torch.get_num_threads()
-    t0 = time.perf_counter()
-    oracle.dense_linear_ce(hidden, weight, labels, logit_softcap=wl.logit_softcap,
-                           dtype=torch.float32)
-    oracle.dense_linear_ce_grads(hidden, weight, labels, logit_softcap=wl.logit_softcap,
-                                 dtype=torch.float32)
-    dt = time.perf_counter() - t0
+    t_start = time.perf_counter()
+    unfused, tiled = _time_cpu_paths(hidden, wl.weight, labels, wl.logit_softcap, iterations,
+                                     warmup)
+    small = workloads.small_head(seed=wl.seed)
+    small_unfused, small_tiled = _time_cpu_paths(small.hidden, small.weight, small.labels, None,
+                                                 iterations, warmup)
     rows = int(keep.numel())
     return {
-        "value": rows / dt,
+        "value": unfused["tokens_per_s"],
         "unit": "tokens/s",
         "cores": cores,
         "kind": "port",
-        "sample": f"fwd+bwd of the float32 oracle on the first {rows} loss-bearing rows "
-                  f"(full H and V), {dt:.2f} s",
+        "sample": f"float32 oracle (unfused path + analytic gradients), forward+backward on the "
+                  f"first {rows} loss-bearing rows at full H and V, median of {iterations} "
+                  f"after {warmup} warm-up passes; extrapolated per row to the whole batch",
+        "oracle_unfused": unfused,
+        "host_tiled_path": dict(tiled, note="turbo_dllm_amd host implementation of the loss "
+                                            "API, vocabulary tile 8192, same rows"),
+        "small_head_full_size": {
+            "rows": small.n_rows, "loss_rows": small.n_loss_rows,
+            "oracle_unfused": small_unfused, "host_tiled_path": small_tiled,
+            "input_rows_per_s_unfused": small.n_rows / small_unfused["forward_backward_s"],
+        },
+        "cpu_seconds_spent": time.perf_counter() - t_start,
     }
 
 
@@ -110,21 +175,40 @@ def measure_compaction_gather(torch, native, device, n, h, hidden):
     }
 
 
-# Bytes between L2 and the memory fabric per launch, from rocprofv3 FETCH_SIZE and WRITE_SIZE
-# runs of this script on the default workload (KiB per dispatch, scaled by what each counter
-# reads for a plain copy of known size: 1.984 for FETCH_SIZE, 1.000 for WRITE_SIZE).  Counters
-# cannot be read from inside the process, so the figures are recorded here per kernel symbol.
-MEASURED_TRAFFIC_BYTES = {
-    "block_diffusion_shard_all_rows": {
-        "lce_forward_stats_kernel": 74.10e9 + 1.25e9,
-        "lce_grad_logits_panel_kernel": 6.00e9 + 1.00e9,
-        "lce_gemm_nt_kernel": 7.17e9 + 0.38e9,
-    },
-}
+def source_fingerprint() -> str:
+    """Short hash of the HIP sources: names the build a profile was taken from."""
+    import hashlib
+
+    digest = hashlib.sha256()
+    csrc = REPO_ROOT / "turbo_dllm_amd" / "csrc"
+    for path in sorted(csrc.glob("*.h")) + sorted(csrc.glob("*.hip")):
+        digest.update(path.name.encode())
+        digest.update(path.read_bytes())
+    return digest.hexdigest()[:12]
 
 
-def measured_traffic(workload, kernel):
-    return MEASURED_TRAFFIC_BYTES.get(workload, {}).get(kernel)
+TRAFFIC_PROFILE = REPO_ROOT / "profiles" / "hbm_traffic_per_kernel.txt"
+
+
+def measured_traffic(workload: str, kernel: str):
+    """Bytes between L2 and the memory fabric per launch of ``kernel`` on
+    ``workload``, from the rocprofv3 FETCH_SIZE / WRITE_SIZE summary under
+    profiles/ (counters cannot be read from inside the process).  The summary
+    names the source fingerprint it was measured at; a figure measured on other
+    sources is reported as stale, not as this build's."""
+    if not TRAFFIC_PROFILE.exists():
+        return None, "no traffic profile"
+    current = source_fingerprint()
+    for line in TRAFFIC_PROFILE.read_text().splitlines():
+        fields = line.split()
+        if len(fields) == 6 and fields[0] == "traffic" and fields[1] == workload \
+                and fields[2] == kernel:
+            total = float(fields[4]) + float(fields[5])
+            if fields[3] == current:
+                return total, f"measured on this build ({current})"
+            return None, (f"stale: {total:.3g} B per launch was measured on sources "
+                          f"{fields[3]}, these are {current}")
+    return None, "not measured for this workload"
 
 
 def library_gemm_reference(torch, device, h, v, rows=8192, panel=16384, reps=5):
@@ -262,7 +346,14 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="block_diffusion_shard_all_rows")
     ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--cpu-rows", type=int, default=2048)
+    ap.add_argument("--cpu-rows", type=int, default=512,
+                    help="loss-bearing rows of the workload the CPU paths are timed on")
+    ap.add_argument("--compaction-mode", choices=("sync", "device", "none"), default="sync",
+                    help="how ignored rows are handled (tiled_linear_cross_entropy."
+                         "set_compaction_mode): exact launches after one host read-back of "
+                         "the row count, no read-back (device-side count), or no compaction")
+    ap.add_argument("--panel-mib", type=int, default=0,
+                    help="budget of the backward's logit-gradient panel in MiB (0: 1 GiB default)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain row copy of the weight matrix (known HBM bytes) "
                          "so rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
@@ -279,11 +370,14 @@ def main() -> int:
 
     from turbo_dllm_amd import _lib
     from turbo_dllm_amd import chunked_linear_ce_native as native
-    from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+    from turbo_dllm_amd.tiled_linear_cross_entropy import (set_compaction_mode,
+                                                           tiled_linear_cross_entropy)
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
+    set_compaction_mode(args.compaction_mode)
+    native.PANEL_BYTES = args.panel_mib << 20
     if args.objective != "ce":
         return bench_next_objective(args)
     device = torch.device("cuda:0")
@@ -321,20 +415,36 @@ def main() -> int:
     ms_median = per_step[len(per_step) // 2] if per_step else float("nan")
     loss_value = float(loss.detach())
 
-    # per-kernel-class durations of one forward + backward (HIP events on the launch stream)
+    # per-kernel-class durations of one forward + backward (HIP events on the launch stream;
+    # the library calls are made directly so that all of them run on this thread)
+    softcap = float(wl.logit_softcap or 0.0)
+    go = torch.ones(1, device=device)
     with torch.no_grad():
-        row_idx, m_dev = native.compact_rows(labels, -100)
-        rows = hidden.detach() if m_dev == n else native.gather_rows(hidden.detach(), row_idx)
-        targets = labels if m_dev == n else native.gather_rows(labels, row_idx)
-        idx = None if m_dev == n else row_idx
-        kw = dict(row_block_size=0, ignore_index=-100, exclude_index=-1,
-                  logit_softcap=float(wl.logit_softcap or 0.0), compute_dtype=hidden.dtype,
-                  weight_dim_first=False, row_idx=idx, n_out=n)
-        go = torch.ones(1, device=device)
-        with _lib.kernel_profile() as prof:
-            _, lse, count = native.forward(rows, weight.detach(), None, targets, **kw)
-            native.backward(rows, weight.detach(), None, targets, lse, count, go,
-                            reduction="mean", **kw)
+        if args.compaction_mode == "device":
+            row_idx, count = native.compact_rows_device(labels, -100)
+            rows, targets, _ = native.gather_loss_rows(hidden.detach(), labels, None, row_idx,
+                                                       count, -100)
+            kw = dict(m=n, row_idx=row_idx, row_count=count, n_out=n, ignore_index=-100,
+                      exclude_index=-1, logit_softcap=softcap)
+            with _lib.kernel_profile() as prof:
+                _, lse, valid, _ = native.masked_loss_forward(
+                    rows, weight.detach(), None, targets, None, want_losses=True, want_sum=False,
+                    **kw)
+                native.masked_loss_backward(rows, weight.detach(), None, targets, None, lse, valid,
+                                            go, reduction="mean", **kw)
+        else:
+            row_idx, m_dev = (None, n) if args.compaction_mode == "none" else \
+                native.compact_rows(labels, -100)
+            rows = hidden.detach() if m_dev == n else native.gather_rows(hidden.detach(), row_idx)
+            targets = labels if m_dev == n else native.gather_rows(labels, row_idx)
+            idx = None if m_dev == n else row_idx
+            kw = dict(row_block_size=0, ignore_index=-100, exclude_index=-1,
+                      logit_softcap=softcap, compute_dtype=hidden.dtype,
+                      weight_dim_first=False, row_idx=idx, n_out=n)
+            with _lib.kernel_profile() as prof:
+                _, lse, count = native.forward(rows, weight.detach(), None, targets, **kw)
+                native.backward(rows, weight.detach(), None, targets, lse, count, go,
+                                reduction="mean", **kw)
         torch.cuda.synchronize()
 
     if args.calibrate_copy:
@@ -364,7 +474,11 @@ def main() -> int:
     achieved = flops_per_launch / 1e12 / (avg_ms / 1e3)
     useful_tflops = 3.0 * contraction_tflop / (ms_per_step / 1e3)
     executed_tflops = 4.0 * contraction_tflop / (ms_per_step / 1e3)
-    plan = _lib.query_plan(m, h, v, _lib.DTYPE_BF16, True, native.PANEL_BYTES)
+    # launches are sized for the loss-bearing rows, or for all rows when the count is not
+    # read back / rows are not compacted
+    plan_rows = m if args.compaction_mode == "sync" else n
+    plan = _lib.query_plan(plan_rows, h, v, _lib.DTYPE_BF16, True, native.PANEL_BYTES)
+    traffic, traffic_note = measured_traffic(wl.name, dominant)
 
     result = {
         "metric": "fused linear-CE fwd+bwd tokens/s",
@@ -383,7 +497,10 @@ def main() -> int:
             "workload": f"{wl.name}: N={n} rows, M={m} loss-bearing, H={h}, V={v}, "
                         f"softcap={wl.logit_softcap}, seed={args.seed}",
             "input_rows_per_s": n / (ms_per_step / 1e3),
+            "compaction_mode": args.compaction_mode,
+            "panel_bytes": native.PANEL_BYTES or (1 << 30),
             "plan": plan,
+            "sources": source_fingerprint(),
         },
         "loss": loss_value,
         "tflops_useful_6MHV": useful_tflops,
@@ -403,7 +520,8 @@ def main() -> int:
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": achieved / PEAK_BF16_TFLOPS,
-            "traffic": measured_traffic(wl.name, dominant),
+            "traffic": traffic,
+            "traffic_source": traffic_note,
             "avg_launch_ms": avg_ms,
             "launches_per_step": launches,
             "flops_per_launch": flops_per_launch,

@@ -419,3 +419,30 @@ def test_label_on_the_excluded_column(gpu_device):
     assert oracle.relative_max_error(dw, rdw) <= GRAD_REL_MAX
     assert oracle.relative_max_error(db, rdb) <= GRAD_REL_MAX
     assert torch.count_nonzero(dw[exclude]) == 0 and float(db[exclude]) == 0.0
+
+
+def test_contiguous_views_at_odd_offsets(gpu_device):
+    """hidden[1:] and weight[v0:] are contiguous but, with rows that are not a
+    multiple of 16 bytes long, no longer 16-byte aligned; the reference accepts
+    any contiguous tensor (tiled_linear_cross_entropy.py:297-301)."""
+    say("offset views, float32 H=33 and bf16 H=100")
+    for dtype, h, v, tol in ((torch.float32, 33, 517, 3e-5), (torch.bfloat16, 100, 1025, GRAD_REL_MAX)):
+        gen = torch.Generator().manual_seed(h)
+        hidden_all = torch.randn(131, h, generator=gen).to(dtype)
+        weight_all = (torch.randn(v + 3, h, generator=gen) * 0.2).to(dtype)
+        labels = torch.randint(0, v, (130,), generator=gen)
+        labels[::7] = -100
+        dev = gpu_device
+        hd = hidden_all.to(dev)[1:].requires_grad_(True)
+        wd = weight_all.to(dev)[3:].requires_grad_(True)
+        assert hd.is_contiguous() and wd.is_contiguous()
+        assert hd.data_ptr() % 16 != 0 or wd.data_ptr() % 16 != 0
+        loss = tiled_linear_cross_entropy(hd, wd, labels.to(dev), dtype=dtype,
+                                          weight_layout="vocab_first")
+        loss.backward()
+        torch.cuda.synchronize()
+        ref = oracle.dense_linear_ce(hidden_all[1:], weight_all[3:], labels)
+        rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden_all[1:], weight_all[3:], labels)
+        torch.testing.assert_close(loss.detach().cpu().double(), ref, rtol=LOSS_RTOL, atol=1e-5)
+        assert oracle.relative_max_error(hd.grad.cpu(), rdh) <= tol
+        assert oracle.relative_max_error(wd.grad.cpu(), rdw) <= tol

@@ -59,6 +59,16 @@ def _ptr(tensor: Optional[torch.Tensor]) -> Optional[int]:
     return tensor.data_ptr()
 
 
+def _dense(tensor: torch.Tensor) -> torch.Tensor:
+    """Contiguous and 16-byte aligned: the MFMA kernels load 16 bytes at a time.
+    A contiguous view at an odd offset (``hidden[1:]`` with a row length that is
+    not a multiple of 16 bytes) is copied; everything else passes through."""
+    tensor = tensor.contiguous()
+    if tensor.numel() and tensor.data_ptr() % 16:
+        tensor = tensor.clone()
+    return tensor
+
+
 def _stream(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
@@ -228,7 +238,7 @@ def scatter_rows(src: torch.Tensor, row_idx: torch.Tensor, n_rows: int) -> torch
 # -------------------------------------------------------------------- forward --
 def _vocab_first(weight: torch.Tensor, weight_dim_first: bool) -> torch.Tensor:
     # The kernels read the head as [V, H]; a [H, V] head is re-laid once here.
-    return weight.t().contiguous() if weight_dim_first else weight.contiguous()
+    return weight.t().contiguous() if weight_dim_first else _dense(weight)
 
 
 def forward(
@@ -261,7 +271,7 @@ def forward(
         raise RuntimeError("weight must be a matrix")
     if weight.dtype != hidden.dtype:
         raise RuntimeError("native linear CE expects hidden and weight of one dtype")
-    hidden = hidden.contiguous()
+    hidden = _dense(hidden)
     weight = _vocab_first(weight, weight_dim_first)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
@@ -299,7 +309,7 @@ def _backward(
     compute_weight_grad, row_idx, n_out,
 ):
     device = _require_device(hidden, weight, bias, labels, lse, valid_count, grad_output, row_idx)
-    hidden = hidden.contiguous()
+    hidden = _dense(hidden)
     weight_vf = _vocab_first(weight, weight_dim_first)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
@@ -447,8 +457,8 @@ def masked_loss_forward(
         raise RuntimeError("native linear CE expects hidden and weight of one dtype")
     if not (want_losses or want_sum):
         raise RuntimeError("masked loss: nothing to compute")
-    hidden = hidden.contiguous()
-    weight = weight.contiguous()
+    hidden = _dense(hidden)
+    weight = _dense(weight)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     h = hidden.shape[1]
     v = weight.shape[0]
@@ -515,8 +525,8 @@ def masked_loss_backward(
     grad_weight | None, grad_bias | None)`` in the input dtypes."""
     device = _require_device(hidden, weight, bias, labels, token_weights, lse, valid_count,
                              grad_output, row_idx, row_count)
-    hidden = hidden.contiguous()
-    weight = weight.contiguous()
+    hidden = _dense(hidden)
+    weight = _dense(weight)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     h = hidden.shape[1]
     v = weight.shape[0]
@@ -591,8 +601,8 @@ def vocab_parallel_forward_local(
         raise RuntimeError("vocab-parallel head width mismatch")
     if weight.dtype != hidden.dtype:
         raise RuntimeError("native linear CE expects hidden and weight of one dtype")
-    hidden = hidden.contiguous()
-    weight = weight.contiguous()
+    hidden = _dense(hidden)
+    weight = _dense(weight)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
     v_local = weight.shape[0]
@@ -639,8 +649,8 @@ def vocab_parallel_backward_local(
     (reference shim, chunked_linear_ce_native.py:218-256): ``grad_hidden`` is
     this shard's partial sum, ``grad_weight`` / ``grad_bias`` cover the shard."""
     device = _require_device(hidden, weight, bias, labels, global_lse, valid_count, grad_output)
-    hidden = hidden.contiguous()
-    weight = weight.contiguous()
+    hidden = _dense(hidden)
+    weight = _dense(weight)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
     v_local = weight.shape[0]
@@ -701,8 +711,8 @@ def soft_embedding(
         raise RuntimeError("soft embedding expects hidden [N, H] and weight [V, H]")
     if weight.dtype != hidden.dtype:
         raise RuntimeError("native linear CE expects hidden and weight of one dtype")
-    hidden = hidden.contiguous()
-    weight = weight.contiguous()
+    hidden = _dense(hidden)
+    weight = _dense(weight)
     m, h = hidden.shape
     v = weight.shape[0]
     code = _dtype_code(hidden)
@@ -726,7 +736,7 @@ def soft_embedding(
 # -------------------------------------------------------------- frozen-head KL --
 def _kl_operands(draft_hidden, draft_weight, teacher_hidden, teacher_weight):
     device = _require_device(draft_hidden, draft_weight, teacher_hidden, teacher_weight)
-    tensors = [t.contiguous() for t in (draft_hidden, draft_weight, teacher_hidden,
+    tensors = [_dense(t) for t in (draft_hidden, draft_weight, teacher_hidden,
                                         teacher_weight)]
     dh, dw, th, tw = tensors
     if dh.dim() != 2 or th.dim() != 2 or dw.dim() != 2 or tw.dim() != 2:
@@ -835,8 +845,8 @@ def dflash_ce_topk_forward(
         raise RuntimeError("CE top-k expects hidden [N, D] and weight [V, D]")
     if weight.dtype != hidden.dtype:
         raise RuntimeError("native linear CE expects hidden and weight of one dtype")
-    hidden = hidden.contiguous()
-    weight = weight.contiguous()
+    hidden = _dense(hidden)
+    weight = _dense(weight)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
     v = weight.shape[0]
@@ -885,8 +895,8 @@ def dflash_ce_topk_backward(
     del row_block_size
     device = _require_device(hidden, weight, labels, lse, probabilities, top_ids, grad_loss,
                              grad_probability, grad_top_values)
-    hidden = hidden.contiguous()
-    weight = weight.contiguous()
+    hidden = _dense(hidden)
+    weight = _dense(weight)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
     v = weight.shape[0]

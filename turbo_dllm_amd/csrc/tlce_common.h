@@ -56,6 +56,22 @@ __host__ __device__ static inline int forward_vocab_splits(int n_ttiles, int n_v
   return s < n_vtiles ? s : n_vtiles;
 }
 
+// K splits of the grad_hidden contraction (`tiles` output tiles per panel): the
+// smallest factor up to max_split that fills at least 90 % of the last wave of
+// 256 workgroups and gives at least two waves (or max_split itself).  Every
+// split accumulates into a float32 slab of its own.  Shared by the host plan
+// and by the kernels when the row count is known only on the device.
+__host__ __device__ static inline int grad_hidden_k_splits(int64_t tiles, int max_split) {
+  int pick = 1;
+  for (int ks = 1; ks <= max_split; ++ks) {
+    const int64_t workgroups = tiles * ks;
+    const int64_t rounds = (workgroups + 255) / 256;
+    pick = ks;
+    if (workgroups * 10 >= rounds * 256 * 9 && (workgroups >= 512 || ks == max_split)) break;
+  }
+  return pick;
+}
+
 constexpr int kXcds = 8;  // MI355X: 8 accelerator dies, workgroups dealt round-robin
 
 // ------------------------------------------------------------- device -------

@@ -86,6 +86,7 @@ struct Plan {
   int64_t vc;         // panel columns
   int n_panels;
   int dh_ksplit;
+  int dh_max_ksplit;  // upper bound of the rule that chose dh_ksplit
 };
 
 inline int engine_class(int64_t h, int dtype) {
@@ -135,15 +136,10 @@ inline Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_gr
   // own float32 slab, summed by the final cast) by the smallest factor that
   // fills at least 90 % of the last wave.
   p.dh_ksplit = 1;
+  p.dh_max_ksplit = 1;
   if (p.engine) {
-    const int64_t tiles = (int64_t)p.n_ttiles * p.n_htiles;
-    const int64_t max_split = std::max<int64_t>(1, std::min<int64_t>(16, p.vc / p.bk / 8));
-    for (int64_t ks = 1; ks <= max_split; ++ks) {
-      const double waves = (double)(tiles * ks) / 256.0;
-      const double fill = waves / (double)ceil_div(tiles * ks, 256);
-      p.dh_ksplit = (int)ks;
-      if (fill >= 0.9 && (waves >= 2.0 || ks == max_split)) break;
-    }
+    p.dh_max_ksplit = (int)std::max<int64_t>(1, std::min<int64_t>(16, p.vc / p.bk / 8));
+    p.dh_ksplit = grad_hidden_k_splits((int64_t)p.n_ttiles * p.n_htiles, p.dh_max_ksplit);
   }
   return p;
 }
@@ -295,6 +291,8 @@ int launch_gemm(GemmArgs a, int ksplit, int cls, hipStream_t stream) {
     return rc;
   const int ksteps = a.k / E::kBK;
   a.k_per_split = (int)ceil_div(ksteps, ksplit) * E::kBK;
+  // ksplit is the number of splits launched; with a device-side row count the
+  // kernel may use fewer of them (a.slab_budget then bounds splits x slab)
   dim3 grid(xcd_grid((int64_t)a.ni * a.nj), ksplit, 1);
   ScopedTimer timer(cls, stream);
   lce_gemm_nt_kernel<E, kAKMajor, kBKMajor><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
@@ -434,6 +432,11 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     dh.c_split_stride = p.mp * h;
     dh.mode = (panel == 0) ? kStoreF32 : kAddF32;
     dh.m_dev = m_dev; dh.m_role = kRowsFollow;
+    // device-side row count: up to four K splits are launched and the kernel picks
+    // how many to use for the real count, within the slabs the plan allocated
+    const int dh_launch_ksplit =
+        m_dev == nullptr ? p.dh_ksplit : std::max(p.dh_ksplit, std::min(4, p.dh_max_ksplit));
+    dh.slab_budget = (int64_t)p.dh_ksplit * p.mp * h;
     GemmArgs dw;
     dw.m_dev = m_dev; dw.m_role = kKFollows; dw.m_round = p.bk;
     dw.k_per_split = 0;
@@ -447,7 +450,7 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
         // grad_hidden: A = weight rows [v0, v0+K) as stored (K-major), B = G
         dh.a = weight_t + v0 * h; dh.lda = h; dh.a_rows = (int)h;
         dh.k = (int)round_up(rows_valid, 64);
-        if (int rc = launch_gemm<E, true, false>(dh, p.dh_ksplit, kClassGradHidden, stream))
+        if (int rc = launch_gemm<E, true, false>(dh, dh_launch_ksplit, kClassGradHidden, stream))
           return rc;
         if (weight_grad) {
           // grad_weight: A = hidden as stored, B = G as stored, both K-major (K = token)
@@ -461,7 +464,7 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     }
     dh.a = wt + v0; dh.lda = p.vp; dh.a_rows = (int)h;
     dh.k = (int)width;
-    if (int rc = launch_gemm<E, false, false>(dh, p.dh_ksplit, kClassGradHidden, stream))
+    if (int rc = launch_gemm<E, false, false>(dh, dh_launch_ksplit, kClassGradHidden, stream))
       return rc;
     if (weight_grad) {
       dw.a = ht; dw.lda = p.mp; dw.a_rows = (int)h;
@@ -481,7 +484,7 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     ScopedTimer timer(kClassOther, stream);
     lce_finalize_grad_hidden_kernel<T><<<(int)m, 256, 0, stream>>>(
         acc32, p.dh_ksplit, p.mp * h, row_idx, (int)m, (int)h, static_cast<T*>(grad_hidden),
-        m_dev);
+        m_dev, p.n_htiles, p.tile, std::max(p.dh_ksplit, std::min(4, p.dh_max_ksplit)));
   }
   TLCE_LAUNCH_CHECK();
   return 0;

@@ -424,15 +424,17 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
         E::set(acc, j, i, fmaf(E::get(acc, j, i), p.logit_scale, b));
     }
   }
-  // workgroup-uniform: rows past v or the excluded column in this tile;
-  // wave-uniform: some lane of this wave owns a label of this tile (rare)
+  // Both selectors of the epilogue variant are workgroup-uniform (the variants
+  // contain workgroup barriers, so every wave must take the same one): rows past
+  // v or the excluded column in this tile; some lane of the workgroup owns a
+  // label of this tile (rare).
   const bool edge = (vbase + E::kTile > p.v) ||
                     (p.exclude >= vbase && p.exclude < vbase + E::kTile);
-  const bool onehot = __ballot(label_here) != 0ull;
+  const bool onehot = __syncthreads_or(label_here ? 1 : 0) != 0;
 
   const int excluded = (int)p.exclude;
   // one logit -> its entry of g (kEdge: the tile holds rows past v or the
-  // excluded column; kOnehot: some lane of this wave owns a label of the tile)
+  // excluded column; kOnehot: some lane of the workgroup owns a label of the tile)
   auto grad_of = [&](float z, int j, int row, bool vok, auto edge_tag, auto onehot_tag) -> float {
     constexpr bool kEdge = decltype(edge_tag)::value;
     constexpr bool kOnehot = decltype(onehot_tag)::value;
@@ -1027,7 +1029,21 @@ struct GemmArgs {
   // (grad_weight): k shrinks to the real count rounded up to m_round.
   const int64_t* m_dev = nullptr;
   int m_role = 0, m_round = 1;
+  int64_t slab_budget = 0;   // kRowsFollow: float32 elements all K-split slabs may take
 };
+
+// K splits and slab stride the grad_hidden contraction uses for a device-side
+// row count: the host plan's rule applied to the real number of token tiles,
+// limited to the splits launched and to the slab memory the plan allocated.
+__device__ __forceinline__ int dynamic_k_splits(int n_ttiles, int n_htiles, int tile, int h,
+                                                int launched, int64_t slab_budget,
+                                                int64_t* stride) {
+  const int64_t slab = (int64_t)n_ttiles * tile * h;
+  int ks = grad_hidden_k_splits((int64_t)n_ttiles * n_htiles, launched);
+  while (ks > 1 && ks * slab > slab_budget) --ks;
+  *stride = slab;
+  return ks;
+}
 enum { kRowsFollow = 1, kKFollows = 2 };
 
 template <class E, bool kAKMajor, bool kBKMajor>
@@ -1038,6 +1054,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
     if (p.m_role == kRowsFollow) {
       p.c_rows = effective_rows(p.c_rows, p.m_dev);
       p.nj = (p.c_rows + E::kTile - 1) / E::kTile;
+      const int ks = dynamic_k_splits(p.nj, p.ni, E::kTile, (int)p.ldc, (int)gridDim.y,
+                                      p.slab_budget, &p.c_split_stride);
+      if ((int)blockIdx.y >= ks) return;
+      p.k_per_split = (p.k / E::kBK + ks - 1) / ks * E::kBK;
     } else if (p.m_role == kKFollows) {
       const int rows = effective_rows(p.k, p.m_dev);
       p.k = (rows + p.m_round - 1) / p.m_round * p.m_round;
@@ -1149,9 +1169,15 @@ template <typename T>
 __global__ __launch_bounds__(256) void lce_finalize_grad_hidden_kernel(
     const float* __restrict__ acc32, int n_splits, int64_t split_stride,
     const int64_t* __restrict__ row_idx, int m, int h, T* __restrict__ out,
-    const int64_t* __restrict__ m_dev) {
+    const int64_t* __restrict__ m_dev, int n_htiles, int tile, int launched_splits) {
   const int r = blockIdx.x;
-  if (r >= effective_rows(m, m_dev)) return;
+  if (m_dev != nullptr) {
+    // the splits and slab stride the contraction derived from the real row count
+    m = effective_rows(m, m_dev);
+    n_splits = dynamic_k_splits((m + tile - 1) / tile, n_htiles, tile, h, launched_splits,
+                                (int64_t)n_splits * split_stride, &split_stride);
+  }
+  if (r >= m) return;
   const int64_t o = (row_idx != nullptr) ? row_idx[r] : (int64_t)r;
   const float* src = acc32 + (int64_t)r * h;
   T* dst = out + o * h;
