@@ -56,10 +56,20 @@ def test_workspace_sizes_and_plan():
     assert plan["n_panels"] * plan["panel_columns"] >= 151936
     assert plan["grad_hidden_k_splits"] == 1
     fwd = lib.tlce_forward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16)
-    assert fwd == 2 * 8 * 32768 * 4  # (max, sum) float32 partials only: no logits buffer
+    assert fwd == 2 * 8 * 32768 * 4  # (max, sum) float32 partials only: the forward stores no logits
+    # the backward stages rounded logit GRADIENTS in one bounded vocabulary panel (1 GiB by
+    # default: 16384 of the 151936 columns, 5.4 % of the float32 logits matrix the reference
+    # blocks through); it is a [rows, panel] buffer, not "no buffer"
     bwd = lib.tlce_backward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16, 1, 0, 0)
     logits_bytes = 32768 * 151936 * 4
+    panel_bytes = plan["panel_columns"] * 32768 * 2
+    assert panel_bytes == 1 << 30 and panel_bytes * 18 < logits_bytes
     assert bwd < logits_bytes // 4
+    # the device-side row count needs room for whatever plan a smaller count selects
+    dyn = lib.tlce_masked_loss_forward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16, 1)
+    assert dyn == 2 * 1024 * 256 * 4 + 32768 * 4
+    assert lib.tlce_masked_loss_forward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16, 0) \
+        == fwd + 32768 * 4
     frozen = lib.tlce_backward_workspace_bytes(32768, 4096, 151936, _lib.DTYPE_BF16, 0, 0, 0)
     assert frozen <= bwd
     # float32 grad_hidden accumulators + one bf16 panel + per-row scales, nothing else
