@@ -12,8 +12,11 @@ import torch
 import linear_ce_oracle as oracle
 from turbo_dllm_amd.dflash_kl import frozen_linear_kl
 from turbo_dllm_amd.dflash_linear_topk import frozen_linear_ce_topk
+from turbo_dllm_amd.layers import VocabParallelLinear
+from turbo_dllm_amd.loss import masked_token_loss
 from turbo_dllm_amd.streaming_soft_embedding import streaming_soft_embedding
-from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+from turbo_dllm_amd.tiled_linear_cross_entropy import (compaction_mode,
+                                                       tiled_linear_cross_entropy)
 
 pytestmark = pytest.mark.gpu
 
@@ -73,6 +76,36 @@ def test_random_case(gpu_device, case):
         assert oracle.relative_max_error(w.grad.cpu(), rdw) <= tol
     if bias is not None:
         assert oracle.relative_max_error(b.grad.cpu(), rdb) <= tol
+
+    # the loss method around the operator, with the row count read back, kept on the
+    # device, or rows left in place (the capacity-sized launches of the device mode
+    # meet every count around the tile edges here, down to one row)
+    mode = ("sync", "device", "none")[case % 3]
+    multiplier = (None, 0.5, 1.75)[(case // 3) % 3]
+    head = VocabParallelLinear(h, v, bias=bias is not None).to(device=dev, dtype=dtype)
+    with torch.no_grad():
+        head.weight.copy_(weight.to(dev))
+        if bias is not None:
+            head.bias.copy_(bias.to(dev))
+    weights = torch.rand(n, generator=gen) + 0.5
+    xm = hidden.to(dev).requires_grad_(True)
+    with compaction_mode(mode):
+        total = masked_token_loss(xm, labels.to(dev), weights.to(dev), head,
+                                  valid_token_count=3.0, mask_token_id=exclude,
+                                  exclude_mask_token=exclude is not None,
+                                  output_multiplier=multiplier, logit_softcap=softcap,
+                                  loss_scale=1.5)
+        total.backward()
+    torch.cuda.synchronize()
+    mkw = dict(bias=bias, exclude_index=exclude, output_multiplier=multiplier,
+               logit_softcap=softcap, loss_scale=1.5)
+    mref = oracle.masked_token_loss(hidden, weight, labels, weights, 3.0, **mkw)
+    mdh, mdw, mdb = oracle.masked_token_loss_grads(hidden, weight, labels, weights, 3.0, **mkw)
+    torch.testing.assert_close(total.detach().cpu().double(), mref.double(), rtol=ltol, atol=ltol)
+    assert oracle.relative_max_error(xm.grad.cpu(), mdh) <= tol, mode
+    assert oracle.relative_max_error(head.weight.grad.cpu(), mdw) <= tol, mode
+    if bias is not None:
+        assert oracle.relative_max_error(head.bias.grad.cpu(), mdb) <= tol, mode
 
     # soft embedding
     soft = streaming_soft_embedding(hidden.to(dev), weight.to(dev), row_chunk_size=64,

@@ -389,16 +389,11 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
   const T* weight = static_cast<const T*>(p.weight);
   typename E::Acc acc;
   const int vbase = p.v0 + pv * E::kTile;
-  eng.mainloop_set(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
-
-  // the bias add applies the logit multiplier itself (z = multiplier * dot + bias)
-  const float raw_scale = kBias ? 1.0f : p.logit_scale;
-  const float inv_cap = kSoftcap ? raw_scale / p.softcap : 0.0f;
-  const float log2e_scaled = TLCE_LOG2E * raw_scale;
-  const float inv_logit_scale = kBias ? 1.0f / p.logit_scale : 1.0f;
   // per owned token column: row of its label inside this tile (-1: none here),
   // lse in base-2 units, and the loss scale (0 for ignored and padding rows,
-  // which zeroes their whole column of g without a per-element test)
+  // which zeroes their whole column of g without a per-element test).  Loaded
+  // before the contraction so that their latency passes under it instead of
+  // standing between the last MFMA and the gradient math.
   int label_row[E::kCols];
   float lse2[E::kCols], scale[E::kCols];
   bool label_here = false;
@@ -415,6 +410,13 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
     lse2[j] = p.lse[rc] * TLCE_LOG2E;
     scale[j] = live ? p.scale[rc] : 0.0f;
   }
+  eng.mainloop_set(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+
+  // the bias add applies the logit multiplier itself (z = multiplier * dot + bias)
+  const float raw_scale = kBias ? 1.0f : p.logit_scale;
+  const float inv_cap = kSoftcap ? raw_scale / p.softcap : 0.0f;
+  const float log2e_scaled = TLCE_LOG2E * raw_scale;
+  const float inv_logit_scale = kBias ? 1.0f / p.logit_scale : 1.0f;
   if (kBias) {
 #pragma unroll
     for (int i = 0; i < E::kRows; ++i) {
@@ -630,14 +632,11 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
   E eng;
   typename E::Acc acc;
   const int vbase = p.v0 + pv * E::kTile;
-  eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
-                   static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
-
-  const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
   constexpr bool grad = kGrad;   // p.mode, fixed at compile time: no mode test per group of 4
   float lse2[E::kCols], scale[E::kCols], partial[E::kCols], tsum[E::kCols];
   float tile_max[E::kCols], tile_sum[E::kCols];
   bool live[E::kCols];
+  // the per-row operands are loaded before the contraction: their latency passes under it
 #pragma unroll
   for (int j = 0; j < E::kCols; ++j) {
     const int r = tt * E::kTile + eng.col(j);
@@ -650,6 +649,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
     tile_max[j] = -INFINITY;
     tile_sum[j] = 0.0f;
   }
+  eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
+                   static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+
+  const float inv_cap = kSoftcap ? 1.0f / p.softcap : 0.0f;
   if (!grad) {
     // maxima of the capped draft logits per owned column (base-2 units) for the
     // tile's softmax partial; the capped values replace the raw accumulators
