@@ -165,7 +165,24 @@ def measure_compaction_gather(torch, native, device, n, h, hidden):
     stop.record()
     torch.cuda.synchronize()
     gather_ms = start.elapsed_time(stop) / reps
+    # the same pass without any host read-back: scan, then ONE gather of hidden rows, labels
+    # and loss weights with the count read on the device
+    weights = torch.ones(n, device=device)
+    for _ in range(3):
+        idx_all, count = native.compact_rows_device(labels, -100)
+        native.gather_loss_rows(hidden, labels, weights, idx_all, count, -100)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        idx_all, count = native.compact_rows_device(labels, -100)
+        native.gather_loss_rows(hidden, labels, weights, idx_all, count, -100)
+    stop.record()
+    torch.cuda.synchronize()
+    device_ms = start.elapsed_time(stop) / reps
+    device_bytes = 8 * n + 8 * m + 4 * m * h + 24 * m
     return {
+        "device_count_ms": device_ms, "device_count_algorithmic_bytes": device_bytes,
+        "device_count_GB_per_s": device_bytes / device_ms / 1e6,
         "rows": n, "loss_rows": m, "ms": ms, "algorithmic_bytes": nbytes,
         "GB_per_s": nbytes / ms / 1e6,
         "gather_only_ms": gather_ms,
@@ -253,6 +270,79 @@ def library_gemm_reference(torch, device, h, v, rows=8192, panel=16384, reps=5):
     return result
 
 
+def bench_masked_loss(args) -> int:
+    """The loss method around the operator (output multiplier, mask token excluded,
+    per-token weights, / valid_token_count) on the block-diffusion shard: the fused
+    path against the reference's sequence of calls on the same kernels."""
+    import torch
+
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    from turbo_dllm_amd import workloads
+    from turbo_dllm_amd.compaction import compact_valid_loss_rows
+    from turbo_dllm_amd.layers import VocabParallelLinear
+    from turbo_dllm_amd.loss import masked_token_loss
+    from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+
+    device = torch.device("cuda:0")
+    native.verify_device(0)
+    wl = workloads.block_diffusion_shard(seed=args.seed)
+    n, m = wl.n_rows, wl.n_loss_rows
+    h, v = wl.hidden.shape[1], wl.weight.shape[0]
+    head = VocabParallelLinear(h, v, bias=False).to(device=device, dtype=torch.bfloat16)
+    with torch.no_grad():
+        head.weight.copy_(wl.weight.to(device))
+    hidden = wl.hidden.to(device).requires_grad_(True)
+    labels = wl.labels.to(device)
+    weights = (torch.rand(n, generator=torch.Generator().manual_seed(args.seed)) + 0.5).to(device)
+
+    def fused():
+        hidden.grad = None
+        head.weight.grad = None
+        loss = masked_token_loss(hidden, labels, weights, head, valid_token_count=float(m),
+                                 mask_token_id=5, output_multiplier=0.5)
+        loss.backward()
+        return loss
+
+    def reference_sequence():          # nemotron/model.py:2078-2151, unfused
+        hidden.grad = None
+        head.weight.grad = None
+        rows, targets, w = compact_valid_loss_rows(hidden, labels, weights, ignore_index=-100)
+        rows = rows * 0.5
+        token_losses = tiled_linear_cross_entropy(rows, head.weight, targets, reduction="none",
+                                                  exclude_index=5, dtype=rows.dtype,
+                                                  weight_layout="vocab_first")
+        loss = (token_losses.reshape(-1).float() * w).sum() / float(m)
+        loss.backward()
+        return loss
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(args.steps):
+            loss = fn()
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / args.steps, float(loss.detach())
+
+    ms, loss = timed(fused)
+    ref_ms, ref_loss = timed(reference_sequence)
+    print(json.dumps({
+        "metric": "masked-token loss fwd+bwd tokens/s", "value": m / (ms / 1e3),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"masked_token_loss on {wl.name}: N={n} rows, M={m} loss-bearing, "
+                               f"H={h}, V={v}, multiplier 0.5, mask token excluded, seed={args.seed}",
+                   "compaction_mode": args.compaction_mode},
+        "loss": loss,
+        "reference_sequence_ms_per_step": ref_ms, "reference_sequence_loss": ref_loss,
+    }), flush=True)
+    return 0
+
+
 def bench_next_objective(args) -> int:
     """The objectives built on the same kernels: frozen-head forward KL
     (forward + backward) and the streaming soft embedding (forward only)."""
@@ -337,9 +427,11 @@ def bench_next_objective(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--objective", choices=("ce", "kl", "soft_embedding", "ce_topk"), default="ce",
-                    help="ce: the headline fused linear cross-entropy (default); kl / "
-                         "soft_embedding: the objectives built on the same kernels")
+    ap.add_argument("--objective",
+                    choices=("ce", "masked_loss", "kl", "soft_embedding", "ce_topk"), default="ce",
+                    help="ce: the headline fused linear cross-entropy (default); masked_loss: the "
+                         "loss method around it on the block-diffusion shard; kl / soft_embedding "
+                         "/ ce_topk: the objectives built on the same kernels")
     ap.add_argument("--rows", type=int, default=8192, help="rows for --objective kl / soft_embedding")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
@@ -378,6 +470,8 @@ def main() -> int:
         return 1
     set_compaction_mode(args.compaction_mode)
     native.PANEL_BYTES = args.panel_mib << 20
+    if args.objective == "masked_loss":
+        return bench_masked_loss(args)
     if args.objective != "ce":
         return bench_next_objective(args)
     device = torch.device("cuda:0")
