@@ -96,3 +96,26 @@ def test_bad_arguments_report_errors_without_a_gpu():
     with pytest.raises(RuntimeError, match="bad shape"):
         _lib.check(rc, "tlce_query_plan")
     assert lib.tlce_forward_workspace_bytes(-1, 8, 8, _lib.DTYPE_BF16) == -1
+
+
+def test_masked_loss_entry_points_validate_before_touching_a_gpu():
+    lib = _lib.library()
+    fake = 4096          # aligned, never dereferenced: validation fails first
+    common = (fake, fake, None, fake, None, None, None, 8, 8, 64, 100, _lib.DTYPE_BF16)
+    # the logit multiplier must be positive (the kernels keep maxima of unscaled dot products)
+    rc = lib.tlce_masked_loss_forward(*common, -100, -1, 0.0, -0.5, None, fake, fake, fake,
+                                      fake, 1 << 20, None)
+    assert rc != 0 and "multiplier must be positive" in _lib.last_error()
+    rc = lib.tlce_masked_loss_backward(fake, fake, None, fake, None, None, None, fake, None, fake,
+                                       8, 8, 64, 100, _lib.DTYPE_BF16, _lib.REDUCTION_SUM,
+                                       -100, -1, 0.0, 0.0, fake, None, None, 0, fake, 1 << 30, None)
+    assert rc != 0 and "multiplier must be positive" in _lib.last_error()
+    # neither per-token losses nor the weighted sum asked for
+    rc = lib.tlce_masked_loss_forward(*common, -100, -1, 0.0, 1.0, None, fake, fake, None,
+                                      fake, 1 << 20, None)
+    assert rc != 0 and "neither" in _lib.last_error()
+    # gather: the weights go in and out together
+    rc = lib.tlce_gather_loss_rows(fake, fake, fake, fake, fake, 8, 64, 128, -100, fake, fake,
+                                   None, None)
+    assert rc != 0 and "weights" in _lib.last_error()
+    assert lib.tlce_masked_loss_forward_workspace_bytes(-1, 8, 8, _lib.DTYPE_BF16, 0) == -1

@@ -251,3 +251,11 @@ def test_device_row_count_forward_is_bit_equal_to_the_exact_plan(gpu_device):
     idx, count = native.compact_rows_device(labels, -100)
     assert int(count) == wl.n_loss_rows
     assert idx[: wl.n_loss_rows].cpu().tolist() == oracle.compact_rows(wl.labels.numpy()).tolist()
+
+
+def test_non_positive_multiplier_takes_the_reference_sequence(gpu_device):
+    """The fused kernels need a positive logit multiplier; any other value goes
+    through the scaled copy of the hidden states, as the reference does."""
+    wl = workloads.small_head(seed=12, scale=16)
+    say("masked_token_loss, multiplier -0.5", "N", wl.n_rows, "M", wl.n_loss_rows)
+    check_masked_loss(gpu_device, wl, mode="sync", multiplier=-0.5)

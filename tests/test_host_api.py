@@ -251,3 +251,36 @@ def test_compaction_and_loss_wrapper_on_host():
     empty.backward()
     with pytest.raises(NotImplementedError):
         VocabParallelLinear(8, 20, tensor_parallel_size=2)
+
+
+def test_native_token_cross_entropy_on_host_and_compaction_modes():
+    from turbo_dllm_amd.loss import native_token_cross_entropy
+    from turbo_dllm_amd.tiled_linear_cross_entropy import (COMPACTION_MODES, compaction_mode,
+                                                           get_compaction_mode,
+                                                           set_compaction_mode)
+
+    torch.manual_seed(8)
+    hidden = torch.randn(7, 8, requires_grad=True)
+    labels = torch.randint(0, 20, (7,))
+    head = torch.nn.Linear(8, 20, bias=True)
+    losses = native_token_cross_entropy(hidden, labels, head, output_multiplier=0.5,
+                                        logit_softcap=6.0)
+    logits = F.linear(hidden.detach() * 0.5, head.weight, head.bias)
+    logits = torch.tanh(logits / 6.0) * 6.0
+    ref = F.cross_entropy(logits, labels, reduction="none")
+    assert losses.shape == labels.shape and losses.dtype == torch.float32
+    torch.testing.assert_close(losses, ref, atol=2e-5, rtol=2e-5)
+    losses.sum().backward()
+    assert hidden.grad is not None and head.weight.grad is not None
+
+    # the compaction mode is a process-wide setting with a scoped form
+    assert COMPACTION_MODES == ("sync", "device", "none") and get_compaction_mode() == "sync"
+    with compaction_mode("device"):
+        assert get_compaction_mode() == "device"
+        with compaction_mode("none"):
+            assert get_compaction_mode() == "none"
+        assert get_compaction_mode() == "device"
+    assert get_compaction_mode() == "sync"
+    with pytest.raises(ValueError):
+        set_compaction_mode("lazy")
+    assert get_compaction_mode() == "sync"
