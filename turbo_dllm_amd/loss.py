@@ -146,9 +146,11 @@ class _FusedTokenLosses(torch.autograd.Function):
         )
 
 
-def _fused_path_applies(hidden, weight, bias, labels, multiplier) -> bool:
+def _fused_path_applies(hidden, weight, bias, labels, multiplier, loss_weights=None) -> bool:
     if not (hidden.is_cuda and weight.is_cuda and labels.is_cuda):
         return False
+    if loss_weights is not None and (not loss_weights.is_cuda or loss_weights.requires_grad):
+        return False   # the fused path forms no gradient for the weights
     if hidden.dtype not in _DEVICE_DTYPES or weight.dtype != hidden.dtype:
         return False
     if bias is not None and (not bias.is_cuda or bias.dtype != hidden.dtype):
@@ -187,7 +189,7 @@ def masked_token_loss(
     bias = bias if isinstance(bias, torch.Tensor) else None
     multiplier = 1.0 if output_multiplier is None else float(output_multiplier)
     if isinstance(weight, torch.Tensor) and weight.dim() == 2 and _fused_path_applies(
-            hidden, weight, bias, labels, multiplier):
+            hidden, weight, bias, labels, multiplier, loss_weights):
         mode = get_compaction_mode()
         if mode == "sync" and labels.numel() == 0:
             return zero_loss_with_module_parameters(hidden, output_head) / valid_token_count * float(
