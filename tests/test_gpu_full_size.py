@@ -367,3 +367,25 @@ def test_soft_embedding_full_size(gpu_device):
     err = oracle.relative_max_error(out[pick], ref)
     say("rel max err", f"{err:.2e}")
     assert err <= 2e-2
+
+
+def test_small_head_full_size_against_the_dense_oracle(gpu_device):
+    """The CPU-runnable configuration (2048 rows, H=1024, V=32000, half the rows
+    loss-bearing) at full size: the whole loss and both gradients against the
+    dense float32 oracle."""
+    wl = workloads.small_head(seed=14)
+    say(wl.name, "N", wl.n_rows, "M", wl.n_loss_rows)
+    hidden = wl.hidden.to(gpu_device).requires_grad_(True)
+    weight = wl.weight.to(gpu_device).requires_grad_(True)
+    loss = tiled_linear_cross_entropy(hidden, weight, wl.labels.to(gpu_device), reduction="mean",
+                                      dtype=torch.bfloat16, weight_layout="vocab_first")
+    loss.backward()
+    torch.cuda.synchronize()
+    ref = oracle.dense_linear_ce(wl.hidden, wl.weight, wl.labels, dtype=torch.float32)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(wl.hidden, wl.weight, wl.labels,
+                                               dtype=torch.float32)
+    rel = abs(float(loss.detach()) - float(ref)) / abs(float(ref))
+    err_h = oracle.relative_max_error(hidden.grad.cpu(), rdh)
+    err_w = oracle.relative_max_error(weight.grad.cpu(), rdw)
+    say(f"loss rel {rel:.2e} dH {err_h:.2e} dW {err_w:.2e}")
+    assert rel <= 1e-3 and err_h <= 2e-2 and err_w <= 2e-2
