@@ -460,7 +460,7 @@ def main() -> int:
 
     import torch
 
-    from turbo_dllm_amd import _lib
+    from turbo_dllm_amd import _lib, options
     from turbo_dllm_amd import chunked_linear_ce_native as native
     from turbo_dllm_amd.tiled_linear_cross_entropy import (set_compaction_mode,
                                                            tiled_linear_cross_entropy)
@@ -469,7 +469,7 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 1
     set_compaction_mode(args.compaction_mode)
-    native.PANEL_BYTES = args.panel_mib << 20
+    options.set_panel_bytes(args.panel_mib << 20)
     if args.objective == "masked_loss":
         return bench_masked_loss(args)
     if args.objective != "ce":
@@ -514,11 +514,11 @@ def main() -> int:
     softcap = float(wl.logit_softcap or 0.0)
     go = torch.ones(1, device=device)
     with torch.no_grad():
-        if args.compaction_mode == "device":
-            row_idx, count = native.compact_rows_device(labels, -100)
-            rows, targets, _ = native.gather_loss_rows(hidden.detach(), labels, None, row_idx,
-                                                       count, -100)
-            kw = dict(m=n, row_idx=row_idx, row_count=count, n_out=n, ignore_index=-100,
+        # the same operands and entry points the loss API uses for this compaction mode
+        rows, targets, _, row_idx, count, m_rows = native.compact_loss_rows(
+            hidden.detach(), labels, None, -100, args.compaction_mode)
+        if count is not None:
+            kw = dict(m=m_rows, row_idx=row_idx, row_count=count, n_out=n, ignore_index=-100,
                       exclude_index=-1, logit_softcap=softcap)
             with _lib.kernel_profile() as prof:
                 _, lse, valid, _ = native.masked_loss_forward(
@@ -527,17 +527,12 @@ def main() -> int:
                 native.masked_loss_backward(rows, weight.detach(), None, targets, None, lse, valid,
                                             go, reduction="mean", **kw)
         else:
-            row_idx, m_dev = (None, n) if args.compaction_mode == "none" else \
-                native.compact_rows(labels, -100)
-            rows = hidden.detach() if m_dev == n else native.gather_rows(hidden.detach(), row_idx)
-            targets = labels if m_dev == n else native.gather_rows(labels, row_idx)
-            idx = None if m_dev == n else row_idx
             kw = dict(row_block_size=0, ignore_index=-100, exclude_index=-1,
                       logit_softcap=softcap, compute_dtype=hidden.dtype,
-                      weight_dim_first=False, row_idx=idx, n_out=n)
+                      weight_dim_first=False, row_idx=row_idx, n_out=n)
             with _lib.kernel_profile() as prof:
-                _, lse, count = native.forward(rows, weight.detach(), None, targets, **kw)
-                native.backward(rows, weight.detach(), None, targets, lse, count, go,
+                _, lse, valid = native.forward(rows, weight.detach(), None, targets, **kw)
+                native.backward(rows, weight.detach(), None, targets, lse, valid, go,
                                 reduction="mean", **kw)
         torch.cuda.synchronize()
 
@@ -571,7 +566,7 @@ def main() -> int:
     # launches are sized for the loss-bearing rows, or for all rows when the count is not
     # read back / rows are not compacted
     plan_rows = m if args.compaction_mode == "sync" else n
-    plan = _lib.query_plan(plan_rows, h, v, _lib.DTYPE_BF16, True, native.PANEL_BYTES)
+    plan = _lib.query_plan(plan_rows, h, v, _lib.DTYPE_BF16, True, options.get_panel_bytes())
     traffic, traffic_note = measured_traffic(wl.name, dominant)
 
     result = {
@@ -592,7 +587,7 @@ def main() -> int:
                         f"softcap={wl.logit_softcap}, seed={args.seed}",
             "input_rows_per_s": n / (ms_per_step / 1e3),
             "compaction_mode": args.compaction_mode,
-            "panel_bytes": native.PANEL_BYTES or (1 << 30),
+            "panel_bytes": options.get_panel_bytes() or (1 << 30),
             "plan": plan,
             "sources": source_fingerprint(),
         },

@@ -79,6 +79,15 @@ int tlce_compact_rows(const int64_t* labels, int64_t n, int64_t ignore_index,
                       int64_t* row_idx_out, int64_t* count_out,
                       void* workspace, int64_t workspace_bytes, void* stream);
 
+/* The same scan over a boolean mask: the ascending indices of mask[i] != 0
+ * (one byte per position, e.g. a torch.bool tensor) and their count.  Device
+ * counterpart of `torch.nonzero(supervised_mask.reshape(-1)).flatten()` at the
+ * DFlash loss call sites (dllm_parallel/core/models/backbones/dflash/model.py:870-871,
+ * dflash2.py:577-578).  Workspace: tlce_compact_workspace_bytes(n). */
+int tlce_compact_mask(const uint8_t* mask, int64_t n, int64_t* row_idx_out,
+                      int64_t* count_out, void* workspace, int64_t workspace_bytes,
+                      void* stream);
+
 /* dst[r, :] = src[row_idx[r], :] for r < m; rows are `row_bytes` long and
  * contiguous in both buffers (index_select along dim 0). */
 int tlce_gather_rows(const void* src, const int64_t* row_idx, int64_t m,
@@ -97,11 +106,11 @@ int tlce_scatter_rows(const void* src, const int64_t* row_idx, int64_t m,
  *   weights_dst[r] = weights_src[row_idx[r]]   (weights optional: both NULL or neither);
  * the rows from *row_count up to the next multiple of 64 (at most padded_rows)
  * become zero rows with label ignore_index and weight 0.  row_idx and
- * row_count are what tlce_compact_rows wrote; `capacity` is the length of the
- * source (the most rows there can be), hidden_dst holds padded_rows >= capacity
- * rows of row_bytes bytes, labels_dst / weights_dst
- * padded_rows entries.  Rows past that stay untouched: consumers given
- * row_count never read them. */
+ * row_count are what tlce_compact_rows wrote; `capacity` is the number of entries
+ * row_idx holds (the most rows there can be; a *row_count outside [0, capacity]
+ * is clamped to it), hidden_dst holds padded_rows >= capacity rows of row_bytes
+ * bytes, labels_dst / weights_dst padded_rows entries.  Rows past that stay
+ * untouched: consumers given row_count never read them. */
 int tlce_gather_loss_rows(const void* hidden_src, const int64_t* labels_src,
                           const float* weights_src, const int64_t* row_idx,
                           const int64_t* row_count, int64_t capacity,
@@ -367,6 +376,22 @@ int tlce_ce_topk_backward(const void* hidden, const void* weight,
                           float logit_softcap, void* grad_hidden,
                           int64_t panel_bytes, void* workspace,
                           int64_t workspace_bytes, void* stream);
+
+/* ---- per-sample loss numerators of the DFlash loss method -----------------
+ * Replaces `numerators.scatter_add_(0, sample_indices, token_loss * position_weights)`
+ * with sample_indices = valid_indices // tokens_per_sample
+ * (dllm_parallel/core/models/backbones/dflash/model.py:918-937):
+ *   out[s] = sum of values[r] * weights[r] over the compacted rows r whose
+ *            position row_idx[r] lies in [s * segment_length, (s + 1) * segment_length)
+ * for s < n_segments, float32.  row_idx (int64, ascending, m entries: what
+ * tlce_compact_mask / tlce_compact_rows wrote) makes each sample's rows one
+ * contiguous run, which one workgroup adds in a fixed order: no atomics, the
+ * same bits on every run.  weights == NULL: plain sums.  row_count (device
+ * int64, optional): the real number of rows when m is only a capacity. */
+int tlce_segment_weighted_sum(const float* values, const float* weights,
+                              const int64_t* row_idx, const int64_t* row_count,
+                              int64_t m, int64_t segment_length, int64_t n_segments,
+                              float* out, void* stream);
 
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be

@@ -38,6 +38,15 @@ What each function follows in the reference (paths relative to its tree):
                            per-token CE * loss weights, / valid_token_count * loss scale
                            (distributed_block_diffusion_loss,
                            dllm_parallel/core/models/backbones/nemotron/model.py:2084-2151).
+  dflash_token_loss(_grads) the DFlash loss method: nonzero(supervised_mask), index_select
+                           of hidden / targets / position weights, per-token loss
+                           (cross entropy for "paper_ce", KL(teacher || draft) for
+                           "speculators_kl"), per-sample numerators by scatter-add,
+                           / (normalization_count + 1e-5), mean over samples, * scale
+                           (distributed_dflash_loss,
+                           dllm_parallel/core/models/backbones/dflash/model.py:862-960).
+  segment_weighted_sum     the scatter-add of that method on its own
+                           (dflash/model.py:918-937), by a Python loop.
   combine_vocab_shards     the MAX / SUM reductions over shards and the loss of
                            dllm_parallel/core/parallel/tensor_parallel/cross_entropy.py:238-252.
 
@@ -51,8 +60,11 @@ tests/golden/, and against the seeded cases of the reference's own test file
 stored vectors and compare to the same library routines.  The two shard
 functions are pinned by the identity that the statistics of any split of the
 vocabulary combine to the dense lse / loss of the unsplit head, by brute force
-on a tiny case, and by the special values of the excluded column.  No function
-here is "parity unpinned".
+on a tiny case, and by the special values of the excluded column.  The DFlash
+loss method is pinned against the sequence of library calls the reference's
+method makes (torch.nonzero, index_select, F.cross_entropy / F.kl_div,
+scatter_add_) with autograd through it, and against a per-sample Python loop.
+No function here is "parity unpinned".
 """
 
 from __future__ import annotations
@@ -434,3 +446,100 @@ def masked_token_loss_grads(
         h, weight, labels.reshape(-1), per_token, bias=bias, reduction="none",
         exclude_index=exclude_index, logit_softcap=logit_softcap, dtype=dtype)
     return (grad_scaled * mult).reshape(hidden.shape), grad_weight, grad_bias
+
+
+def segment_weighted_sum(values, weights, row_idx, segment_length: int, n_segments: int):
+    """out[s] = sum of values[r] * weights[r] over the rows whose position
+    row_idx[r] lies in sample s (float64, plain Python loop)."""
+    out = [0.0] * n_segments
+    for r in range(len(row_idx)):
+        s = int(row_idx[r]) // int(segment_length)
+        out[s] += float(values[r]) * (1.0 if weights is None else float(weights[r]))
+    return torch.tensor(out, dtype=torch.float64)
+
+
+def _dflash_rows(hidden_states, supervised_mask, position_weights, dtype):
+    keep = supervised_mask.reshape(-1).bool()
+    idx = torch.nonzero(keep, as_tuple=False).flatten()
+    rows = hidden_states.reshape(-1, hidden_states.shape[-1])[idx]
+    weights = position_weights.reshape(-1)[idx].to(dtype)
+    return idx, rows, weights
+
+
+def dflash_token_loss(
+    hidden_states: torch.Tensor,
+    target_token_ids: torch.Tensor,
+    supervised_mask: torch.Tensor,
+    position_weights: torch.Tensor,
+    draft_weight: torch.Tensor,
+    normalization_count: torch.Tensor,
+    *,
+    loss_kind: str,
+    teacher_hidden_states: Optional[torch.Tensor] = None,
+    teacher_weight: Optional[torch.Tensor] = None,
+    logit_softcap: Optional[float] = None,
+    loss_scale: float = 1.0,
+    dtype: torch.dtype = torch.float64,
+):
+    """mean_b( sum_{r in sample b} loss_r * w_r / (normalization_count[b] + 1e-5) ) * loss_scale
+    over the supervised positions of a [B, T] batch (dflash/model.py:862-960).
+    ``teacher_hidden_states`` are taken as already normalised (the reference
+    applies its verifier norm, a module outside this path, just before)."""
+    batch, tokens = supervised_mask.shape
+    idx, rows, weights = _dflash_rows(hidden_states, supervised_mask, position_weights, dtype)
+    if idx.numel() == 0:
+        return torch.zeros((), dtype=dtype)
+    if loss_kind == "paper_ce":
+        labels = target_token_ids.reshape(-1)[idx]
+        token_loss = dense_linear_ce(rows, draft_weight, labels, reduction="none",
+                                     logit_softcap=logit_softcap, dtype=dtype)
+    elif loss_kind == "speculators_kl":
+        teacher = teacher_hidden_states.reshape(-1, teacher_hidden_states.shape[-1])[idx]
+        token_loss = dense_frozen_kl(rows, draft_weight, teacher, teacher_weight,
+                                     logit_softcap=logit_softcap, dtype=dtype)
+    else:
+        raise ValueError(f"unsupported DFlash loss {loss_kind!r}")
+    numerators = torch.zeros(batch, dtype=dtype)
+    numerators.scatter_add_(0, idx // tokens, token_loss.to(dtype) * weights)
+    return (numerators / (normalization_count.to(dtype) + 1.0e-5)).mean() * float(loss_scale)
+
+
+def dflash_token_loss_grads(
+    hidden_states: torch.Tensor,
+    target_token_ids: torch.Tensor,
+    supervised_mask: torch.Tensor,
+    position_weights: torch.Tensor,
+    draft_weight: torch.Tensor,
+    normalization_count: torch.Tensor,
+    *,
+    loss_kind: str,
+    teacher_hidden_states: Optional[torch.Tensor] = None,
+    teacher_weight: Optional[torch.Tensor] = None,
+    logit_softcap: Optional[float] = None,
+    loss_scale: float = 1.0,
+    dtype: torch.dtype = torch.float64,
+):
+    """Analytic (grad_hidden_states, grad_draft_weight) of ``dflash_token_loss``
+    (grad_draft_weight is None for the KL, whose heads are frozen): the per-token
+    scale is w_r / (normalization_count[b_r] + 1e-5) / B * loss_scale."""
+    batch, tokens = supervised_mask.shape
+    idx, rows, weights = _dflash_rows(hidden_states, supervised_mask, position_weights, dtype)
+    grad_hidden = torch.zeros(hidden_states.reshape(-1, hidden_states.shape[-1]).shape, dtype=dtype)
+    if idx.numel() == 0:
+        return grad_hidden.reshape(hidden_states.shape), None
+    per_token = weights / (normalization_count.to(dtype)[idx // tokens] + 1.0e-5) / batch \
+        * float(loss_scale)
+    if loss_kind == "paper_ce":
+        labels = target_token_ids.reshape(-1)[idx]
+        grad_rows, grad_weight, _ = dense_linear_ce_grads(
+            rows, draft_weight, labels, per_token, reduction="none",
+            logit_softcap=logit_softcap, dtype=dtype)
+    elif loss_kind == "speculators_kl":
+        teacher = teacher_hidden_states.reshape(-1, teacher_hidden_states.shape[-1])[idx]
+        grad_rows = dense_frozen_kl_grad(rows, draft_weight, teacher, teacher_weight, per_token,
+                                         logit_softcap=logit_softcap, dtype=dtype)
+        grad_weight = None
+    else:
+        raise ValueError(f"unsupported DFlash loss {loss_kind!r}")
+    grad_hidden[idx] = grad_rows.to(dtype)
+    return grad_hidden.reshape(hidden_states.shape), grad_weight

@@ -29,3 +29,15 @@ def gpu_device():
 
     native.verify_device(0)  # raises if the HIP library is missing or the arch is wrong
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def set_panel_budget():
+    """Returns a function that bounds the backward's staging panel (bytes) for the
+    rest of the test, through the package's context-local option."""
+    import contextlib
+
+    from turbo_dllm_amd import options
+
+    with contextlib.ExitStack() as stack:
+        yield lambda nbytes: stack.enter_context(options.panel_budget(int(nbytes)))

@@ -58,12 +58,11 @@ GPU_CASES = [
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("case", GPU_CASES, ids=[c[0] for c in GPU_CASES])
-def test_device_path_matches_oracle(gpu_device, case, monkeypatch):
+def test_device_path_matches_oracle(gpu_device, case, set_panel_budget):
     name, dtype, n, hd, ht, v, softcap, std, loss_tol, grad_tol = case
     print("[case]", name, flush=True)
-    from turbo_dllm_amd import chunked_linear_ce_native as native
     if "two_panels" in name:
-        monkeypatch.setattr(native, "PANEL_BYTES", 768 * 512 * 2)   # 512 columns per panel
+        set_panel_budget(768 * 512 * 2)   # 512 columns per panel
     gen = torch.Generator().manual_seed({"ref_bf16_seed31": 31, "ref_bf16_softcap_seed37": 37}
                                         .get(name, len(name)))
     dh = torch.randn(n, hd, generator=gen).to(dtype)

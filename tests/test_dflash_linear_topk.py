@@ -60,12 +60,11 @@ GPU_CASES = [
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("case", GPU_CASES, ids=[c[0] for c in GPU_CASES])
-def test_device_path_matches_oracle(gpu_device, case, monkeypatch):
+def test_device_path_matches_oracle(gpu_device, case, set_panel_budget):
     name, dtype, n, h, v, k, softcap, mult, std, panel_bytes = case
     print("[case]", name, flush=True)
-    from turbo_dllm_amd import chunked_linear_ce_native as native
     if panel_bytes:
-        monkeypatch.setattr(native, "PANEL_BYTES", panel_bytes)
+        set_panel_budget(panel_bytes)
     gen = torch.Generator().manual_seed(len(name) + k)
     hidden = torch.randn(n, h, generator=gen).to(dtype)
     weight = (torch.randn(v, h, generator=gen) * std).to(dtype)

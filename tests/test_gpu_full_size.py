@@ -3,7 +3,9 @@ a dense oracle over every row and column.
 
   * every per-row loss against the float32 oracle computed in row chunks;
   * grad_hidden on sampled rows and grad_weight on sampled vocabulary rows
-    against the oracle formula (each depends on one row / one column only);
+    against the oracle formula (each depends on one row / one column only), with
+    the oracle's lse over every loss-bearing row - also at the shape the
+    benchmark times (32768 loss-bearing rows);
   * <grad_weight, weight> == <grad_hidden, hidden>: both equal sum(G * logits);
   * columns of grad_weight sum to zero (softmax minus onehot sums to zero per row);
   * doubling grad_output doubles every gradient bit for bit (scaling by a power
@@ -52,70 +54,29 @@ def oracle_lse_in_chunks(wl, rows, chunk=512):
 
 
 def test_qwen3_8b_head_full_size(gpu_device):
-    wl = workloads.qwen3_8b_head(seed=5)
-    n, m = wl.n_rows, wl.n_loss_rows
-    say("qwen3_8b_head N", n, "M", m)
-    losses, dh, dw = run(gpu_device, wl)
-    keep = wl.labels != -100
-    rows = torch.nonzero(keep).flatten()
-
-    # every loss-bearing row against the oracle; ignored rows exactly zero
-    ref_loss, ref_lse = oracle_lse_in_chunks(wl, rows)
-    torch.testing.assert_close(losses[rows], ref_loss, rtol=1e-3, atol=1e-4)
-    assert torch.count_nonzero(losses[~keep]) == 0
-    assert torch.count_nonzero(dh[~keep]) == 0
-
-    # grad_hidden on sampled rows (depends on that row only)
-    gen = torch.Generator().manual_seed(1)
-    pick = rows[torch.randperm(m, generator=gen)[:32]]
-    rdh, _, _ = oracle.dense_linear_ce_grads(
-        wl.hidden[pick], wl.weight, wl.labels[pick], torch.full((32,), 1.0 / m),
-        reduction="none", logit_softcap=wl.logit_softcap, dtype=torch.float32)
-    err = oracle.relative_max_error(dh[pick], rdh)
-    say("grad_hidden sampled rows rel max err", f"{err:.2e}")
-    assert err <= 2e-2
-
-    # grad_weight on sampled vocabulary rows: dW[v] = sum_r g[r, v] * h_r
-    vs = torch.cat([torch.randint(0, wl.weight.shape[0], (24,), generator=gen),
-                    wl.labels[rows[:8]]])                       # include rows that are labels
-    h32 = wl.hidden[rows].float()
-    z = h32 @ wl.weight[vs].float().t()
-    g = torch.exp(z - ref_lse[:, None])
-    g -= (wl.labels[rows][:, None] == vs[None, :]).float()
-    g /= m
-    rdw = g.t() @ h32
-    err = oracle.relative_max_error(dw[vs], rdw)
-    say("grad_weight sampled rows rel max err", f"{err:.2e}")
-    assert err <= 2e-2
-
-    # <dW, W> == <dH, H>
-    lhs = float((dw.double() * wl.weight.double()).sum())
-    rhs = float((dh.double() * wl.hidden.double()).sum())
-    say("inner products", lhs, rhs)
-    assert abs(lhs - rhs) <= 2e-2 * max(abs(lhs), abs(rhs))
-
-    # columns of grad_weight sum to zero
-    col = dw.double().sum(dim=0).abs()
-    scale = dw.double().abs().sum(dim=0)
-    assert float((col / scale).max()) <= 2e-2
+    check_configuration_full_size(gpu_device, workloads.qwen3_8b_head(seed=5))
 
 
-def test_headline_shape_properties(gpu_device):
+def test_headline_shape_against_oracle(gpu_device):
+    """The shape the benchmark times (32768 loss-bearing rows, ten vocabulary
+    panels, float32 grad_hidden accumulation over ten passes): every loss, sampled
+    grad_hidden rows and sampled grad_weight rows against the float32 oracle with
+    the oracle's own lse, then the size-independent properties."""
     wl = workloads.block_diffusion_shard(seed=0, all_rows_loss_bearing=True)
-    say("block_diffusion_shard_all_rows N", wl.n_rows)
-    losses, dh, dw = run(gpu_device, wl)
+    n = wl.n_rows
+    v = wl.weight.shape[0]
+    plan_columns = 16384           # width of a vocabulary panel at this shape
     gen = torch.Generator().manual_seed(2)
-    pick = torch.randperm(wl.n_rows, generator=gen)[:64]
-    ref_loss, _ = oracle_lse_in_chunks(wl, pick)
-    torch.testing.assert_close(losses[pick], ref_loss, rtol=1e-3, atol=1e-4)
-    assert bool(torch.isfinite(losses).all())
-    lhs = float((dw.double() * wl.weight.double()).sum())
-    rhs = float((dh.double() * wl.hidden.double()).sum())
-    say("inner products", lhs, rhs)
-    assert abs(lhs - rhs) <= 2e-2 * max(abs(lhs), abs(rhs))
-    col = dw.double().sum(dim=0).abs()
-    scale = dw.double().abs().sum(dim=0)
-    assert float((col / scale).max()) <= 2e-2
+    # token rows at the 256-row tile edges and random ones; vocabulary rows at both ends,
+    # on either side of the first and the last panel boundary, random ones and labels
+    token_rows = torch.cat([torch.tensor([0, 255, 256, 16383, 16384, n - 257, n - 256, n - 1]),
+                            torch.randperm(n, generator=gen)[:40]])
+    last_panel = (v // plan_columns) * plan_columns
+    vocab_rows = torch.cat([torch.tensor([0, 1, plan_columns - 1, plan_columns, plan_columns + 1,
+                                          last_panel - 1, last_panel, v - 256, v - 1]),
+                            torch.randint(0, v, (31,), generator=gen)])
+    losses, dh, dw = check_configuration_full_size(gpu_device, wl, token_rows=token_rows,
+                                                   vocab_rows=vocab_rows)
     # linearity in grad_output, bit for bit
     _, dh2, dw2 = run(gpu_device, wl, grad_scale=2.0)
     assert torch.equal(dh2.float(), dh.float() * 2.0)
@@ -138,13 +99,17 @@ def test_block_diffusion_labels_compaction_full_size(gpu_device):
 
 
 # ------------------------------------------------- remaining configurations ----
-def check_configuration_full_size(dev, wl, *, loss_rows=768, check_column_sums=True):
-    """One benchmark configuration at full size against the oracle by sampling:
-    per-row losses and grad_hidden rows depend on their own row only, so sampled
-    rows are checked completely; grad_weight rows need every loss-bearing row but
-    only their own vocabulary column, with lse_r = loss_r + target_r taken from
-    the device's losses (themselves checked on the sample) and the oracle's
-    target logits."""
+def check_configuration_full_size(dev, wl, *, check_column_sums=True, token_rows=None,
+                                  vocab_rows=None):
+    """One benchmark configuration at full size against the float32 oracle.
+
+    The oracle's per-row loss and lse are computed for every loss-bearing row (in
+    row chunks), so every loss is compared.  A grad_hidden row depends on its own
+    row only: sampled rows are checked completely.  A grad_weight row needs every
+    loss-bearing row but only its own vocabulary column: sampled vocabulary rows
+    (both ends, label rows, random ones) are formed from the oracle's lse over
+    all rows.  Nothing on the reference side of a comparison comes from the
+    device."""
     n, m = wl.n_rows, wl.n_loss_rows
     h, v = wl.hidden.shape[1], wl.weight.shape[0]
     cap = wl.logit_softcap
@@ -158,38 +123,35 @@ def check_configuration_full_size(dev, wl, *, loss_rows=768, check_column_sums=T
     assert bool(torch.isfinite(losses).all()) and bool(torch.isfinite(dh.float()).all())
     assert bool(torch.isfinite(dw.float()).all())
 
-    gen = torch.Generator().manual_seed(1)
-    sample = rows[torch.randperm(m, generator=gen)[:min(loss_rows, m)]]
-    ref_loss, _ = oracle_lse_in_chunks(wl, sample)
-    torch.testing.assert_close(losses[sample], ref_loss, rtol=1e-3, atol=1e-4)
-    say("losses on", sample.numel(), "sampled rows ok")
+    ref_loss, ref_lse = oracle_lse_in_chunks(wl, rows)
+    torch.testing.assert_close(losses[rows], ref_loss, rtol=1e-3, atol=1e-4)
+    say("losses on all", rows.numel(), "loss-bearing rows ok")
 
-    pick = sample[:32]
+    gen = torch.Generator().manual_seed(1)
+    if token_rows is None:
+        token_rows = rows[torch.randperm(m, generator=gen)[:32]]
     rdh, _, _ = oracle.dense_linear_ce_grads(
-        wl.hidden[pick], wl.weight, wl.labels[pick], torch.full((pick.numel(),), 1.0 / m),
+        wl.hidden[token_rows], wl.weight, wl.labels[token_rows],
+        torch.full((token_rows.numel(),), 1.0 / m),
         reduction="none", logit_softcap=cap, dtype=torch.float32)
-    err = oracle.relative_max_error(dh[pick], rdh)
-    say("grad_hidden sampled rows rel max err", f"{err:.2e}")
+    err = oracle.relative_max_error(dh[token_rows], rdh)
+    say("grad_hidden on", token_rows.numel(), "sampled rows rel max err", f"{err:.2e}")
     assert err <= 2e-2
 
-    # grad_weight on sampled vocabulary rows (some of them label rows, the first and the last)
-    vs = torch.cat([torch.randint(0, v, (22,), generator=gen), wl.labels[rows[:8]],
-                    torch.tensor([0, v - 1])])
+    if vocab_rows is None:
+        vocab_rows = torch.cat([torch.randint(0, v, (22,), generator=gen), torch.tensor([0, v - 1])])
+    vs = torch.cat([vocab_rows, wl.labels[rows[:8]]])     # some of them label rows
     h32 = wl.hidden[rows].float()
     y = wl.labels[rows]
-    target = (h32 * wl.weight[y].float()).sum(dim=1)
-    if cap:
-        target = torch.tanh(target / cap) * cap
-    lse = losses[rows] + target
     z = h32 @ wl.weight[vs].float().t()
     dcap = 1.0
     if cap:
         t = torch.tanh(z / cap)
         z, dcap = t * cap, 1.0 - t * t
-    g = (torch.exp(z - lse[:, None]) - (y[:, None] == vs[None, :]).float()) * dcap / m
+    g = (torch.exp(z - ref_lse[:, None]) - (y[:, None] == vs[None, :]).float()) * dcap / m
     rdw = g.t() @ h32
     err = oracle.relative_max_error(dw[vs], rdw)
-    say("grad_weight sampled rows rel max err", f"{err:.2e}")
+    say("grad_weight on", vs.numel(), "sampled vocabulary rows rel max err", f"{err:.2e}")
     assert err <= 2e-2
 
     lhs = float((dw.double() * wl.weight.double()).sum())
@@ -200,6 +162,7 @@ def check_configuration_full_size(dev, wl, *, loss_rows=768, check_column_sums=T
         col = dw.double().sum(dim=0).abs()
         scale = dw.double().abs().sum(dim=0)
         assert float((col / scale).max()) <= 2e-2
+    return losses, dh, dw
 
 
 def test_block_diffusion_shard_full_size(gpu_device):
@@ -209,7 +172,7 @@ def test_block_diffusion_shard_full_size(gpu_device):
 def test_gemma_softcap_head_full_size(gpu_device):
     # H=3840, V=262144 (1024 vocabulary tiles, four panels), soft cap 30
     check_configuration_full_size(gpu_device, workloads.gemma_softcap_head(seed=7),
-                                  loss_rows=512, check_column_sums=False)
+                                  check_column_sums=False)
 
 
 def test_sparse_drafter_head_full_size(gpu_device):
@@ -219,7 +182,7 @@ def test_sparse_drafter_head_full_size(gpu_device):
     plan = _lib.query_plan(wl.n_loss_rows, 4096, 151936, _lib.DTYPE_BF16, True)
     say("plan", plan)
     assert plan["grad_hidden_k_splits"] > 1
-    check_configuration_full_size(gpu_device, wl, loss_rows=4096)
+    check_configuration_full_size(gpu_device, wl)
 
 
 def test_block_diffusion_shard_full_size_without_host_read_back(gpu_device):

@@ -78,7 +78,8 @@ def check_against_oracle(dev, hidden, weight, labels, *, bias=None, reduction="m
 @pytest.mark.parametrize("n,density", [(0, 0.5), (1, 1.0), (1, 0.0), (63, 0.5), (64, 0.5),
                                        (65, 0.5), (1023, 0.3), (1024, 0.3), (1025, 0.3),
                                        (32768, 0.5), (35011, 0.05), (100003, 0.0),
-                                       (100003, 1.0), (1 << 20, 0.7)])
+                                       (100003, 1.0), (262144, 0.5), (262145, 0.5),
+                                       (1 << 20, 0.7), ((1 << 24) + 5, 0.31)])
 def test_compaction_indices_are_bit_exact(gpu_device, n, density):
     say("compaction", n, density)
     rng = np.random.default_rng(n * 7 + int(density * 100))
@@ -93,6 +94,54 @@ def test_compaction_indices_are_bit_exact(gpu_device, n, density):
     labels2[labels2 == -100] = -1
     idx2, m2 = native.compact_rows(torch.from_numpy(labels2).to(gpu_device), -100)
     assert m2 == n and np.array_equal(idx2.cpu().numpy(), np.arange(n))
+
+
+@pytest.mark.parametrize("n,density", [(0, 0.5), (1, 1.0), (1, 0.0), (65, 0.5), (1025, 0.3),
+                                       (32768, 0.25), (262145, 0.9), (1 << 20, 0.05),
+                                       ((1 << 24) + 77, 0.5)])
+@pytest.mark.parametrize("kind", ["bool", "uint8", "float"])
+def test_mask_compaction_equals_torch_nonzero(gpu_device, n, density, kind):
+    """The boolean-mask form of the scan (the DFlash call sites compact
+    `supervised_mask`, dflash/model.py:870-871): bit-exact against torch.nonzero
+    on the host, up to sizes that take the block-offset scan."""
+    if kind != "bool" and n > (1 << 20):
+        pytest.skip("the large size is covered once")
+    say("mask compaction", n, density, kind)
+    gen = torch.Generator().manual_seed(n * 3 + int(density * 100))
+    keep = torch.rand(n, generator=gen) < density
+    mask = {"bool": keep, "uint8": keep.to(torch.uint8) * 7, "float": keep.float() * -2.5}[kind]
+    expect = torch.nonzero(keep, as_tuple=False).flatten()
+    idx, m = native.compact_mask(mask.to(gpu_device))
+    assert m == expect.numel() and idx.dtype == torch.int64
+    assert torch.equal(idx.cpu(), expect)
+    # a 2-D mask is scanned in its flattened order
+    if n and n % 4 == 0:
+        idx2, m2 = native.compact_mask(mask.reshape(4, -1).to(gpu_device))
+        assert m2 == m and torch.equal(idx2.cpu(), expect)
+
+
+def test_fused_gather_clamps_the_device_row_count(gpu_device):
+    """A row count beyond the capacity (a stale or corrupt counter) must not walk
+    past the index buffer: the gather treats it as the capacity."""
+    dev = gpu_device
+    torch.manual_seed(4)
+    n, h = 200, 64
+    hidden = torch.randn(n, h).bfloat16()
+    labels = torch.randint(0, 50, (n,))
+    labels[torch.rand(n) < 0.5] = -100
+    idx, count = native.compact_rows_device(labels.to(dev), -100)
+    m = int(count.item())
+    keep = torch.nonzero(labels != -100).flatten()
+    big = torch.tensor([10 * n], dtype=torch.long, device=dev)
+    rows, targets, _ = native.gather_loss_rows(hidden.to(dev), labels.to(dev), None, idx, big,
+                                               -100, capacity=m)
+    assert rows.shape[0] == (m + 63) // 64 * 64
+    assert torch.equal(rows[:m].cpu(), hidden[keep]) and torch.equal(targets[:m].cpu(), labels[keep])
+    assert torch.count_nonzero(rows[m:].float()) == 0 and bool((targets[m:] == -100).all())
+    negative = torch.tensor([-3], dtype=torch.long, device=dev)
+    rows, targets, _ = native.gather_loss_rows(hidden.to(dev), labels.to(dev), None, idx, negative,
+                                               -100, capacity=m)
+    torch.cuda.synchronize()       # nothing gathered, nothing faulted
 
 
 @pytest.mark.parametrize("row_shape,dtype", [((4096,), torch.bfloat16), ((96,), torch.bfloat16),
@@ -341,13 +390,9 @@ def test_panel_count_does_not_change_results(gpu_device):
     weight = (torch.randn(3000, 256) * 0.1).bfloat16()
     labels = torch.randint(0, 3000, (600,))
     base = run_api(gpu_device, hidden, weight, labels, reduction="mean", dtype=torch.bfloat16)
-    old = native.PANEL_BYTES
-    try:
-        native.PANEL_BYTES = 768 * 256 * 2 * 2 * 3   # three 256-column tiles per panel
+    with native.panel_budget(768 * 256 * 2 * 2 * 3):   # three 256-column tiles per panel
         multi = run_api(gpu_device, hidden, weight, labels, reduction="mean",
                         dtype=torch.bfloat16)
-    finally:
-        native.PANEL_BYTES = old
     assert torch.equal(base[0], multi[0])
     assert torch.equal(base[2], multi[2])                      # grad_weight: same tiles, same order
     assert oracle.relative_max_error(multi[1], base[1].double()) < 1e-2   # grad_hidden: split differs
@@ -367,16 +412,11 @@ def test_direct_engine_in_place_operands(gpu_device, m, h, v, panel_tiles):
     weight = (torch.randn(v, h) * 0.2).bfloat16()
     labels = torch.randint(0, v, (m + 7,))
     labels[torch.randperm(m + 7)[:7]] = -100
-    old = native.PANEL_BYTES
-    try:
-        if panel_tiles:
-            mp = -(-m // 256) * 256
-            native.PANEL_BYTES = mp * 256 * 2 * panel_tiles
+    mp = -(-m // 256) * 256
+    with native.panel_budget(mp * 256 * 2 * panel_tiles):   # 0: the library default
         check_against_oracle(gpu_device, hidden, weight, labels, reduction="mean")
         check_against_oracle(gpu_device, hidden, weight, labels, reduction="sum", frozen=True,
                              logit_softcap=4.0)
-    finally:
-        native.PANEL_BYTES = old
 
 
 # ------------------------------------------- benchmark configurations, scaled ----

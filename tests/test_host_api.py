@@ -273,7 +273,7 @@ def test_native_token_cross_entropy_on_host_and_compaction_modes():
     losses.sum().backward()
     assert hidden.grad is not None and head.weight.grad is not None
 
-    # the compaction mode is a process-wide setting with a scoped form
+    # the compaction mode is a context-local setting with a scoped form
     assert COMPACTION_MODES == ("sync", "device", "none") and get_compaction_mode() == "sync"
     with compaction_mode("device"):
         assert get_compaction_mode() == "device"
@@ -284,3 +284,69 @@ def test_native_token_cross_entropy_on_host_and_compaction_modes():
     with pytest.raises(ValueError):
         set_compaction_mode("lazy")
     assert get_compaction_mode() == "sync"
+
+
+def test_options_are_local_to_the_calling_thread():
+    """Two trainers in one process can choose different compaction modes and
+    panel budgets: a setting made in one thread is invisible in another."""
+    import threading
+
+    from turbo_dllm_amd import options
+
+    seen = {}
+    ready, release = threading.Event(), threading.Event()
+
+    def other():
+        seen["start"] = (options.get_compaction_mode(), options.get_panel_bytes())
+        with options.compaction_mode("none"), options.panel_budget(1 << 20):
+            ready.set()
+            release.wait(10)
+            seen["inside"] = (options.get_compaction_mode(), options.get_panel_bytes())
+
+    with options.compaction_mode("device"), options.panel_budget(1 << 28):
+        thread = threading.Thread(target=other)
+        thread.start()
+        assert ready.wait(10)
+        # the other thread's choices did not leak into this one
+        assert options.get_compaction_mode() == "device" and options.get_panel_bytes() == 1 << 28
+        release.set()
+        thread.join(10)
+    assert seen["start"] == ("sync", 0)            # a new thread starts from the defaults
+    assert seen["inside"] == ("none", 1 << 20)
+    assert options.get_compaction_mode() == "sync" and options.get_panel_bytes() == 0
+    assert options.resolve_compaction(None) == "sync"
+    assert options.resolve_compaction("device") == "device"
+    with pytest.raises(ValueError):
+        options.resolve_compaction("lazy")
+    with pytest.raises(ValueError):
+        with options.panel_budget(-1):
+            pass
+    old = options.set_panel_bytes(4096)
+    assert old == 0 and options.get_panel_bytes() == 4096
+    options.set_panel_bytes(old)
+
+
+def test_verify_dflash_symbols():
+    """Start-up check of the DFlash executor (reference shim,
+    chunked_linear_ce_native.py:353-363): unknown kinds raise ValueError, known
+    ones resolve the library and the entry points that loss needs."""
+    from turbo_dllm_amd import _lib
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+
+    for kind in ("paper_ce", "speculators_kl", "dflash", "dpace",
+                 "dpace-cumulative-confidence-only", "dpace-continuation-value-only"):
+        native.verify_dflash_symbols(loss_kind=kind)
+    with pytest.raises(ValueError, match="unsupported DFlash loss 'kl'"):
+        native.verify_dflash_symbols(loss_kind="kl")
+    with pytest.raises(TypeError):
+        native.verify_dflash_symbols("paper_ce")        # keyword-only, as in the reference
+    # a library without the entry points fails the check, not the first training step
+    class Stub:
+        pass
+    real = _lib.library
+    try:
+        _lib.library = lambda: Stub()
+        with pytest.raises(_lib.NativeLibraryMissing, match="tlce_kl_workspace_bytes"):
+            native.verify_dflash_symbols(loss_kind="speculators_kl")
+    finally:
+        _lib.library = real

@@ -450,3 +450,98 @@ def test_masked_token_loss_oracle_matches_library_expression(multiplier, softcap
     torch.testing.assert_close(dw, weight.grad, atol=1e-12, rtol=1e-10)
     torch.testing.assert_close(db, bias.grad, atol=1e-12, rtol=1e-10)
     assert torch.count_nonzero(dh[[1, 7]]) == 0
+
+
+# ----------------------------------------------------------- DFlash loss method ----
+def _dflash_case(seed, batch=3, tokens=7, h=6, ht=5, v=11, density=0.5):
+    gen = torch.Generator().manual_seed(seed)
+    hidden = torch.randn(batch, tokens, h, generator=gen, dtype=torch.float64)
+    teacher = torch.randn(batch, tokens, ht, generator=gen, dtype=torch.float64)
+    draft_w = torch.randn(v, h, generator=gen, dtype=torch.float64) * 0.7
+    teacher_w = torch.randn(v, ht, generator=gen, dtype=torch.float64) * 0.7
+    targets = torch.randint(0, v, (batch, tokens), generator=gen)
+    mask = torch.rand(batch, tokens, generator=gen) < density
+    weights = torch.rand(batch, tokens, generator=gen, dtype=torch.float64) + 0.25
+    counts = mask.sum(dim=1).to(torch.float64) + 1.0
+    return hidden, teacher, draft_w, teacher_w, targets, mask, weights, counts
+
+
+@pytest.mark.parametrize("loss_kind", ["paper_ce", "speculators_kl"])
+@pytest.mark.parametrize("softcap", [None, 3.0])
+def test_dflash_loss_oracle_matches_the_reference_call_sequence(loss_kind, softcap):
+    """The sequence of library calls distributed_dflash_loss makes
+    (dflash/model.py:870-955): nonzero, index_select, F.cross_entropy / F.kl_div
+    on dense logits, scatter_add_, / (count + 1e-5), mean, * scale; gradients by
+    autograd through it."""
+    hidden, teacher, draft_w, teacher_w, targets, mask, weights, counts = _dflash_case(41)
+    hidden = hidden.requires_grad_(True)
+    draft_w = draft_w.requires_grad_(True)
+    idx = torch.nonzero(mask.reshape(-1), as_tuple=False).flatten()
+    rows = hidden.reshape(-1, hidden.shape[-1]).index_select(0, idx)
+    pw = weights.reshape(-1).index_select(0, idx)
+
+    def capped(z):
+        return z if softcap is None else softcap * torch.tanh(z / softcap)
+    draft_logits = capped(F.linear(rows, draft_w))
+    if loss_kind == "paper_ce":
+        token_loss = F.cross_entropy(draft_logits, targets.reshape(-1).index_select(0, idx),
+                                     reduction="none")
+    else:
+        trows = teacher.reshape(-1, teacher.shape[-1]).index_select(0, idx)
+        teacher_logits = capped(F.linear(trows, teacher_w))
+        token_loss = F.kl_div(F.log_softmax(draft_logits, dim=-1),
+                              F.softmax(teacher_logits, dim=-1), reduction="none").sum(dim=-1)
+    numerators = torch.zeros(mask.shape[0], dtype=torch.float64)
+    numerators.scatter_add_(0, torch.div(idx, mask.shape[1], rounding_mode="floor"),
+                            token_loss * pw)
+    expect = (numerators / (counts + 1.0e-5)).mean() * 1.75
+    expect.backward()
+
+    kw = dict(loss_kind=loss_kind, teacher_hidden_states=teacher, teacher_weight=teacher_w,
+              logit_softcap=softcap, loss_scale=1.75)
+    got = oracle.dflash_token_loss(hidden.detach(), targets, mask, weights, draft_w.detach(),
+                                   counts, **kw)
+    torch.testing.assert_close(got, expect.detach(), rtol=1e-12, atol=1e-12)
+    dh, dw = oracle.dflash_token_loss_grads(hidden.detach(), targets, mask, weights,
+                                            draft_w.detach(), counts, **kw)
+    torch.testing.assert_close(dh, hidden.grad, rtol=1e-10, atol=1e-12)
+    assert torch.count_nonzero(dh.reshape(-1, dh.shape[-1])[~mask.reshape(-1)]) == 0
+    if loss_kind == "paper_ce":
+        torch.testing.assert_close(dw, draft_w.grad, rtol=1e-10, atol=1e-12)
+    else:
+        assert dw is None
+
+
+def test_dflash_loss_oracle_per_sample_loop_and_empty_batch():
+    hidden, teacher, draft_w, teacher_w, targets, mask, weights, counts = _dflash_case(43)
+    mask[1] = False                       # a sample without supervised positions
+    batch, tokens = mask.shape
+    total = 0.0
+    for b in range(batch):                # brute force, one sample and one position at a time
+        num = 0.0
+        for t in range(tokens):
+            if not bool(mask[b, t]):
+                continue
+            z = [float(hidden[b, t] @ draft_w[v]) for v in range(draft_w.shape[0])]
+            lse = math.log(sum(math.exp(x) for x in z))
+            num += (lse - z[int(targets[b, t])]) * float(weights[b, t])
+        total += num / (float(counts[b]) + 1.0e-5)
+    got = oracle.dflash_token_loss(hidden, targets, mask, weights, draft_w, counts,
+                                   loss_kind="paper_ce")
+    assert abs(float(got) - total / batch) <= 1e-12 * abs(total)
+    # the scatter-add on its own
+    idx = torch.nonzero(mask.reshape(-1)).flatten()
+    vals = torch.arange(1, idx.numel() + 1, dtype=torch.float64)
+    w = weights.reshape(-1)[idx]
+    expect = torch.zeros(batch, dtype=torch.float64).scatter_add_(0, idx // tokens, vals * w)
+    torch.testing.assert_close(oracle.segment_weighted_sum(vals, w, idx, tokens, batch), expect)
+    assert float(oracle.segment_weighted_sum(vals, None, idx, tokens, batch)[1]) == 0.0
+    # nothing supervised: exactly zero, zero gradient
+    none = torch.zeros_like(mask)
+    assert float(oracle.dflash_token_loss(hidden, targets, none, weights, draft_w, counts,
+                                          loss_kind="paper_ce")) == 0.0
+    dh, dw = oracle.dflash_token_loss_grads(hidden, targets, none, weights, draft_w, counts,
+                                            loss_kind="paper_ce")
+    assert torch.count_nonzero(dh) == 0 and dw is None
+    with pytest.raises(ValueError):
+        oracle.dflash_token_loss(hidden, targets, mask, weights, draft_w, counts, loss_kind="kl")

@@ -15,13 +15,14 @@ __all__ = [
     "VocabParallelLinear",
     "chunked_linear_ce_native",
     "compact_valid_loss_rows",
+    "dflash_token_loss",
     "frozen_linear_ce_topk",
     "frozen_linear_kl",
     "masked_token_loss",
     "tiled_linear_cross_entropy",
 ]
 
-_SUBMODULES = {"chunked_linear_ce_native", "compaction", "layers", "loss", "build",
+_SUBMODULES = {"chunked_linear_ce_native", "compaction", "layers", "loss", "build", "options",
                "dflash_kl", "dflash_linear_topk", "streaming_soft_embedding"}
 
 
@@ -39,6 +40,12 @@ def compact_valid_loss_rows(*args: Any, **kwargs: Any) -> Any:
 
 def masked_token_loss(*args: Any, **kwargs: Any) -> Any:
     from .loss import masked_token_loss as impl
+
+    return impl(*args, **kwargs)
+
+
+def dflash_token_loss(*args: Any, **kwargs: Any) -> Any:
+    from .loss import dflash_token_loss as impl
 
     return impl(*args, **kwargs)
 

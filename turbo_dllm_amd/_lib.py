@@ -30,6 +30,10 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p],
     ),
+    "tlce_compact_mask": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p],
+    ),
     "tlce_gather_rows": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "tlce_scatter_rows": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "tlce_fill_zero": (c_int, [c_void_p, c_int64, c_void_p]),
@@ -182,6 +186,10 @@ SIGNATURES = {
             c_float, c_float, c_void_p,                         # multiplier softcap grad_hidden
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
+    ),
+    "tlce_segment_weighted_sum": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p],
     ),
     "tlce_profile_begin": (c_int, []),
     "tlce_profile_end": (c_int, [c_void_p, c_void_p, c_int]),

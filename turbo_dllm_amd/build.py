@@ -78,8 +78,17 @@ def _run(command: list[str], verbose: bool) -> None:
         print(stderr, file=sys.stderr)
 
 
-def build_library(verbose: bool = False, jobs: int | None = None) -> Path:
-    """Compiles every HIP source for gfx950 and links the shared library."""
+def _newest_source_time() -> float:
+    sources = [*CSRC_DIR.glob("*.h"), *CSRC_DIR.glob("*.hip"),
+               PACKAGE_DIR.parent / "include" / "tlce.h", Path(__file__)]
+    return max(path.stat().st_mtime for path in sources)
+
+
+def build_library(verbose: bool = False, jobs: int | None = None,
+                  incremental: bool = False) -> Path:
+    """Compiles every HIP source for gfx950 and links the shared library.
+    ``incremental`` skips objects newer than every source and header (for the
+    edit-compile loop; the default recompiles everything)."""
     hipcc = find_hipcc()
     OBJECT_DIR.mkdir(exist_ok=True)
     objects = [OBJECT_DIR / (name + ".o") for name, _, _ in UNITS]
@@ -87,6 +96,10 @@ def build_library(verbose: bool = False, jobs: int | None = None) -> Path:
         [hipcc, *HIPCC_FLAGS, *defines, "-c", str(CSRC_DIR / source), "-o", str(obj)]
         for (_, source, defines), obj in zip(UNITS, objects)
     ]
+    if incremental:
+        newest = _newest_source_time()
+        commands = [command for command, obj in zip(commands, objects)
+                    if not obj.exists() or obj.stat().st_mtime < newest]
     if jobs is None:
         jobs = min(len(commands), os.cpu_count() or 1, 16)
     with ThreadPoolExecutor(max_workers=max(int(jobs), 1)) as pool:
@@ -97,4 +110,4 @@ def build_library(verbose: bool = False, jobs: int | None = None) -> Path:
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_library(verbose=True, incremental="--incremental" in sys.argv[1:]))

@@ -28,9 +28,7 @@ _DTYPE_CODES = {
     torch.bfloat16: _lib.DTYPE_BF16,
 }
 
-# Upper bound, in bytes, of the logit-gradient staging panel of the backward
-# pass (0 selects the library default of 1 GiB).
-PANEL_BYTES = 0
+from .options import get_panel_bytes, panel_budget  # noqa: F401  (panel_budget re-exported)
 
 
 def _reduction_code(reduction: str) -> int:
@@ -99,6 +97,37 @@ def verify_device(device: torch.device | int | None = None) -> None:
     _lib.check(_lib.library().tlce_check_device(int(index or 0)), "tlce_check_device")
 
 
+_DFLASH_LOSS_KINDS = frozenset({
+    "paper_ce", "speculators_kl", "dflash", "dpace",
+    "dpace-cumulative-confidence-only", "dpace-continuation-value-only",
+})
+# entry points each family of DFlash losses calls in the library
+_DFLASH_SYMBOLS = {
+    "paper_ce": ("tlce_forward", "tlce_backward", "tlce_compact_mask"),
+    "speculators_kl": ("tlce_kl_workspace_bytes", "tlce_kl_forward", "tlce_kl_backward",
+                       "tlce_compact_mask"),
+    "ce_topk": ("tlce_ce_topk_forward_workspace_bytes", "tlce_ce_topk_backward_workspace_bytes",
+                "tlce_ce_topk_forward", "tlce_ce_topk_backward", "tlce_compact_mask"),
+}
+
+
+def verify_dflash_symbols(*, loss_kind: str) -> None:
+    """Start-up check of the DFlash executor: raises ``ValueError`` for an unknown
+    loss kind and a loader error when the library is absent or lacks an entry
+    point that loss needs, so that a missing build fails before the first step
+    and not inside it (reference shim, chunked_linear_ce_native.py:353-363,
+    which resolves its DFlash extension the same way)."""
+    if loss_kind not in _DFLASH_LOSS_KINDS:
+        raise ValueError(f"unsupported DFlash loss {loss_kind!r}")
+    family = loss_kind if loss_kind in ("paper_ce", "speculators_kl") else "ce_topk"
+    lib = _lib.library()          # raises NativeLibraryMissing when it has not been built
+    for name in _DFLASH_SYMBOLS[family]:
+        if not hasattr(lib, name):
+            raise _lib.NativeLibraryMissing(
+                f"{_lib.LIBRARY_PATH} does not export {name!r}, which DFlash loss "
+                f"{loss_kind!r} needs; rebuild the library")
+
+
 # ----------------------------------------------------------------- compaction --
 def compact_rows(labels: torch.Tensor, ignore_index: int) -> tuple[torch.Tensor, int]:
     """``nonzero(labels != ignore_index).flatten()`` on the device.
@@ -150,6 +179,47 @@ def compact_rows_device(labels: torch.Tensor, ignore_index: int) -> tuple[torch.
     return row_idx[:n], count
 
 
+def _mask_bytes(mask: torch.Tensor) -> torch.Tensor:
+    mask = mask.reshape(-1)
+    if mask.dtype == torch.bool:
+        return mask.contiguous().view(torch.uint8)
+    if mask.dtype == torch.uint8:
+        return mask.contiguous()
+    return (mask != 0).view(torch.uint8)
+
+
+def compact_mask_device(mask: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """``nonzero(mask).flatten()`` on the device without a host read-back: the
+    index buffer at full length (its first ``count`` entries are defined) and the
+    count as a device int64 tensor of one element.  ``mask`` is a bool / uint8
+    tensor (anything else is compared with 0 first)."""
+    device = _require_device(mask)
+    flags = _mask_bytes(mask)
+    n = flags.numel()
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        row_idx = torch.empty(max(n, 1), dtype=torch.long, device=device)
+        count = torch.empty(1, dtype=torch.long, device=device)
+        ws = _workspace(lib.tlce_compact_workspace_bytes(n), device)
+        _lib.check(
+            lib.tlce_compact_mask(
+                _ptr(flags), n, row_idx.data_ptr(), count.data_ptr(),
+                ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_compact_mask",
+        )
+    return row_idx[:n], count
+
+
+def compact_mask(mask: torch.Tensor) -> tuple[torch.Tensor, int]:
+    """``nonzero(mask).flatten()`` (ascending int64) and its length, read back
+    once: the host synchronisation ``valid_indices.numel()`` costs the
+    reference too (dflash/model.py:885)."""
+    row_idx, count = compact_mask_device(mask)
+    m = int(count.item())
+    return row_idx[:m], m
+
+
 def gather_loss_rows(
     hidden: torch.Tensor,
     labels: torch.Tensor,
@@ -157,37 +227,111 @@ def gather_loss_rows(
     row_idx: torch.Tensor,
     row_count: torch.Tensor,
     ignore_index: int,
+    capacity: int | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor | None]:
     """Hidden rows, labels and (optional) float32 loss weights of the first
     ``row_count`` positions in ``row_idx``, gathered in one launch with the
-    count read on the device.  The outputs have ``round_up(n, 64)`` rows; rows
-    from the count up to the next multiple of 64 are zero / ignored / weight 0."""
+    count read on the device.  ``capacity`` bounds the count (default: all ``n``
+    rows; a caller that has read the count back passes it).  The outputs have
+    ``round_up(capacity, 64)`` rows; rows from the count up to the next
+    multiple of 64 are zero / ignored / weight 0."""
     device = _require_device(hidden, labels, weights, row_idx, row_count)
     hidden = hidden.contiguous()
     labels = labels.reshape(-1).to(torch.long).contiguous()
     n, h = hidden.shape
-    if labels.numel() != n or row_idx.numel() != n:
+    capacity = n if capacity is None else int(capacity)
+    if labels.numel() != n or not 0 <= capacity <= n or row_idx.numel() < capacity:
         raise RuntimeError("gather_loss_rows: hidden, labels and row_idx lengths differ")
     if weights is not None:
         weights = weights.reshape(-1).to(torch.float32).contiguous()
         if weights.numel() != n:
             raise RuntimeError("gather_loss_rows: weights length differs")
-    padded = (n + 63) // 64 * 64
+    padded = (capacity + 63) // 64 * 64
     row_bytes = h * hidden.element_size()
     with torch.cuda.device(device):
         rows = torch.empty((padded, h), dtype=hidden.dtype, device=device)
         targets = torch.empty(padded, dtype=torch.long, device=device)
         w = None if weights is None else torch.empty(padded, dtype=torch.float32, device=device)
-        if n:
+        if capacity:
             _lib.check(
                 _lib.library().tlce_gather_loss_rows(
                     hidden.data_ptr(), labels.data_ptr(), _ptr(weights), row_idx.data_ptr(),
-                    row_count.data_ptr(), n, padded, row_bytes, int(ignore_index),
+                    row_count.data_ptr(), capacity, padded, row_bytes, int(ignore_index),
                     rows.data_ptr(), targets.data_ptr(), _ptr(w), _stream(device),
                 ),
                 "tlce_gather_loss_rows",
             )
     return rows, targets, w
+
+
+def compact_loss_rows(
+    hidden: torch.Tensor,
+    labels: torch.Tensor,
+    weights: torch.Tensor | None,
+    ignore_index: int,
+    mode: str,
+):
+    """The row compaction in front of the loss kernels, by compaction mode.
+
+    Returns ``(rows, targets, token_weights, row_idx, row_count, m)``: the
+    operands the ``masked_loss_*`` / ``forward`` entry points take.  "none":
+    the inputs as they are.  "sync": one scan, the count read back, then one
+    fused gather of exactly the loss-bearing rows (padded with zero rows to a
+    multiple of 64, which is what the count on the device, handed on as
+    ``row_count``, licenses the kernels to read).  "device": the same without
+    the read-back, every buffer sized for all rows."""
+    n = hidden.shape[0]
+    if mode == "none" or n == 0:
+        return hidden, labels, weights, None, None, n
+    row_idx, row_count = compact_rows_device(labels, ignore_index)
+    if mode == "device":
+        rows, targets, token_weights = gather_loss_rows(hidden, labels, weights, row_idx,
+                                                        row_count, ignore_index)
+        return rows, targets, token_weights, row_idx, row_count, n
+    m = int(row_count.item())
+    if m == n:
+        return hidden, labels, weights, None, None, n
+    if m == 0:
+        return (hidden[:0], labels[:0], None if weights is None else weights[:0],
+                row_idx[:0], None, 0)
+    rows, targets, token_weights = gather_loss_rows(hidden, labels, weights, row_idx, row_count,
+                                                    ignore_index, capacity=m)
+    return rows, targets, token_weights, row_idx[:m], row_count, m
+
+
+def segment_weighted_sum(
+    values: torch.Tensor,
+    weights: torch.Tensor | None,
+    row_idx: torch.Tensor,
+    segment_length: int,
+    n_segments: int,
+    row_count: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``out[s] = sum(values[r] * weights[r])`` over the compacted rows whose
+    position ``row_idx[r]`` lies in sample ``s`` (positions ``[s * L, (s + 1) * L)``),
+    float32 ``[n_segments]``, summed in a fixed order (no atomics): the
+    reference's ``numerators.scatter_add_`` (dflash/model.py:925-937) for
+    ascending ``row_idx``."""
+    device = _require_device(values, weights, row_idx, row_count)
+    values = values.reshape(-1).to(torch.float32).contiguous()
+    m = values.numel()
+    if weights is not None:
+        weights = weights.reshape(-1).to(torch.float32).contiguous()
+        if weights.numel() != m:
+            raise RuntimeError("segment_weighted_sum: values and weights lengths differ")
+    row_idx = row_idx.reshape(-1).to(torch.long).contiguous()
+    if row_idx.numel() < m:
+        raise RuntimeError("segment_weighted_sum: row_idx holds fewer entries than values")
+    with torch.cuda.device(device):
+        out = torch.empty(int(n_segments), dtype=torch.float32, device=device)
+        _lib.check(
+            _lib.library().tlce_segment_weighted_sum(
+                _ptr(values), _ptr(weights), _ptr(row_idx), _ptr(row_count), m,
+                int(segment_length), int(n_segments), _ptr(out), _stream(device),
+            ),
+            "tlce_segment_weighted_sum",
+        )
+    return out
 
 
 def gather_rows(src: torch.Tensor, row_idx: torch.Tensor) -> torch.Tensor:
@@ -335,7 +479,7 @@ def _backward(
         )
         ws = _workspace(
             lib.tlce_backward_workspace_bytes(
-                m, h, v, code, int(compute_weight_grad), int(bias is not None), PANEL_BYTES
+                m, h, v, code, int(compute_weight_grad), int(bias is not None), get_panel_bytes()
             ),
             device,
         )
@@ -346,7 +490,7 @@ def _backward(
                 m, n_out, h, v, code,
                 reduction_code, int(ignore_index), int(exclude_index), float(logit_softcap),
                 _ptr(grad_hidden), _ptr(grad_weight), _ptr(grad_bias32),
-                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_backward",
         )
@@ -531,6 +675,12 @@ def masked_loss_backward(
     h = hidden.shape[1]
     v = weight.shape[0]
     m = hidden.shape[0] if m is None else int(m)
+    # the C ABI cannot see tensor lengths: the same row checks as the forward
+    need_rows = (m + 63) // 64 * 64 if row_count is not None else m
+    if hidden.shape[0] < need_rows or labels.numel() < m or lse.numel() < m:
+        raise RuntimeError("masked loss: hidden / labels / lse hold fewer rows than m")
+    if weight.dim() != 2 or weight.shape[1] != h or weight.dtype != hidden.dtype:
+        raise RuntimeError("masked loss expects weight [V, D] in the dtype of hidden")
     n_out = m if n_out is None else int(n_out)
     code = _dtype_code(hidden)
     reduction_code = _reduction_code(reduction)
@@ -541,6 +691,9 @@ def masked_loss_backward(
     bias32 = None if bias is None else bias.to(torch.float32).contiguous()
     if token_weights is not None:
         token_weights = token_weights.reshape(-1).to(torch.float32).contiguous()
+        if token_weights.numel() < m:
+            raise RuntimeError("masked loss: token_weights holds fewer entries than m")
+    lse = lse.reshape(-1).to(torch.float32).contiguous()
     lib = _lib.library()
     with torch.cuda.device(device):
         grad_hidden = torch.empty((n_out, h), dtype=hidden.dtype, device=device)
@@ -552,7 +705,7 @@ def masked_loss_backward(
         )
         ws = _workspace(
             lib.tlce_backward_workspace_bytes(
-                m, h, v, code, int(compute_weight_grad), int(bias is not None), PANEL_BYTES
+                m, h, v, code, int(compute_weight_grad), int(bias is not None), get_panel_bytes()
             ),
             device,
         )
@@ -564,7 +717,7 @@ def masked_loss_backward(
                 int(ignore_index), int(exclude_index), float(logit_softcap),
                 float(logit_multiplier),
                 _ptr(grad_hidden), _ptr(grad_weight), _ptr(grad_bias32),
-                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_masked_loss_backward",
         )
@@ -673,7 +826,7 @@ def vocab_parallel_backward_local(
         )
         ws = _workspace(
             lib.tlce_backward_workspace_bytes(
-                m, h, v_local, code, 1, int(bias is not None), PANEL_BYTES
+                m, h, v_local, code, 1, int(bias is not None), get_panel_bytes()
             ),
             device,
         )
@@ -685,7 +838,7 @@ def vocab_parallel_backward_local(
                 reduction_code, int(vocab_start), int(ignore_index), int(exclude_index),
                 float(logit_softcap),
                 _ptr(grad_hidden), _ptr(grad_weight), _ptr(grad_bias32),
-                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_backward_local",
         )
@@ -721,12 +874,12 @@ def soft_embedding(
         out = torch.empty((m, h), dtype=hidden.dtype, device=device)
         if m == 0:
             return out
-        ws = _workspace(lib.tlce_soft_embedding_workspace_bytes(m, h, v, code, PANEL_BYTES), device)
+        ws = _workspace(lib.tlce_soft_embedding_workspace_bytes(m, h, v, code, get_panel_bytes()), device)
         _lib.check(
             lib.tlce_soft_embedding(
                 _ptr(hidden), _ptr(weight), m, h, v, code,
                 float(logit_softcap), float(embedding_scale), _ptr(out),
-                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_soft_embedding",
         )
@@ -772,12 +925,12 @@ def dflash_kl_forward(
         teacher_lse = torch.empty(m, dtype=torch.float32, device=device)
         if m == 0:
             return losses, draft_lse, teacher_lse
-        ws = _workspace(lib.tlce_kl_workspace_bytes(m, hd, ht, v, code, PANEL_BYTES), device)
+        ws = _workspace(lib.tlce_kl_workspace_bytes(m, hd, ht, v, code, get_panel_bytes()), device)
         _lib.check(
             lib.tlce_kl_forward(
                 _ptr(dh), _ptr(dw), _ptr(th), _ptr(tw), m, hd, ht, v, code,
                 float(logit_softcap), _ptr(losses), _ptr(draft_lse), _ptr(teacher_lse),
-                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_kl_forward",
         )
@@ -812,13 +965,13 @@ def dflash_kl_backward(
         grad_hidden = torch.empty((m, hd), dtype=dh.dtype, device=device)
         if m == 0:
             return grad_hidden
-        ws = _workspace(lib.tlce_kl_workspace_bytes(m, hd, ht, v, code, PANEL_BYTES), device)
+        ws = _workspace(lib.tlce_kl_workspace_bytes(m, hd, ht, v, code, get_panel_bytes()), device)
         _lib.check(
             lib.tlce_kl_backward(
                 _ptr(dh), _ptr(dw), _ptr(th), _ptr(tw),
                 _ptr(draft_lse), _ptr(teacher_lse), _ptr(grad_output),
                 m, hd, ht, v, code, float(logit_softcap), _ptr(grad_hidden),
-                PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_kl_backward",
         )
@@ -861,14 +1014,14 @@ def dflash_ce_topk_forward(
         top_ids = torch.empty((m, k), dtype=torch.long, device=device)
         if m:
             ws = _workspace(
-                lib.tlce_ce_topk_forward_workspace_bytes(m, h, v, code, PANEL_BYTES), device
+                lib.tlce_ce_topk_forward_workspace_bytes(m, h, v, code, get_panel_bytes()), device
             )
             _lib.check(
                 lib.tlce_ce_topk_forward(
                     _ptr(hidden), _ptr(weight), _ptr(labels), m, h, v, code, k,
                     float(output_multiplier), float(logit_softcap),
                     _ptr(loss), _ptr(probability), _ptr(top_values), _ptr(top_ids), _ptr(lse),
-                    PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                    get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
                 ),
                 "tlce_ce_topk_forward",
             )
@@ -912,14 +1065,14 @@ def dflash_ce_topk_backward(
         grad_hidden = torch.empty((m, h), dtype=hidden.dtype, device=device)
         if m:
             ws = _workspace(
-                lib.tlce_ce_topk_backward_workspace_bytes(m, h, v, code, PANEL_BYTES), device
+                lib.tlce_ce_topk_backward_workspace_bytes(m, h, v, code, get_panel_bytes()), device
             )
             _lib.check(
                 lib.tlce_ce_topk_backward(
                     _ptr(hidden), _ptr(weight), _ptr(labels), _ptr(lse), _ptr(top_ids),
                     _ptr(ce_scale), _ptr(gtv), m, h, v, code, k,
                     float(output_multiplier), float(logit_softcap), _ptr(grad_hidden),
-                    PANEL_BYTES, ws.data_ptr(), ws.numel(), _stream(device),
+                    get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
                 ),
                 "tlce_ce_topk_backward",
             )

@@ -578,6 +578,26 @@ extern "C" int tlce_ce_topk_backward(const void* hidden, const void* weight,
                                       stream));
 }
 
+// ------------------------------------------------ per-sample loss numerators --
+extern "C" int tlce_segment_weighted_sum(const float* values, const float* weights,
+                                         const int64_t* row_idx, const int64_t* row_count,
+                                         int64_t m, int64_t segment_length, int64_t n_segments,
+                                         float* out, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  TLCE_REQUIRE(m >= 0 && segment_length > 0 && n_segments >= 0 && n_segments < (1ll << 31),
+               "segment_weighted_sum: bad sizes m=%lld segment_length=%lld n_segments=%lld",
+               (long long)m, (long long)segment_length, (long long)n_segments);
+  if (n_segments == 0) return 0;
+  TLCE_REQUIRE(out != nullptr, "segment_weighted_sum: out is null");
+  TLCE_REQUIRE(m == 0 || (values != nullptr && row_idx != nullptr),
+               "segment_weighted_sum: null pointer");
+  ScopedTimer timer(kClassOther, stream);
+  lce_segment_weighted_sum_kernel<<<(int)n_segments, 256, 0, stream>>>(
+      values, weights, row_idx, row_count, m, segment_length, out);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
 extern "C" int tlce_profile_begin(void) {
   TLCE_REQUIRE(g_profiler == nullptr, "profile_begin: a session is already open on this thread");
   g_profiler = new Profiler();

@@ -45,6 +45,44 @@ __global__ __launch_bounds__(1024) void lce_sum_kernel(const float* __restrict__
   if (threadIdx.x == 0) out[0] = part[0];
 }
 
+// Per-sample numerators of the DFlash loss (numerators.scatter_add_(0, sample_indices,
+// token_loss * position_weights), dflash/model.py:925-937) without atomics: the
+// compacted rows are in ascending position order, so the rows of sample s (positions
+// [s * segment_length, (s + 1) * segment_length)) are one contiguous run of row_idx,
+// found by two binary searches; one workgroup per sample adds the run in a fixed
+// order (strided partial sums, then a pairwise tree): reproducible run to run.
+__global__ __launch_bounds__(256) void lce_segment_weighted_sum_kernel(
+    const float* __restrict__ values, const float* __restrict__ weights,
+    const int64_t* __restrict__ row_idx, const int64_t* __restrict__ row_count, int64_t m,
+    int64_t segment_length, float* __restrict__ out) {
+  __shared__ float part[256];
+  if (row_count != nullptr) {
+    const int64_t c = *row_count;
+    m = c < 0 ? 0 : (c < m ? c : m);
+  }
+  auto lower_bound = [&](int64_t position) -> int64_t {   // first r with row_idx[r] >= position
+    int64_t lo = 0, hi = m;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (row_idx[mid] < position) lo = mid + 1;
+      else hi = mid;
+    }
+    return lo;
+  };
+  const int64_t first = lower_bound((int64_t)blockIdx.x * segment_length);
+  const int64_t last = lower_bound(((int64_t)blockIdx.x + 1) * segment_length);
+  float s = 0.0f;
+  for (int64_t r = first + threadIdx.x; r < last; r += 256)
+    s += weights != nullptr ? values[r] * weights[r] : values[r];
+  part[threadIdx.x] = s;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = part[0];
+}
+
 // losses[r] = losses[r] + tsum[r] * lse_draft[r] + 1  (see lce_kl_panel_kernel)
 __global__ __launch_bounds__(256) void lce_kl_finish_kernel(float* losses, const float* tsum,
                                                             const float* lse, int m) {

@@ -25,6 +25,7 @@ class _FrozenLinearKL(torch.autograd.Function):
         losses, draft_lse, teacher_lse = native.dflash_kl_forward(*operands, float(logit_softcap))
         ctx.save_for_backward(*operands, draft_lse, teacher_lse)
         ctx.logit_softcap = float(logit_softcap)
+        ctx.panel_bytes = native.get_panel_bytes()   # the backward may run on another thread
         return losses
 
     @staticmethod
@@ -32,8 +33,9 @@ class _FrozenLinearKL(torch.autograd.Function):
         from . import chunked_linear_ce_native as native
 
         *operands, draft_lse, teacher_lse = ctx.saved_tensors
-        grad_hidden = native.dflash_kl_backward(*operands, draft_lse, teacher_lse,
-                                                grad_output.contiguous(), ctx.logit_softcap)
+        with native.panel_budget(ctx.panel_bytes):
+            grad_hidden = native.dflash_kl_backward(*operands, draft_lse, teacher_lse,
+                                                    grad_output.contiguous(), ctx.logit_softcap)
         return grad_hidden, None, None, None, None
 
 

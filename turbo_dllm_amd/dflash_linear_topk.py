@@ -31,6 +31,7 @@ class _NativeFrozenLinearCETopK(torch.autograd.Function):
         ctx.save_for_backward(hidden, weight, labels, lse, probability, top_ids)
         ctx.output_multiplier = float(output_multiplier)
         ctx.logit_softcap = float(logit_softcap)
+        ctx.panel_bytes = native.get_panel_bytes()   # the backward may run on another thread
         ctx.mark_non_differentiable(top_ids)
         return loss, probability, top_values, top_ids
 
@@ -40,14 +41,15 @@ class _NativeFrozenLinearCETopK(torch.autograd.Function):
 
         hidden, weight, labels, lse, probability, top_ids = ctx.saved_tensors
         zeros = torch.zeros_like(probability)
-        grad_hidden = native.dflash_ce_topk_backward(
-            hidden, weight, labels, lse, probability, top_ids,
-            zeros if grad_loss is None else grad_loss,
-            zeros if grad_probability is None else grad_probability,
-            grad_top_values,
-            row_block_size=0, output_multiplier=ctx.output_multiplier,
-            logit_softcap=ctx.logit_softcap,
-        )
+        with native.panel_budget(ctx.panel_bytes):
+            grad_hidden = native.dflash_ce_topk_backward(
+                hidden, weight, labels, lse, probability, top_ids,
+                zeros if grad_loss is None else grad_loss,
+                zeros if grad_probability is None else grad_probability,
+                grad_top_values,
+                row_block_size=0, output_multiplier=ctx.output_multiplier,
+                logit_softcap=ctx.logit_softcap,
+            )
         return grad_hidden, None, None, None, None, None
 
 

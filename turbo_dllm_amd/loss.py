@@ -27,8 +27,9 @@ from typing import Optional
 import torch
 from torch import nn
 
-from .compaction import compact_valid_loss_rows
-from .tiled_linear_cross_entropy import get_compaction_mode, tiled_linear_cross_entropy
+from .compaction import compact_valid_loss_rows, gather_rows
+from .options import resolve_compaction
+from .tiled_linear_cross_entropy import tiled_linear_cross_entropy
 
 _DEVICE_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
 
@@ -61,20 +62,8 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
         weight = weight.contiguous()
         n = hidden_flat.shape[0]
 
-        row_idx = row_count = None
-        rows, targets, token_weights, m = hidden_flat, labels_flat, weights_flat, n
-        if mode == "sync":
-            row_idx, m = native.compact_rows(labels_flat, -100)
-            if m == n:
-                row_idx = None
-            else:
-                rows = native.gather_rows(hidden_flat, row_idx)
-                targets = native.gather_rows(labels_flat, row_idx)
-                token_weights = native.gather_rows(weights_flat, row_idx)
-        elif mode == "device":
-            row_idx, row_count = native.compact_rows_device(labels_flat, -100)
-            rows, targets, token_weights = native.gather_loss_rows(
-                hidden_flat, labels_flat, weights_flat, row_idx, row_count, -100)
+        rows, targets, token_weights, row_idx, row_count, m = native.compact_loss_rows(
+            hidden_flat, labels_flat, weights_flat, -100, mode)
         _, lse, _, weighted_sum = native.masked_loss_forward(
             rows, weight, bias, targets, token_weights, m=m, row_idx=row_idx,
             row_count=row_count, n_out=n, ignore_index=-100, exclude_index=exclude_index,
@@ -85,6 +74,7 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
         ctx.hidden_shape = hidden.shape
         ctx.n_rows, ctx.m = n, m
         ctx.multiplier, ctx.exclude_index, ctx.logit_softcap = multiplier, exclude_index, logit_softcap
+        ctx.panel_bytes = native.get_panel_bytes()   # the backward may run on another thread
         return weighted_sum.reshape(())
 
     @staticmethod
@@ -92,13 +82,14 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
         from . import chunked_linear_ce_native as native
 
         rows, weight, bias, targets, token_weights, lse, row_idx, row_count = ctx.saved_tensors
-        grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(
-            rows, weight, bias, targets, token_weights, lse, None, grad_output,
-            reduction="sum", m=ctx.m, row_idx=row_idx, row_count=row_count, n_out=ctx.n_rows,
-            ignore_index=-100, exclude_index=ctx.exclude_index,
-            logit_softcap=ctx.logit_softcap, logit_multiplier=ctx.multiplier,
-            compute_weight_grad=ctx.needs_input_grad[1],
-        )
+        with native.panel_budget(ctx.panel_bytes):
+            grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(
+                rows, weight, bias, targets, token_weights, lse, None, grad_output,
+                reduction="sum", m=ctx.m, row_idx=row_idx, row_count=row_count, n_out=ctx.n_rows,
+                ignore_index=-100, exclude_index=ctx.exclude_index,
+                logit_softcap=ctx.logit_softcap, logit_multiplier=ctx.multiplier,
+                compute_weight_grad=ctx.needs_input_grad[1],
+            )
         return (
             grad_hidden.reshape(ctx.hidden_shape),
             grad_weight if ctx.needs_input_grad[1] else None,
@@ -125,6 +116,7 @@ class _FusedTokenLosses(torch.autograd.Function):
         ctx.save_for_backward(rows, weight, bias, targets, lse, valid_count)
         ctx.hidden_shape = hidden.shape
         ctx.multiplier, ctx.logit_softcap = multiplier, logit_softcap
+        ctx.panel_bytes = native.get_panel_bytes()
         return losses.reshape(labels.shape)
 
     @staticmethod
@@ -132,12 +124,13 @@ class _FusedTokenLosses(torch.autograd.Function):
         from . import chunked_linear_ce_native as native
 
         rows, weight, bias, targets, lse, valid_count = ctx.saved_tensors
-        grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(
-            rows, weight, bias, targets, None, lse, valid_count, grad_output,
-            reduction="none", ignore_index=-100, exclude_index=-1,
-            logit_softcap=ctx.logit_softcap, logit_multiplier=ctx.multiplier,
-            compute_weight_grad=ctx.needs_input_grad[1],
-        )
+        with native.panel_budget(ctx.panel_bytes):
+            grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(
+                rows, weight, bias, targets, None, lse, valid_count, grad_output,
+                reduction="none", ignore_index=-100, exclude_index=-1,
+                logit_softcap=ctx.logit_softcap, logit_multiplier=ctx.multiplier,
+                compute_weight_grad=ctx.needs_input_grad[1],
+            )
         return (
             grad_hidden.reshape(ctx.hidden_shape),
             grad_weight if ctx.needs_input_grad[1] else None,
@@ -170,6 +163,7 @@ def masked_token_loss(
     output_multiplier: Optional[float] = None,
     logit_softcap: Optional[float] = None,
     loss_scale: float = 1.0,
+    compaction: Optional[str] = None,
 ) -> torch.Tensor:
     """Weighted masked-token cross entropy of ``output_head`` on ``hidden``.
 
@@ -179,8 +173,9 @@ def masked_token_loss(
     or ``nn.Linear``, or a module that only offers ``parallel_cross_entropy``.
 
     Device tensors with a linear head take the fused path (see the module
-    docstring); how it compacts rows follows
-    ``tiled_linear_cross_entropy.set_compaction_mode``.  Host tensors, and heads
+    docstring); how it compacts rows follows ``compaction`` ("sync", "device" or
+    "none") or, when that is None, the calling context's
+    ``options.compaction_mode``.  Host tensors, and heads
     without a weight matrix, take the reference's sequence of calls.
     """
     excluded = int(mask_token_id) if (exclude_mask_token and mask_token_id is not None) else None
@@ -190,7 +185,7 @@ def masked_token_loss(
     multiplier = 1.0 if output_multiplier is None else float(output_multiplier)
     if isinstance(weight, torch.Tensor) and weight.dim() == 2 and _fused_path_applies(
             hidden, weight, bias, labels, multiplier, loss_weights):
-        mode = get_compaction_mode()
+        mode = resolve_compaction(compaction)
         if mode == "sync" and labels.numel() == 0:
             return zero_loss_with_module_parameters(hidden, output_head) / valid_token_count * float(
                 loss_scale)
@@ -268,3 +263,116 @@ def native_token_cross_entropy(
             weight_layout="vocab_first",
         )
     return losses.reshape(labels.shape).float()
+
+
+# ------------------------------------------------------------ DFlash loss method --
+class _SegmentWeightedSum(torch.autograd.Function):
+    """``out[s] = sum_r values[r] * weights[r]`` over the compacted rows of sample
+    ``s``, in a fixed order on the device (the reference's ``scatter_add_`` of the
+    per-token losses into per-sample numerators, dflash/model.py:925-937)."""
+
+    @staticmethod
+    def forward(ctx, values, weights, row_idx, segment_length, n_segments):  # type: ignore[override]
+        from . import chunked_linear_ce_native as native
+
+        ctx.save_for_backward(weights, row_idx)
+        ctx.segment_length = int(segment_length)
+        return native.segment_weighted_sum(values, weights, row_idx, segment_length, n_segments)
+
+    @staticmethod
+    def backward(ctx, grad_out):  # type: ignore[override]
+        weights, row_idx = ctx.saved_tensors
+        sample = torch.div(row_idx, ctx.segment_length, rounding_mode="floor")
+        return grad_out.index_select(0, sample) * weights, None, None, None, None
+
+
+def dflash_token_loss(
+    hidden_states: torch.Tensor,
+    target_token_ids: torch.Tensor,
+    supervised_mask: torch.Tensor,
+    position_weights: torch.Tensor,
+    lm_head: nn.Module,
+    *,
+    loss_kind: str,
+    normalization_count: torch.Tensor,
+    loss_scale: float = 1.0,
+    logit_softcap: Optional[float] = None,
+    teacher_hidden_states: Optional[torch.Tensor] = None,
+    teacher_head: Optional[nn.Module] = None,
+    teacher_norm: Optional[nn.Module] = None,
+) -> torch.Tensor:
+    """The DFlash drafter loss over the supervised positions of a ``[B, T]`` batch:
+
+        loss = mean_b( sum_{r in sample b} token_loss_r * w_r / (count_b + 1e-5) ) * loss_scale
+
+    One-GPU counterpart of ``distributed_dflash_loss``
+    (dllm_parallel/core/models/backbones/dflash/model.py:862-960).
+    ``hidden_states`` [B, T, H], ``target_token_ids`` / ``supervised_mask`` (bool) /
+    ``position_weights`` [B, T], ``normalization_count`` [B].  ``loss_kind``:
+
+      "paper_ce"        cross entropy of ``lm_head`` against the target tokens
+                        (``tiled_linear_cross_entropy``, reduction "none");
+      "speculators_kl"  forward KL of the frozen teacher head against the frozen draft
+                        head (``frozen_linear_kl``) on ``teacher_norm(teacher rows)``.
+
+    On the GPU the mask is scanned by the library's ballot / prefix-sum kernel,
+    rows are gathered by its gather kernel, and the per-sample numerators are
+    summed in a fixed order by one workgroup per sample (no ``scatter_add_``
+    atomics).  A batch with no supervised position returns a zero that keeps
+    the graph of ``hidden_states`` and ``lm_head`` alive, as the reference does.
+    """
+    from .dflash_kl import frozen_linear_kl
+
+    if loss_kind not in ("paper_ce", "speculators_kl"):
+        raise ValueError(f"unsupported DFlash loss {loss_kind!r}")
+    if supervised_mask.dim() != 2:
+        raise ValueError("DFlash supervised mask must be [batch, tokens]")
+    batch_size, tokens_per_sample = (int(x) for x in supervised_mask.shape)
+    hidden_flat = hidden_states.reshape(-1, hidden_states.shape[-1])
+    device_path = hidden_states.is_cuda
+    if device_path:
+        from . import chunked_linear_ce_native as native
+
+        valid_indices, n_valid = native.compact_mask(supervised_mask)
+    else:
+        valid_indices = torch.nonzero(supervised_mask.reshape(-1), as_tuple=False).flatten()
+        n_valid = valid_indices.numel()
+
+    denominators = normalization_count.to(device=hidden_states.device, dtype=torch.float32)
+    if tuple(denominators.shape) != (batch_size,):
+        raise ValueError("DFlash normalization count must contain one value per sample")
+
+    if n_valid == 0:
+        # numerators are all zero: only the dependence on the parameters remains
+        zero = zero_loss_with_module_parameters(hidden_states, lm_head)
+        numerators = zero.reshape(1).expand(batch_size) * 1.0
+    else:
+        hidden = gather_rows(hidden_flat, valid_indices)
+        weights = gather_rows(position_weights.reshape(-1).contiguous(),
+                              valid_indices).to(torch.float32)
+        if loss_kind == "speculators_kl":
+            if teacher_hidden_states is None or teacher_head is None:
+                raise RuntimeError("DFlash KL requires teacher logits")
+            with torch.no_grad():
+                teacher_hidden = gather_rows(
+                    teacher_hidden_states.reshape(-1, teacher_hidden_states.shape[-1]),
+                    valid_indices)
+                if teacher_norm is not None:
+                    teacher_hidden = teacher_norm(teacher_hidden)
+            token_loss = frozen_linear_kl(hidden, lm_head.weight, teacher_hidden,
+                                          teacher_head.weight, logit_softcap=logit_softcap)
+        else:
+            targets = gather_rows(target_token_ids.reshape(-1).contiguous(), valid_indices)
+            # the rows are compacted and every one of them bears loss
+            token_loss = tiled_linear_cross_entropy(
+                hidden, lm_head.weight, targets, reduction="none", dtype=hidden.dtype,
+                weight_layout="vocab_first", logit_softcap=logit_softcap, compaction="none")
+        if device_path:
+            numerators = _SegmentWeightedSum.apply(token_loss.float(), weights, valid_indices,
+                                                   tokens_per_sample, batch_size)
+        else:
+            sample_indices = torch.div(valid_indices, tokens_per_sample, rounding_mode="floor")
+            numerators = torch.zeros(batch_size, dtype=torch.float32, device=token_loss.device)
+            numerators = numerators.scatter_add(0, sample_indices, token_loss.float() * weights)
+    loss = (numerators / (denominators + 1.0e-5)).mean()
+    return loss * float(loss_scale)

@@ -22,47 +22,12 @@ from the softmax outright, also under a soft cap
 
 from __future__ import annotations
 
-import contextlib
 from typing import Optional
 
 import torch
 
-# How the device path deals with rows whose label is ``ignore_index``:
-#   "sync"   (default) compact them away on the device and read the count of
-#            loss-bearing rows back once, so every launch is sized exactly (the
-#            one host synchronisation the reference's call sites incur as well,
-#            nemotron/model.py:4244-4248);
-#   "device" compact them away without any host read-back: launches are sized
-#            for all rows and the kernels take the count from device memory, so
-#            the whole loss (forward and backward) can be recorded into a HIP
-#            graph;
-#   "none"   no compaction: the caller has compacted already (the reference's
-#            call sites do) or accepts GEMM work on ignored rows; the kernels
-#            zero their loss and gradient like the reference operator.
-COMPACTION_MODES = ("sync", "device", "none")
-_compaction_mode = "sync"
-
-
-def set_compaction_mode(mode: str) -> str:
-    """Selects how the device path handles ignored rows; returns the old mode."""
-    global _compaction_mode
-    if mode not in COMPACTION_MODES:
-        raise ValueError(f"compaction mode must be one of {COMPACTION_MODES}")
-    old, _compaction_mode = _compaction_mode, mode
-    return old
-
-
-def get_compaction_mode() -> str:
-    return _compaction_mode
-
-
-@contextlib.contextmanager
-def compaction_mode(mode: str):
-    old = set_compaction_mode(mode)
-    try:
-        yield
-    finally:
-        set_compaction_mode(old)
+from .options import (COMPACTION_MODES, compaction_mode, get_compaction_mode,  # noqa: F401
+                      resolve_compaction, set_compaction_mode)
 
 
 def _canonical_dtype(dtype: torch.dtype | str) -> torch.dtype:
@@ -267,7 +232,7 @@ class _HostTiledLinearCrossEntropy(torch.autograd.Function):
 
 # ---------------------------------------------------------------- device path --
 def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, exclude_index,
-                    compute_dtype, weight_dim_first, logit_softcap):
+                    compute_dtype, weight_dim_first, logit_softcap, mode):
     """Shared forward of the trainable- and frozen-head autograd functions.
 
     Mirrors ``_ChunkedDenseLinearCrossEntropy.forward``
@@ -284,21 +249,9 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
     if bias is not None:
         bias = bias.contiguous()
     n = hidden_flat.shape[0]
-    mode = _compaction_mode
 
-    row_idx = row_count = None
-    rows, targets, m = hidden_flat, labels_flat, n
-    if mode == "sync":
-        row_idx, m = native.compact_rows(labels_flat, ignore_index)
-        if m == n:
-            row_idx = None
-        else:
-            rows = native.gather_rows(hidden_flat, row_idx)
-            targets = native.gather_rows(labels_flat, row_idx)
-    elif mode == "device" and n > 0:
-        row_idx, row_count = native.compact_rows_device(labels_flat, ignore_index)
-        rows, targets, _ = native.gather_loss_rows(hidden_flat, labels_flat, None, row_idx,
-                                                   row_count, ignore_index)
+    rows, targets, _, row_idx, row_count, m = native.compact_loss_rows(
+        hidden_flat, labels_flat, None, ignore_index, mode)
 
     if row_count is None:
         losses, lse, valid_count = native.forward(
@@ -309,19 +262,22 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
         )
     else:
         losses, lse, valid_count, _ = native.masked_loss_forward(
-            rows, weight_vf, bias, targets, None, m=n, row_idx=row_idx, row_count=row_count,
+            rows, weight_vf, bias, targets, None, m=m, row_idx=row_idx, row_count=row_count,
             n_out=n, ignore_index=ignore_index, exclude_index=exclude_index,
             logit_softcap=float(logit_softcap), want_losses=True, want_sum=False,
         )
     ctx.save_for_backward(rows, weight_vf, bias, targets, lse, valid_count, row_idx, row_count)
     ctx.hidden_shape = hidden.shape
-    ctx.n_rows = n
+    ctx.n_rows, ctx.m = n, m
     ctx.reduction = reduction
     ctx.ignore_index = int(ignore_index)
     ctx.exclude_index = int(exclude_index)
     ctx.compute_dtype = compute_dtype
     ctx.weight_dim_first = weight_dim_first
     ctx.logit_softcap = float(logit_softcap)
+    # the backward may run on an autograd worker thread, which does not see this
+    # thread's context: the panel budget in force now travels with the node
+    ctx.panel_bytes = native.get_panel_bytes()
     if reduction == "none":
         return losses.reshape(labels.shape)
     if reduction == "sum":
@@ -333,29 +289,30 @@ def _device_backward(ctx, grad_output, frozen: bool):
     from . import chunked_linear_ce_native as native
 
     rows, weight_vf, bias, targets, lse, valid_count, row_idx, row_count = ctx.saved_tensors
-    if row_count is None:
-        call = native.backward_frozen_weight if frozen else native.backward
-        grad_hidden, grad_weight, grad_bias = call(
-            rows, weight_vf, bias, targets, lse, valid_count, grad_output,
-            row_block_size=0, reduction=ctx.reduction, ignore_index=ctx.ignore_index,
-            exclude_index=ctx.exclude_index, logit_softcap=ctx.logit_softcap,
-            compute_dtype=ctx.compute_dtype, weight_dim_first=False,
-            row_idx=row_idx, n_out=ctx.n_rows,
-        )
-    else:
-        grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(
-            rows, weight_vf, bias, targets, None, lse, valid_count, grad_output,
-            reduction=ctx.reduction, m=ctx.n_rows, row_idx=row_idx, row_count=row_count,
-            n_out=ctx.n_rows, ignore_index=ctx.ignore_index, exclude_index=ctx.exclude_index,
-            logit_softcap=ctx.logit_softcap, compute_weight_grad=not frozen,
-        )
+    with native.panel_budget(ctx.panel_bytes):
+        if row_count is None:
+            call = native.backward_frozen_weight if frozen else native.backward
+            grad_hidden, grad_weight, grad_bias = call(
+                rows, weight_vf, bias, targets, lse, valid_count, grad_output,
+                row_block_size=0, reduction=ctx.reduction, ignore_index=ctx.ignore_index,
+                exclude_index=ctx.exclude_index, logit_softcap=ctx.logit_softcap,
+                compute_dtype=ctx.compute_dtype, weight_dim_first=False,
+                row_idx=row_idx, n_out=ctx.n_rows,
+            )
+        else:
+            grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(
+                rows, weight_vf, bias, targets, None, lse, valid_count, grad_output,
+                reduction=ctx.reduction, m=ctx.m, row_idx=row_idx, row_count=row_count,
+                n_out=ctx.n_rows, ignore_index=ctx.ignore_index, exclude_index=ctx.exclude_index,
+                logit_softcap=ctx.logit_softcap, compute_weight_grad=not frozen,
+            )
     if not frozen and ctx.weight_dim_first:
         grad_weight = grad_weight.t().contiguous()
     return (
         grad_hidden.reshape(ctx.hidden_shape),
         None if frozen else grad_weight,
         None if bias is None else grad_bias,
-    ) + (None,) * 8
+    ) + (None,) * 9
 
 
 class _ChunkedDenseLinearCrossEntropy(torch.autograd.Function):
@@ -363,10 +320,12 @@ class _ChunkedDenseLinearCrossEntropy(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, weight, bias, labels, row_block_size, reduction, ignore_index,
-                exclude_index, compute_dtype, weight_dim_first, logit_softcap):  # type: ignore[override]
+                exclude_index, compute_dtype, weight_dim_first, logit_softcap,
+                compaction="sync"):  # type: ignore[override]
         del row_block_size
         return _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index,
-                               exclude_index, compute_dtype, weight_dim_first, logit_softcap)
+                               exclude_index, compute_dtype, weight_dim_first, logit_softcap,
+                               compaction)
 
     @staticmethod
     def backward(ctx, grad_output):  # type: ignore[override]
@@ -379,10 +338,12 @@ class _ChunkedFrozenLinearCrossEntropy(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, hidden, weight, bias, labels, row_block_size, reduction, ignore_index,
-                exclude_index, compute_dtype, weight_dim_first, logit_softcap):  # type: ignore[override]
+                exclude_index, compute_dtype, weight_dim_first, logit_softcap,
+                compaction="sync"):  # type: ignore[override]
         del row_block_size
         return _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index,
-                               exclude_index, compute_dtype, weight_dim_first, logit_softcap)
+                               exclude_index, compute_dtype, weight_dim_first, logit_softcap,
+                               compaction)
 
     @staticmethod
     def backward(ctx, grad_output):  # type: ignore[override]
@@ -414,6 +375,7 @@ def tiled_linear_cross_entropy(
     logit_softcap: float | None = None,
     dtype: torch.dtype | str = torch.float32,
     weight_layout: str = "auto",
+    compaction: Optional[str] = None,
 ) -> torch.Tensor:
     """Linear projection plus cross entropy without materializing [N, V] logits.
 
@@ -429,6 +391,10 @@ def tiled_linear_cross_entropy(
       exclude_index: vocabulary id removed from the softmax (e.g. the mask token).
       logit_softcap: positive cap applied as ``cap * tanh(logit / cap)``.
       dtype: matmul dtype of the host path; accumulation is float32 everywhere.
+      compaction: how the device path removes ignored rows ("sync", "device" or
+        "none", see ``options.COMPACTION_MODES``); None takes the mode of the
+        calling context (``compaction_mode(...)``).  Not part of the reference's
+        signature; the host path ignores it.
 
     Returns the same value as ``F.cross_entropy(hidden @ lm_head.T + bias, labels)``
     up to floating-point associativity; float32, shaped like ``labels`` for
@@ -453,7 +419,7 @@ def tiled_linear_cross_entropy(
         )
         return implementation.apply(
             hidden, lm_head, bias, labels, 0, reduction, int(ignore_index), excluded,
-            compute_dtype, weight_dim_first, softcap,
+            compute_dtype, weight_dim_first, softcap, resolve_compaction(compaction),
         )
     if hidden.is_cuda or lm_head.is_cuda or labels.is_cuda:
         raise RuntimeError(
