@@ -139,3 +139,51 @@ def test_ties_go_to_the_smaller_id(gpu_device):
     assert torch.count_nonzero(vals) == 0
     torch.testing.assert_close(loss.cpu(), torch.full((n,), float(torch.log(torch.tensor(float(v))))),
                                rtol=1e-5, atol=1e-5)
+
+
+EXACT_CASES = [
+    # name, rows, h, v, k, multiplier, panel_bytes (0 = default: one panel)
+    ("k1_five_chunks", 70, 64, 70000, 1, 1.0, 0),
+    ("k16_two_panels_two_chunks", 300, 64, 40000, 16, 1.0, 512 * 20480 * 4),
+    ("k256_selection_rounds", 40, 64, 40000, 256, 0.5, 0),
+    ("k16_many_panels", 130, 32, 20000, 16, 2.0, 256 * 2048 * 4),
+    ("k256_many_panels", 257, 64, 33000, 256, 1.0, 512 * 4096 * 4),
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", EXACT_CASES, ids=[c[0] for c in EXACT_CASES])
+def test_selection_is_exact_on_exactly_representable_logits(gpu_device, case, set_panel_budget):
+    """The selection isolated from matmul rounding: small-integer hidden states and
+    weights in eighths make every product and every float32 partial sum exact, so
+    the device's logits equal the oracle's bit for bit and the top-k ids and
+    values must too, ties (there are thousands per row) going to the smaller id
+    (at::topk semantics of the reference, fused_linear_ce_cuda.cu:1602 /
+    dflash_linear_topk.py:100-158).  Covers rows spanning several 16384-logit
+    chunks, several vocabulary panels, and k = 256 (selection rounds)."""
+    name, n, h, v, k, mult, panel_bytes = case
+    print("[case] exact top-k", name, flush=True)
+    if panel_bytes:
+        set_panel_budget(panel_bytes)
+    gen = torch.Generator().manual_seed(len(name) * 7 + k)
+    hidden = torch.randint(-3, 4, (n, h), generator=gen).to(torch.bfloat16)
+    weight = (torch.randint(-8, 9, (v, h), generator=gen).float() / 8.0).to(torch.bfloat16)
+    # a few rows with extreme ties: constant rows and rows with one distinct logit
+    hidden[0] = 0
+    if n > 2:
+        hidden[1] = 0
+        hidden[1, 0] = 1
+    labels = torch.randint(0, v, (n,), generator=gen)
+    loss, prob, vals, ids = frozen_linear_ce_topk(hidden.to(gpu_device), weight.to(gpu_device),
+                                                  labels.to(gpu_device), top_k=k,
+                                                  output_multiplier=mult)
+    torch.cuda.synchronize()
+    r_loss, _, r_vals, r_ids, _ = oracle.dense_ce_topk(hidden, weight, labels, k,
+                                                       output_multiplier=mult)
+    z = oracle._topk_logits(hidden, weight, mult, None, torch.float64)[0]
+    assert bool((z == z.float().double()).all())          # the logits are float32-exact
+    ties = int((z[:, :, None] == r_vals[:, None, -1:]).sum(dim=1).max())
+    print("[case] logits tied with the k-th value in the worst row:", ties, flush=True)
+    assert torch.equal(ids.cpu(), r_ids)
+    assert torch.equal(vals.cpu().double(), r_vals)
+    torch.testing.assert_close(loss.cpu().double(), r_loss, rtol=1e-4, atol=1e-4)

@@ -129,3 +129,55 @@ def test_whole_loss_with_device_row_count_replays_for_any_mask(gpu_device, n, h,
             native.gather_rows(weights, idx), row_idx=idx if m < n else None, n_out=n,
             want_losses=False, want_sum=True, **kw)
         assert torch.equal(total, got[0]), (replay, rate)
+
+
+@pytest.mark.parametrize("n,hd,ht,v,softcap", [(300, 128, 64, 1536, 0.0), (130, 72, 96, 1025, 5.0)])
+def test_frozen_kl_graph_replays_match_eager(gpu_device, n, hd, ht, v, softcap, set_panel_budget):
+    """The KL of two frozen heads, forward and backward, from one graph: its
+    loss is accumulated per vocabulary tile and merged in a fixed order (no
+    float atomics), so replays and eager runs agree bit for bit, and so do
+    repeated eager runs."""
+    print("[case] KL graph capture", n, hd, ht, v, softcap, flush=True)
+    dev = gpu_device
+    set_panel_budget(512 * 512 * 2)      # several vocabulary panels
+    gen = torch.Generator().manual_seed(n + v)
+    draft_w = (torch.randn(v, hd, generator=gen) * 0.2).bfloat16().to(dev)
+    teacher_w = (torch.randn(v, ht, generator=gen) * 0.2).bfloat16().to(dev)
+
+    def make():
+        return (torch.randn(n, hd, generator=gen).bfloat16(),
+                torch.randn(n, ht, generator=gen).bfloat16(),
+                torch.rand(n, generator=gen) + 0.5)
+
+    def run(draft_h, teacher_h, go):
+        losses, draft_lse, teacher_lse = native.dflash_kl_forward(draft_h, draft_w, teacher_h,
+                                                                  teacher_w, softcap)
+        grad = native.dflash_kl_backward(draft_h, draft_w, teacher_h, teacher_w, draft_lse,
+                                         teacher_lse, go, softcap)
+        return losses, grad
+
+    static = [torch.zeros(n, hd, dtype=torch.bfloat16, device=dev),
+              torch.zeros(n, ht, dtype=torch.bfloat16, device=dev),
+              torch.zeros(n, dtype=torch.float32, device=dev)]
+    first = make()
+    for s, t in zip(static, first):
+        s.copy_(t)
+    run(*static)                                  # warm-up: one-time kernel attributes
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outputs = run(*static)
+    torch.cuda.synchronize()
+    for replay in range(4):
+        case = first if replay == 0 else make()
+        for s, t in zip(static, case):
+            s.copy_(t)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outputs]
+        eager = run(*[t.to(dev) for t in case])   # eager work between replays
+        again = run(*[t.to(dev) for t in case])
+        torch.cuda.synchronize()
+        for name, a, b, c in zip(("losses", "grad_hidden"), got, eager, again):
+            assert torch.equal(a, b), (replay, name)
+            assert torch.equal(b, c), (replay, name, "eager runs differ")

@@ -37,10 +37,42 @@ def draw(case):
     )
 
 
-@pytest.mark.parametrize("case", range(48))
+def within(name, err, bar):
+    """One error against its bar, printed so that a log names the measured value."""
+    print("[err]", name, f"{float(err):.3e}", "bar", bar, flush=True)
+    assert float(err) <= bar, (name, float(err), bar)
+
+
+# Draws of the same generator that a 40 000-case run once found outside the usual bars,
+# kept in the suite.  Two of them (float32 inputs with a soft cap) were the hardware tanh
+# approximation, 1 - 2 / (1 + e^2x), losing relative accuracy for small arguments; the
+# float32 engine now calls the library's tanhf / exp2f and they hold the plain bars
+# (measured 4e-6 and 2e-6).  The other three are the masked-token loss with output
+# multiplier 1.75 on one or two rows and a 3-word vocabulary: the row is predicted
+# confidently, so its whole gradient is the difference exp(z - lse) - 1 (and its mirror
+# image on the other two columns), a cancellation that leaves float32 arithmetic - and
+# the 16-bit rounding of the staged gradient - a relative error of eps / |g|.  The
+# reference's kernel forms the same difference (fused_linear_ce_cuda.cu:270-283).  With
+# more rows the other rows set the gradient's scale and the same absolute error is
+# invisible.  `widen` is the factor on the gradient bar; `measured` what this build gives.
+HARD_CASES = {
+    7954: dict(widen=2.0, measured="3.7e-2 against 2e-2",
+               why="bf16, 2 rows, V=3: one rounded gradient entry of magnitude 1e-5"),
+    17331: dict(widen=1.0, measured="1.8e-5 against 2e-5",
+                why="float32, 1 row, V=3, soft cap 30: was the tanh approximation"),
+    17376: dict(widen=2.0, measured="2.4e-5 against 2e-5",
+                why="float32, 1 row, V=3, bias: exp(z - lse) - 1 cancels"),
+    21238: dict(widen=3.0, measured="4.1e-5 against 2e-5",
+                why="float32, 1 row, V=3, bias: exp(z - lse) - 1 cancels"),
+    37105: dict(widen=1.0, measured="1.6e-6 against 2e-5",
+                why="float32, 1 row, soft cap 2: was the tanh approximation"),
+}
+
+
+@pytest.mark.parametrize("case", list(range(48)) + sorted(HARD_CASES))
 def test_random_case(gpu_device, case):
     c = draw(case)
-    print("[case]", case, c, flush=True)
+    print("[case]", case, c, HARD_CASES.get(case, ""), flush=True)
     dev = gpu_device
     n, h, v, dtype, softcap = c["n"], c["h"], c["v"], c["dtype"], c["softcap"]
     gen = torch.Generator().manual_seed(case)
@@ -54,7 +86,8 @@ def test_random_case(gpu_device, case):
     labels[torch.rand(n, generator=gen) < 0.3] = -100
     if int((labels != -100).sum()) == 0:
         labels[0] = 0 if exclude != 0 else 1 % v
-    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    widen = HARD_CASES.get(case, {}).get("widen", 1.0)
+    tol = (2e-5 if dtype == torch.float32 else 2e-2) * widen
     ltol = 1e-5 if dtype == torch.float32 else 1e-3
 
     # cross entropy, forward and backward
@@ -71,11 +104,11 @@ def test_random_case(gpu_device, case):
     ref = oracle.dense_linear_ce(hidden, weight, labels, **kw)
     rdh, rdw, rdb = oracle.dense_linear_ce_grads(hidden, weight, labels, go, **kw)
     torch.testing.assert_close(loss.detach().cpu().double(), ref.double(), rtol=ltol, atol=ltol)
-    assert oracle.relative_max_error(x.grad.cpu(), rdh) <= tol
+    within("ce dH", oracle.relative_max_error(x.grad.cpu(), rdh), tol)
     if not c["frozen"]:
-        assert oracle.relative_max_error(w.grad.cpu(), rdw) <= tol
+        within("ce dW", oracle.relative_max_error(w.grad.cpu(), rdw), tol)
     if bias is not None:
-        assert oracle.relative_max_error(b.grad.cpu(), rdb) <= tol
+        within("ce db", oracle.relative_max_error(b.grad.cpu(), rdb), tol)
 
     # the loss method around the operator, with the row count read back, kept on the
     # device, or rows left in place (the capacity-sized launches of the device mode
@@ -102,16 +135,17 @@ def test_random_case(gpu_device, case):
     mref = oracle.masked_token_loss(hidden, weight, labels, weights, 3.0, **mkw)
     mdh, mdw, mdb = oracle.masked_token_loss_grads(hidden, weight, labels, weights, 3.0, **mkw)
     torch.testing.assert_close(total.detach().cpu().double(), mref.double(), rtol=ltol, atol=ltol)
-    assert oracle.relative_max_error(xm.grad.cpu(), mdh) <= tol, mode
-    assert oracle.relative_max_error(head.weight.grad.cpu(), mdw) <= tol, mode
+    within(f"masked loss dH ({mode})", oracle.relative_max_error(xm.grad.cpu(), mdh), tol)
+    within(f"masked loss dW ({mode})", oracle.relative_max_error(head.weight.grad.cpu(), mdw), tol)
     if bias is not None:
-        assert oracle.relative_max_error(head.bias.grad.cpu(), mdb) <= tol, mode
+        within(f"masked loss db ({mode})", oracle.relative_max_error(head.bias.grad.cpu(), mdb),
+               tol)
 
     # soft embedding
     soft = streaming_soft_embedding(hidden.to(dev), weight.to(dev), row_chunk_size=64,
                                     vocab_chunk_size=64, logit_softcap=softcap)
     expect = oracle.dense_soft_embedding(hidden, weight, logit_softcap=softcap)
-    assert oracle.relative_max_error(soft.cpu(), expect) <= tol
+    within("soft embedding", oracle.relative_max_error(soft.cpu(), expect), tol)
 
     # forward KL against a teacher head of another width
     ht = c["h_teacher"]
@@ -129,7 +163,7 @@ def test_random_case(gpu_device, case):
         rtol=10 * ltol, atol=10 * ltol)
     kl_grad = oracle.dense_frozen_kl_grad(hidden, weight, teacher_h, teacher_w, scale,
                                           logit_softcap=softcap)
-    assert oracle.relative_max_error(xk.grad.cpu(), kl_grad) <= 2 * tol
+    within("kl grad", oracle.relative_max_error(xk.grad.cpu(), kl_grad), 2 * tol)
 
     # cross entropy with top-k (16-bit inputs run in the library)
     if dtype != torch.float32:
@@ -148,4 +182,4 @@ def test_random_case(gpu_device, case):
         torch.testing.assert_close(values.detach().cpu().double(), rv, rtol=1e-3, atol=1e-3)
         rg = oracle.dense_ce_topk_grad(hidden, weight, targets, ids.cpu(), gl, gp, gv,
                                        output_multiplier=0.8, logit_softcap=softcap)
-        assert oracle.relative_max_error(xt.grad.cpu(), rg) <= tol
+        within("ce top-k grad", oracle.relative_max_error(xt.grad.cpu(), rg), tol)

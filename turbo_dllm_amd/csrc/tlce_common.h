@@ -129,6 +129,27 @@ __device__ __forceinline__ float fast_tanh(float x) {
   return 1.0f - 2.0f * fast_rcp(1.0f + e);
 }
 
+// Elementwise math by engine.  The float32 engine (float32 inputs, held to the
+// reference's 2e-5 bars) takes the library routines: fast_tanh loses relative
+// accuracy for small arguments (1 - 2 / (1 + e) cancels), which the soft cap's
+// derivative then carries into the gradient.  The 16-bit engines take the
+// hardware approximations, whose error is far below the rounding of their inputs.
+template <bool kPrecise>
+__device__ __forceinline__ float exp2_of(float x) {
+  if constexpr (kPrecise) return exp2f(x);
+  else return fast_exp2(x);
+}
+template <bool kPrecise>
+__device__ __forceinline__ float log2_of(float x) {
+  if constexpr (kPrecise) return log2f(x);
+  else return fast_log2(x);
+}
+template <bool kPrecise>
+__device__ __forceinline__ float tanh_of(float x) {
+  if constexpr (kPrecise) return tanhf(x);
+  else return fast_tanh(x);
+}
+
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

@@ -58,6 +58,7 @@ struct MfmaTileLayout {
   static constexpr int kCols = kTN;          // tile columns owned per thread
   static constexpr int kRows = kTM * 16;     // tile rows held per owned column
   static constexpr int kShare = 4;           // threads that hold the same column
+  static constexpr bool kPrecise = false;    // hardware exp / rcp approximations in the epilogues
   static_assert(kWavesN * kTN * 32 == kTile, "waves must tile the 256 B rows");
 
   struct Acc { f32x16_t c[kTM][kTN]; };

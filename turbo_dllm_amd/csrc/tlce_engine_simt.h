@@ -24,6 +24,7 @@ struct SimtEngine {
   static constexpr int kRows = 16;
   static constexpr int kShare = 4;
   static constexpr bool kHasKMajor = false;
+  static constexpr bool kPrecise = sizeof(T_) == 4;   // float32 inputs: library exp / tanh
 
   struct Acc { float c[kRows]; };
 

@@ -317,8 +317,8 @@ int launch_transpose(const T* in, int64_t ld_in, int64_t rows, int64_t cols, T* 
 // beside the C ABI.
 int fill_zero(void* dst, int64_t bytes, hipStream_t stream);
 int launch_token_scale(const ScaleArgs& sa, hipStream_t stream);
-int launch_kl_finish(float* losses, const float* tsum, const float* lse, int64_t m,
-                     hipStream_t stream);
+int launch_kl_finish(float* losses, const float* loss_part, const float* tsum_part, int n_tiles,
+                     int64_t part_ld, const float* lse, int64_t m, hipStream_t stream);
 int launch_topk_scan(const TopkScanArgs& sa, hipStream_t stream);
 int launch_sum(const float* x, int64_t n, float* out, hipStream_t stream);
 
@@ -540,18 +540,17 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
 // Both heads run on one engine class (the less demanding of the two hidden sizes).
 struct KlLayout {
   // stats: the teacher's forward partials, then the draft's per-tile partials
-  // (part_max, part_sum: n_vtiles x mp float32 each); backward: BackwardLayout
-  // of the draft head
-  int64_t stats, tile_part, ones, tsum, backward, total;
+  // (part_max, part_sum, loss terms, teacher mass: n_vtiles x mp float32 each);
+  // backward: BackwardLayout of the draft head
+  int64_t stats, tile_part, ones, backward, total;
 };
 
 inline KlLayout kl_layout(const Plan& pd, const Plan& pt, int64_t m, int64_t hd, int dtype) {
   KlLayout l;
   l.stats = 0;
   l.tile_part = align256((int64_t)pd.n_vtiles * pd.mp * 4);
-  int64_t off = std::max(2 * l.tile_part, forward_layout(pt).total);
+  int64_t off = std::max(4 * l.tile_part, forward_layout(pt).total);
   l.ones = off;      off += align256(pd.mp * 4);
-  l.tsum = off;      off += align256(pd.mp * 4);
   l.backward = off;  off += backward_layout(pd, m, hd, dtype, false).total;
   l.total = off;
   return l;
@@ -586,8 +585,8 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
              const void* teacher_hidden, const void* teacher_weight, const float* draft_lse,
              const float* teacher_lse, const float* ones, const float* scale, int64_t m,
              int64_t hd, int64_t ht, int64_t v, float softcap, int64_t v0, int64_t width,
-             void* g, float* losses, float* tsum, float* part_max, float* part_sum, int mode,
-             hipStream_t stream) {
+             void* g, float* loss_part, float* tsum_part, float* part_max, float* part_sum,
+             int mode, hipStream_t stream) {
   GradLogitsArgs ga;
   ga.hidden = teacher_hidden; ga.weight = teacher_weight; ga.bias = nullptr;
   ga.labels = nullptr; ga.lse = teacher_lse; ga.scale = ones;
@@ -603,7 +602,7 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
   ka.hidden = draft_hidden; ka.weight = draft_weight; ka.lse = draft_lse; ka.scale = scale;
   ka.m = (int)m; ka.h = (int)hd; ka.v = (int)v; ka.softcap = softcap;
   ka.v0 = (int)v0; ka.n_ttiles = pd.n_ttiles; ka.n_ptiles = (int)(width / pd.tile);
-  ka.panel = g; ka.ld = pd.vc; ka.losses = losses; ka.tsum = tsum;
+  ka.panel = g; ka.ld = pd.vc; ka.loss_part = loss_part; ka.tsum_part = tsum_part;
   ka.part_max = part_max; ka.part_sum = part_sum; ka.part_ld = (int)pd.mp; ka.mode = mode;
   return launch_kl_panel<E>(ka, stream);
 }
@@ -621,16 +620,15 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
                                ws + l.stats, stream, RowOptions{}))
     return rc;
   float* ones = reinterpret_cast<float*>(ws + l.ones);
-  float* tsum = reinterpret_cast<float*>(ws + l.tsum);
   float* part_max = reinterpret_cast<float*>(ws + l.stats);
   float* part_sum = reinterpret_cast<float*>(ws + l.stats + l.tile_part);
+  float* loss_part = reinterpret_cast<float*>(ws + l.stats + 2 * l.tile_part);
+  float* tsum_part = reinterpret_cast<float*>(ws + l.stats + 3 * l.tile_part);
   ScaleArgs sa;
   sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = nullptr; sa.valid_count = nullptr;
   sa.m = (int)m; sa.mp = (int)pd.mp; sa.reduction = TLCE_REDUCTION_SUM; sa.ignore = 0;
   sa.scale = ones; sa.constant = 1.0f; sa.multiplier = 1.0f;
   if (int rc = launch_token_scale(sa, stream)) return rc;
-  if (int rc = fill_zero(tsum, pd.mp * 4, stream)) return rc;
-  if (int rc = fill_zero(losses, m * 4, stream)) return rc;
   // one pass over the draft head per panel: loss terms and the draft's per-tile
   // softmax partials (the teacher partials above are dead by now)
   const BackwardLayout bl = backward_layout(pd, m, hd, dtype, false);
@@ -640,7 +638,8 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
     const int64_t width = std::min<int64_t>(pd.vc, pd.vp - v0);
     if (int rc = kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight,
                              nullptr, teacher_lse, ones, nullptr, m, hd, ht, v, softcap, v0,
-                             width, g, losses, tsum, part_max, part_sum, kKlLoss, stream))
+                             width, g, loss_part, tsum_part, part_max, part_sum, kKlLoss,
+                             stream))
       return rc;
   }
   CombineArgs ca;
@@ -656,7 +655,9 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
     ScopedTimer timer(kClassCombine, stream);
     lce_combine_loss_kernel<T><<<(int)ceil_div(m, kCombineRowsPerBlock), 256, 0, stream>>>(ca);
     TLCE_LAUNCH_CHECK();
-    if (int rc = launch_kl_finish(losses, tsum, draft_lse, m, stream)) return rc;
+    if (int rc = launch_kl_finish(losses, loss_part, tsum_part, pd.n_vtiles, pd.mp, draft_lse, m,
+                                  stream))
+      return rc;
   }
   return 0;
 }

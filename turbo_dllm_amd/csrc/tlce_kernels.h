@@ -103,7 +103,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
 #pragma unroll
         for (int j = 0; j < E::kCols; ++j) {
           float z = E::get(acc, j, i);
-          if (kSoftcap) z = p.softcap * fast_tanh(z * inv_cap);
+          if (kSoftcap) z = p.softcap * tanh_of<E::kPrecise>(z * inv_cap);
           E::set(acc, j, i, ok ? z : -INFINITY);
         }
       }
@@ -116,10 +116,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
       for (int i = 0; i < E::kRows; ++i) tile_max = fmaxf(tile_max, E::get(acc, j, i));
       const float new_max = fmaxf(run_max[j], tile_max * log2e_scaled);
       if (new_max > -INFINITY) {
-        float s = run_sum[j] * fast_exp2(run_max[j] - new_max);
+        float s = run_sum[j] * exp2_of<E::kPrecise>(run_max[j] - new_max);
 #pragma unroll
         for (int i = 0; i < E::kRows; ++i)
-          s += fast_exp2(fmaf(E::get(acc, j, i), log2e_scaled, -new_max));
+          s += exp2_of<E::kPrecise>(fmaf(E::get(acc, j, i), log2e_scaled, -new_max));
         run_sum[j] = s;
         run_max[j] = new_max;
       }
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
     if (mx > -INFINITY) {
 #pragma unroll
       for (int s = 0; s < E::kShare; ++s)
-        sum += sh_sum[s * E::kTile + c] * fast_exp2(sh_max[s * E::kTile + c] - mx);
+        sum += sh_sum[s * E::kTile + c] * exp2_of<E::kPrecise>(sh_max[s * E::kTile + c] - mx);
     }
     const int64_t o = (int64_t)vs * p.part_ld + tt * E::kTile + c;
     p.part_max[o] = mx;
@@ -244,7 +244,7 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
     float sum = 0.0f;
     for (int s = lane; s < p.nsplit; s += 64) {
       const float pm = p.part_max[(int64_t)s * p.part_ld + r];
-      if (pm > -INFINITY) sum += p.part_sum[(int64_t)s * p.part_ld + r] * fast_exp2(pm - mx);
+      if (pm > -INFINITY) sum += p.part_sum[(int64_t)s * p.part_ld + r] * exp2_of<sizeof(T) == 4>(pm - mx);
     }
     sum = wave_sum(sum);
     const float lse = (mx + log2f(sum)) * TLCE_LN2;
@@ -443,12 +443,12 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
     float dcap = 1.0f;
     float g;
     if (kSoftcap) {
-      const float t = fast_tanh(z * inv_cap);   // inv_cap includes logit_scale
+      const float t = tanh_of<E::kPrecise>(z * inv_cap);   // inv_cap includes logit_scale
       z = p.softcap * t;
       dcap = 1.0f - t * t;
-      g = fast_exp2(fmaf(z, TLCE_LOG2E, -lse2[j]));
+      g = exp2_of<E::kPrecise>(fmaf(z, TLCE_LOG2E, -lse2[j]));
     } else {
-      g = fast_exp2(fmaf(z, log2e_scaled, -lse2[j]));
+      g = exp2_of<E::kPrecise>(fmaf(z, log2e_scaled, -lse2[j]));
     }
     if (kOnehot && row == label_row[j]) g -= 1.0f;
     g *= scale[j];
@@ -588,8 +588,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 // t = softmax(cap(z_teacher)) rounded to the input dtype (written by
 // lce_grad_logits_panel_kernel in its probabilities mode).  This kernel
 // recomputes the draft logits tile and, with lp = cap(z_draft) - lse_draft:
-//   mode kKlLoss: losses[token] += sum_v ( t * (log t - cap(z_draft)) - t ),
-//                 tsum[token] += sum_v t, and the tile's (max, sum exp) of the
+//   mode kKlLoss: per vocabulary tile and token, sum_v ( t * (log t - cap(z_draft)) - t )
+//                 and sum_v t go to loss_part / tsum_part (one slot per tile, no
+//                 atomics: the caller adds the tiles in a fixed order, so the loss
+//                 is reproducible run to run), and the tile's (max, sum exp) of the
 //                 draft logits go to the forward partial arrays, so that no
 //                 separate statistics pass over the draft head is needed.  The
 //                 caller finishes with loss = losses + tsum * lse_draft + 1: the
@@ -612,8 +614,8 @@ struct KlPanelArgs {
   int n_ttiles, n_ptiles;
   void* panel;          // [mp, ld] teacher probabilities in, logit gradients out
   int64_t ld;
-  float* losses;        // kKlLoss: [m], accumulated with atomics
-  float* tsum;          // kKlLoss: [m], accumulated with atomics
+  float* loss_part;     // kKlLoss: [n vocabulary tiles, part_ld] loss terms of the tile
+  float* tsum_part;     // kKlLoss: [n vocabulary tiles, part_ld] teacher mass of the tile
   float* part_max;      // kKlLoss: [n vocabulary tiles, part_ld] base-2 tile maxima
   float* part_sum;      //          and sums of exp2(z2 - max2), as the forward writes them
   int part_ld;
@@ -662,7 +664,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
 #pragma unroll
       for (int j = 0; j < E::kCols; ++j) {
         float z = E::get(acc, j, i);
-        if (kSoftcap) z = p.softcap * fast_tanh(z * inv_cap);
+        if (kSoftcap) z = p.softcap * tanh_of<E::kPrecise>(z * inv_cap);
         z = vok ? z * TLCE_LOG2E : -INFINITY;
         E::set(acc, j, i, z);
         tile_max[j] = fmaxf(tile_max[j], z);
@@ -684,21 +686,21 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
       if (grad) {
         float dcap = 1.0f;
         if (kSoftcap) {
-          const float th = fast_tanh(z * inv_cap);
+          const float th = tanh_of<E::kPrecise>(z * inv_cap);
           z = p.softcap * th;
           dcap = 1.0f - th * th;
         }
         const float lp2 = fmaf(z, TLCE_LOG2E, -lse2[j]);   // log2 of the draft probability
-        const float v = (fast_exp2(lp2) - t[u]) * scale[j] * dcap;
+        const float v = (exp2_of<E::kPrecise>(lp2) - t[u]) * scale[j] * dcap;
         g[u] = vok ? v : 0.0f;
       } else {
         // z already is the capped draft logit in base-2 units (-inf past the vocabulary)
         // selects, not branches: the lanes of a wave disagree on tv > 0
         const float tv = t[u];
-        const float e = fast_exp2(z - tile_max[j]);
+        const float e = exp2_of<E::kPrecise>(z - tile_max[j]);
         tile_sum[j] += vok ? e : 0.0f;
         const bool use = vok && tv > 0.0f;
-        const float term = tv * ((fast_log2(tv) - z) * TLCE_LN2) - tv;
+        const float term = tv * ((log2_of<E::kPrecise>(tv) - z) * TLCE_LN2) - tv;
         partial[j] += use ? term : 0.0f;
         tsum[j] += use ? tv : 0.0f;
       }
@@ -739,15 +741,24 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
         // the next quarter of the tile is being processed
         __syncthreads();
         constexpr int kPieces = E::kTokensPerIndex * 32;
+        constexpr int kMine = kPieces / E::kThreads;
+        uint4 val[kMine];   // LDS reads first, then the stores: one wait per quarter
 #pragma unroll
-        for (int it = 0; it < kPieces / E::kThreads; ++it) {
+        for (int it = 0; it < kMine; ++it) {
           const int c = it * E::kThreads + threadIdx.x;
           const int tok = E::token_of_index(j, c >> 5);
           const int ch = c & 31;
-          stream_store16(
-              panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 8,
-              *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)));
+          val[it] = *reinterpret_cast<const uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16));
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int it = 0; it < kMine; ++it) {
+          const int c = it * E::kThreads + threadIdx.x;
+          const int tok = E::token_of_index(j, c >> 5);
+          const int ch = c & 31;
+          stream_store16(panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow + ch * 8, val[it]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   } else {
@@ -766,25 +777,20 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
     }
   }
   if (!grad) {
-#pragma unroll
-    for (int j = 0; j < E::kCols; ++j) {
-      const float total = eng.reduce_over_rows_in_wave(partial[j]);
-      const float total_t = eng.reduce_over_rows_in_wave(tsum[j]);
-      if (eng.row_leader() && live[j]) {
-        atomicAdd(p.losses + tt * E::kTile + eng.col(j), total);
-        atomicAdd(p.tsum + tt * E::kTile + eng.col(j), total_t);
-      }
-    }
-    // merge the kShare threads that hold the same token column and publish the
-    // tile's partial, as the forward kernel does per vocabulary split
+    // merge the kShare threads that hold the same token column, in a fixed order,
+    // and publish the tile's partials, as the forward kernel does per vocabulary split
     __syncthreads();
     float* sh_max = reinterpret_cast<float*>(smem);
     float* sh_sum = sh_max + E::kShare * E::kTile;
+    float* sh_loss = sh_sum + E::kShare * E::kTile;
+    float* sh_tsum = sh_loss + E::kShare * E::kTile;
     const int slot = eng.share_slot();
 #pragma unroll
     for (int j = 0; j < E::kCols; ++j) {
       sh_max[slot * E::kTile + eng.col(j)] = tile_max[j];
       sh_sum[slot * E::kTile + eng.col(j)] = tile_sum[j];
+      sh_loss[slot * E::kTile + eng.col(j)] = partial[j];
+      sh_tsum[slot * E::kTile + eng.col(j)] = tsum[j];
     }
     __syncthreads();
     const int tile_index = vbase / E::kTile;
@@ -792,15 +798,20 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
       float mx = -INFINITY;
 #pragma unroll
       for (int sl = 0; sl < E::kShare; ++sl) mx = fmaxf(mx, sh_max[sl * E::kTile + c]);
-      float sum = 0.0f;
-      if (mx > -INFINITY) {
+      float sum = 0.0f, loss = 0.0f, mass = 0.0f;
 #pragma unroll
-        for (int sl = 0; sl < E::kShare; ++sl)
-          sum += sh_sum[sl * E::kTile + c] * fast_exp2(sh_max[sl * E::kTile + c] - mx);
+      for (int sl = 0; sl < E::kShare; ++sl) {
+        if (mx > -INFINITY)
+          sum += sh_sum[sl * E::kTile + c] *
+                 exp2_of<E::kPrecise>(sh_max[sl * E::kTile + c] - mx);
+        loss += sh_loss[sl * E::kTile + c];
+        mass += sh_tsum[sl * E::kTile + c];
       }
       const int64_t o = (int64_t)tile_index * p.part_ld + tt * E::kTile + c;
       p.part_max[o] = mx;
       p.part_sum[o] = sum;
+      p.loss_part[o] = loss;
+      p.tsum_part[o] = mass;
     }
   }
 }
@@ -844,7 +855,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_logits_panel_kernel(LogitsPan
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const float raw = E::get(acc, j, i4 + u);
-      const float val = kSoftcap ? p.softcap * fast_tanh(raw * inv_cap) : raw * p.logit_scale;
+      const float val = kSoftcap ? p.softcap * tanh_of<E::kPrecise>(raw * inv_cap) : raw * p.logit_scale;
       z[u] = (vbase + eng.row(i4 + u) < p.v) ? val : -INFINITY;
     }
     return make_float4(z[0], z[1], z[2], z[3]);
@@ -1049,6 +1060,139 @@ __device__ __forceinline__ int dynamic_k_splits(int n_ttiles, int n_htiles, int 
 }
 enum { kRowsFollow = 1, kKFollows = 2 };
 
+// Output stage of the contraction kernels for the direct engine: the accumulator
+// tile leaves through LDS (free after the main loop) in whole output rows, so that
+// one wave instruction touches 1 KiB (float32) or 512 B (2-byte types) of one row
+// instead of 64 pieces 16 or 8 bytes long in 64 different rows.
+//
+// float32 output (the grad_hidden slabs): the tile is 256 KiB, twice the LDS, and
+// goes in two halves, the rows of two owned column indices each (128 rows of
+// 1 KiB, 16-byte chunk c of staged row s in slot c ^ (s & 63)).  kAdd: the slab's
+// old values of a half are requested before its rows are staged, so their
+// latency passes under the staging.
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+
+template <class E, bool kAdd>
+__device__ __forceinline__ void store_tile_f32_by_rows(const E& eng, const typename E::Acc& acc,
+                                                       char* smem, float* c, int64_t ldc,
+                                                       int row0, int col0, int c_rows,
+                                                       int c_cols) {
+  constexpr int kPerIndex = E::kTokensPerIndex;                 // rows per owned index
+  constexpr int kMine = (2 * kPerIndex * 64) / E::kThreads;     // 16-byte pieces per thread
+  constexpr int kBatch = 8;
+  constexpr int kBatches = kMine / kBatch;
+  constexpr int kAhead = 2;                                     // batches of old values in flight
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    if (half) __syncthreads();                                  // the first half has been read out
+    // piece `it` of this thread: output row / column and whether it exists
+    auto place = [&](int it, int* s_row, int* ch, int* out_row, int* out_col) -> bool {
+      const int idx = it * E::kThreads + threadIdx.x;
+      *s_row = idx >> 6;
+      *ch = idx & 63;
+      *out_row = row0 + E::token_of_index(2 * half + *s_row / kPerIndex, *s_row % kPerIndex);
+      *out_col = col0 + *ch * 4;
+      return *out_row < c_rows && *out_col < c_cols;
+    };
+    f32x4_t old[kAdd ? kBatches : 1][kAdd ? kBatch : 1];
+    auto request_old = [&](int batch) {
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        int s_row, ch, out_row, out_col;
+        const bool ok = place(batch * kBatch + u, &s_row, &ch, &out_row, &out_col);
+        const f32x4_t zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        old[batch][u] =
+            ok ? *reinterpret_cast<const f32x4_t*>(c + (int64_t)out_row * ldc + out_col) : zero;
+      }
+    };
+    if (kAdd) {
+#pragma unroll
+      for (int b = 0; b < kAhead; ++b) request_old(b);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; ++jj) {
+      const int j = 2 * half + jj;
+      const int t = (eng.col(j) / (E::kTile / 2)) * 32 + (eng.col(j) & 31);
+      const int s_row = jj * kPerIndex + t;
+#pragma unroll
+      for (int i4 = 0; i4 < E::kRows; i4 += 4) {
+        const int chunk = eng.row(i4) >> 2;
+        const f32x4_t quad = {E::get(acc, j, i4), E::get(acc, j, i4 + 1), E::get(acc, j, i4 + 2),
+                              E::get(acc, j, i4 + 3)};
+        *reinterpret_cast<f32x4_t*>(smem + s_row * 1024 + ((chunk ^ (s_row & 63)) * 16)) = quad;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < kBatches; ++b) {
+      if (kAdd && b + kAhead < kBatches) request_old(b + kAhead);
+      f32x4_t val[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int idx = (b * kBatch + u) * E::kThreads + threadIdx.x;
+        const int s_row = idx >> 6, ch = idx & 63;
+        val[u] = *reinterpret_cast<const f32x4_t*>(smem + s_row * 1024 +
+                                                   ((ch ^ (s_row & 63)) * 16));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        int s_row, ch, out_row, out_col;
+        const bool ok = place(b * kBatch + u, &s_row, &ch, &out_row, &out_col);
+        f32x4_t v = val[u];
+        if (kAdd) v += old[b][u];
+        if (ok) *reinterpret_cast<f32x4_t*>(c + (int64_t)out_row * ldc + out_col) = v;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+}
+
+// 2-byte output (the rows of grad_weight): the whole 128 KiB tile is staged as
+// [row][column] (512-byte rows, 16-byte chunk c of row r in slot c ^ (r & 31)).
+template <class E>
+__device__ __forceinline__ void store_tile_t_by_rows(const E& eng, const typename E::Acc& acc,
+                                                     char* smem, typename E::T* c, int64_t ldc,
+                                                     int row0, int col0, int c_rows, int c_cols) {
+  using T = typename E::T;
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    const int r = eng.col(j);
+#pragma unroll
+    for (int i4 = 0; i4 < E::kRows; i4 += 4) {
+      const int vq = eng.row(i4) >> 2;
+      T* dst = reinterpret_cast<T*>(smem + r * 512 + (((vq >> 1) ^ (r & 31)) * 16) + (vq & 1) * 8);
+      store4<T>(dst, E::get(acc, j, i4), E::get(acc, j, i4 + 1), E::get(acc, j, i4 + 2),
+                E::get(acc, j, i4 + 3));
+    }
+  }
+  __syncthreads();
+  constexpr int kMine = (E::kTile * 32) / E::kThreads;   // 16-byte pieces per thread
+  constexpr int kBatch = 8;
+#pragma unroll
+  for (int b0 = 0; b0 < kMine; b0 += kBatch) {
+    u32x4_t val[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int idx = (b0 + u) * E::kThreads + threadIdx.x;
+      const int r = idx >> 5, ch = idx & 31;
+      val[u] = *reinterpret_cast<const u32x4_t*>(smem + r * 512 + ((ch ^ (r & 31)) * 16));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int idx = (b0 + u) * E::kThreads + threadIdx.x;
+      const int r = idx >> 5, ch = idx & 31;
+      const int out_row = row0 + r, out_col = col0 + ch * 8;
+      if (out_row < c_rows && out_col < c_cols)
+        *reinterpret_cast<u32x4_t*>(c + (int64_t)out_row * ldc + out_col) = val[u];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
+
 template <class E, bool kAKMajor, bool kBKMajor>
 __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
   extern __shared__ __align__(16) char smem[];
@@ -1091,41 +1235,59 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
                      acc, smem);
   }
 
-  // runs of 4 can be moved as one vector when every row start keeps them aligned
-  const bool vec_ok = (p.ldc % 4 == 0) && (p.c_cols % 4 == 0) &&
-                      (reinterpret_cast<uintptr_t>(p.c) % 16 == 0);
+  if constexpr (E::kHasKMajor && sizeof(T) == 2 && E::kCols == 4) {
+    // The direct engine is only planned for hidden sizes that are multiples of 64
+    // and its outputs (workspace slabs, rows of grad_weight) are 16-byte aligned:
+    // whole output rows leave through LDS (the main loop has ended on a barrier).
+    const int row0 = tj * E::kTile, col0 = ti * E::kTile;
+    if (p.mode == kStoreT) {
+      store_tile_t_by_rows<E>(eng, acc, smem, static_cast<T*>(p.c), p.ldc, row0, col0, p.c_rows,
+                              p.c_cols);
+    } else if (p.mode == kStoreF32) {
+      store_tile_f32_by_rows<E, false>(eng, acc, smem, static_cast<float*>(p.c), p.ldc, row0,
+                                       col0, p.c_rows, p.c_cols);
+    } else {
+      store_tile_f32_by_rows<E, true>(eng, acc, smem, static_cast<float*>(p.c), p.ldc, row0,
+                                      col0, p.c_rows, p.c_cols);
+    }
+  } else {
+    // runs of 4 can be moved as one vector when every row start keeps them aligned
+    const bool vec_ok = (p.ldc % 4 == 0) && (p.c_cols % 4 == 0) &&
+                        (reinterpret_cast<uintptr_t>(p.c) % 16 == 0);
 #pragma unroll
-  for (int j = 0; j < E::kCols; ++j) {
-    const int out_row = tj * E::kTile + eng.col(j);
-    if (out_row >= p.c_rows) continue;
+    for (int j = 0; j < E::kCols; ++j) {
+      const int out_row = tj * E::kTile + eng.col(j);
+      if (out_row >= p.c_rows) continue;
 #pragma unroll
-    for (int i = 0; i < E::kRows; i += 4) {
-      const int out_col = ti * E::kTile + eng.row(i);
-      if (out_col >= p.c_cols) continue;
-      const int64_t o = (int64_t)out_row * p.ldc + out_col;
-      const float v0 = E::get(acc, j, i), v1 = E::get(acc, j, i + 1);
-      const float v2 = E::get(acc, j, i + 2), v3 = E::get(acc, j, i + 3);
-      if (vec_ok) {
-        if (p.mode == kStoreT) {
-          store4<T>(static_cast<T*>(p.c) + o, v0, v1, v2, v3);
-        } else if (p.mode == kStoreF32) {
-          *reinterpret_cast<float4*>(static_cast<float*>(p.c) + o) = make_float4(v0, v1, v2, v3);
-        } else {
-          float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.c) + o);
-          float4 old = *dst;
-          *dst = make_float4(old.x + v0, old.y + v1, old.z + v2, old.w + v3);
-        }
-      } else {
-        const float vals[4] = {v0, v1, v2, v3};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (out_col + e >= p.c_cols) continue;
+      for (int i = 0; i < E::kRows; i += 4) {
+        const int out_col = ti * E::kTile + eng.row(i);
+        if (out_col >= p.c_cols) continue;
+        const int64_t o = (int64_t)out_row * p.ldc + out_col;
+        const float v0 = E::get(acc, j, i), v1 = E::get(acc, j, i + 1);
+        const float v2 = E::get(acc, j, i + 2), v3 = E::get(acc, j, i + 3);
+        if (vec_ok) {
           if (p.mode == kStoreT) {
-            static_cast<T*>(p.c)[o + e] = from_float<T>(vals[e]);
+            store4<T>(static_cast<T*>(p.c) + o, v0, v1, v2, v3);
           } else if (p.mode == kStoreF32) {
-            static_cast<float*>(p.c)[o + e] = vals[e];
+            *reinterpret_cast<float4*>(static_cast<float*>(p.c) + o) =
+                make_float4(v0, v1, v2, v3);
           } else {
-            static_cast<float*>(p.c)[o + e] += vals[e];
+            float4* dst = reinterpret_cast<float4*>(static_cast<float*>(p.c) + o);
+            float4 old = *dst;
+            *dst = make_float4(old.x + v0, old.y + v1, old.z + v2, old.w + v3);
+          }
+        } else {
+          const float vals[4] = {v0, v1, v2, v3};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (out_col + e >= p.c_cols) continue;
+            if (p.mode == kStoreT) {
+              static_cast<T*>(p.c)[o + e] = from_float<T>(vals[e]);
+            } else if (p.mode == kStoreF32) {
+              static_cast<float*>(p.c)[o + e] = vals[e];
+            } else {
+              static_cast<float*>(p.c)[o + e] += vals[e];
+            }
           }
         }
       }

@@ -43,9 +43,10 @@ int launch_token_scale(const ScaleArgs& sa, hipStream_t stream) {
   return 0;
 }
 
-int launch_kl_finish(float* losses, const float* tsum, const float* lse, int64_t m,
-                     hipStream_t stream) {
-  lce_kl_finish_kernel<<<(int)ceil_div(m, 256), 256, 0, stream>>>(losses, tsum, lse, (int)m);
+int launch_kl_finish(float* losses, const float* loss_part, const float* tsum_part, int n_tiles,
+                     int64_t part_ld, const float* lse, int64_t m, hipStream_t stream) {
+  lce_kl_finish_kernel<<<(int)ceil_div(m, 256), 256, 0, stream>>>(losses, loss_part, tsum_part,
+                                                                  n_tiles, part_ld, lse, (int)m);
   TLCE_LAUNCH_CHECK();
   return 0;
 }

@@ -83,11 +83,20 @@ __global__ __launch_bounds__(256) void lce_segment_weighted_sum_kernel(
   if (threadIdx.x == 0) out[blockIdx.x] = part[0];
 }
 
-// losses[r] = losses[r] + tsum[r] * lse_draft[r] + 1  (see lce_kl_panel_kernel)
-__global__ __launch_bounds__(256) void lce_kl_finish_kernel(float* losses, const float* tsum,
-                                                            const float* lse, int m) {
+// losses[r] = sum_t loss_part[t][r] + (sum_t tsum_part[t][r]) * lse_draft[r] + 1, the
+// vocabulary tiles t added in ascending order (see lce_kl_panel_kernel).
+__global__ __launch_bounds__(256) void lce_kl_finish_kernel(float* losses, const float* loss_part,
+                                                            const float* tsum_part, int n_tiles,
+                                                            int64_t part_ld, const float* lse,
+                                                            int m) {
   const int r = blockIdx.x * 256 + threadIdx.x;
-  if (r < m) losses[r] = losses[r] + tsum[r] * lse[r] + 1.0f;
+  if (r >= m) return;
+  float loss = 0.0f, mass = 0.0f;
+  for (int t = 0; t < n_tiles; ++t) {
+    loss += loss_part[(int64_t)t * part_ld + r];
+    mass += tsum_part[(int64_t)t * part_ld + r];
+  }
+  losses[r] = loss + mass * lse[r] + 1.0f;
 }
 
 // Ordering of (value, id) pairs: larger value first, then smaller id.
