@@ -192,6 +192,40 @@ int tlce_backward(const void* hidden, const void* weight, const float* bias,
                   int64_t panel_bytes,
                   void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- head stored [h, v] ("dim first") -------------------------------------
+ * The reference's extension takes `weight_dim_first` (fused_linear_ce.cpp:104,121)
+ * and hands the layout to its GEMMs as a transpose flag.  Here the same: with
+ * the entry points below `weight` and `grad_weight` are [h, v] row-major and
+ * are read and written in place (the head as a K-major MFMA operand of the two
+ * logits contractions, its columns as K-contiguous rows of the grad_hidden
+ * contraction, grad_weight produced with the operand roles swapped); no
+ * transposed copy of either matrix is made.  Everything else is as for
+ * tlce_forward / tlce_backward, same workspaces.
+ * Supported where tlce_dim_first_supported(h, v, dtype) returns 1: 16-bit
+ * inputs with h and v multiples of 64.  Other shapes are refused with an
+ * error; their callers re-lay the head to [v, h] once and use tlce_forward /
+ * tlce_backward. */
+int tlce_dim_first_supported(int64_t h, int64_t v, int dtype);
+
+int tlce_forward_dim_first(const void* hidden, const void* weight, const float* bias,
+                           const int64_t* labels, const int64_t* row_idx,
+                           int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                           int64_t ignore_index, int64_t exclude_index,
+                           float logit_softcap,
+                           float* losses, float* lse, float* valid_count,
+                           void* workspace, int64_t workspace_bytes, void* stream);
+
+int tlce_backward_dim_first(const void* hidden, const void* weight, const float* bias,
+                            const int64_t* labels, const int64_t* row_idx,
+                            const float* lse, const float* valid_count,
+                            const float* grad_output,
+                            int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+                            int reduction_code, int64_t ignore_index,
+                            int64_t exclude_index, float logit_softcap,
+                            void* grad_hidden, void* grad_weight, float* grad_bias,
+                            int64_t panel_bytes,
+                            void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- masked-token loss ---------------------------------------------------
  * The arithmetic the reference's loss method wraps around the operator
  * (distributed_block_diffusion_loss, nemotron/model.py:2084-2151;

@@ -119,3 +119,20 @@ def test_masked_loss_entry_points_validate_before_touching_a_gpu():
                                    None, None)
     assert rc != 0 and "weights" in _lib.last_error()
     assert lib.tlce_masked_loss_forward_workspace_bytes(-1, 8, 8, _lib.DTYPE_BF16, 0) == -1
+
+
+def test_dim_first_entry_points_validate_before_touching_a_gpu():
+    lib = _lib.library()
+    assert lib.tlce_dim_first_supported(4096, 151936, _lib.DTYPE_BF16) == 1
+    assert lib.tlce_dim_first_supported(4096, 151936, _lib.DTYPE_F32) == 0     # float32 inputs
+    assert lib.tlce_dim_first_supported(4096, 151937, _lib.DTYPE_BF16) == 0    # partial K slab
+    assert lib.tlce_dim_first_supported(72, 1024, _lib.DTYPE_BF16) == 0        # staged engine
+    assert lib.tlce_dim_first_supported(0, 64, _lib.DTYPE_BF16) == 0
+    fake = 4096          # aligned, never dereferenced: validation fails first
+    rc = lib.tlce_forward_dim_first(fake, fake, None, fake, None, 8, 8, 64, 100, _lib.DTYPE_BF16,
+                                    -100, -1, 0.0, fake, fake, fake, fake, 1 << 20, None)
+    assert rc != 0 and "read in place only" in _lib.last_error()
+    rc = lib.tlce_backward_dim_first(fake, fake, None, fake, None, fake, fake, fake, 8, 8, 64, 100,
+                                     _lib.DTYPE_F32, _lib.REDUCTION_SUM, -100, -1, 0.0, fake,
+                                     fake, None, 0, fake, 1 << 30, None)
+    assert rc != 0 and "read in place only" in _lib.last_error()

@@ -313,6 +313,80 @@ def test_dim_first_and_non_contiguous(gpu_device):
     assert torch.equal(auto, loss.detach())
 
 
+@pytest.mark.parametrize("m,h,v,opts", [
+    (300, 128, 1536, {}),
+    (1000, 256, 4160, dict(bias=True, logit_softcap=5.0, exclude_index=7)),   # v % 256 != 0
+    (130, 64, 640, dict(reduction="none", frozen=True)),
+    (700, 192, 2048, dict(reduction="sum", panel_tiles=3, ignored=0.0)),     # several panels
+])
+def test_dim_first_head_is_read_in_place(gpu_device, m, h, v, opts):
+    """A [H, V] head with 16-bit inputs and H, V multiples of 64 goes to the
+    library as it is stored (tlce_*_dim_first, the reference's `weight_dim_first`
+    flag, fused_linear_ce.cpp:104,121): same results as the oracle's dim-first
+    branch, grad_weight comes back [H, V], and no [V, H] copy of the head is
+    allocated on the way."""
+    opts = dict(opts)
+    say("dim-first in place", m, h, v, opts)
+    torch.manual_seed(m + v)
+    hidden = torch.randn(m, h).bfloat16()
+    weight = (torch.randn(h, v) * 0.2).bfloat16()               # [H, V]
+    bias = torch.randn(v).bfloat16() if opts.pop("bias", False) else None
+    labels = torch.randint(0, v, (m,))
+    exclude = opts.get("exclude_index")
+    if exclude is not None:
+        labels[labels == exclude] = exclude + 1
+    labels[torch.rand(m) < opts.pop("ignored", 0.25)] = -100
+    frozen = opts.pop("frozen", False)
+    panel_tiles = opts.pop("panel_tiles", 0)
+    reduction = opts.pop("reduction", "mean")
+    assert native.dim_first_in_place(weight.to(gpu_device), True)
+    assert not native.dim_first_in_place(weight.to(gpu_device), False)
+    mp = -(-m // 256) * 256
+    with native.panel_budget(mp * 256 * 2 * panel_tiles):
+        grad_out = torch.randn(m) if reduction == "none" else None
+        loss, dh, dw, db = check_against_oracle(
+            gpu_device, hidden, weight, labels, bias=bias, reduction=reduction, frozen=frozen,
+            weight_layout="dim_first", grad_out=grad_out, **opts)
+    if not frozen:
+        assert dw.shape == (h, v)
+    # the same head laid out [V, H]: same tiles in the same order; only the label's logit is
+    # summed in another order (a strided column instead of a row)
+    vf = run_api(gpu_device, hidden, weight.t().contiguous(), labels, bias=bias, frozen=True,
+                 grad_out=grad_out, reduction=reduction, dtype=torch.bfloat16,
+                 weight_layout="vocab_first", **opts)
+    torch.testing.assert_close(loss, vf[0], rtol=1e-5, atol=1e-5)
+    # no transposed copy: the forward's peak allocation stays far below one more head
+    dev = gpu_device
+    x, w, y = hidden.to(dev), weight.to(dev), labels.to(dev)
+    big_v = 64 * 1024
+    w_big = (torch.randn(h, big_v, device=dev) * 0.2).bfloat16()
+    y_big = torch.randint(0, big_v, (m,), device=dev)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats(dev)
+    before = torch.cuda.memory_allocated(dev)
+    with torch.no_grad():
+        out = tiled_linear_cross_entropy(x, w_big, y_big, dtype=torch.bfloat16,
+                                         weight_layout="dim_first")
+    torch.cuda.synchronize()
+    extra = torch.cuda.max_memory_allocated(dev) - before
+    say("peak extra bytes", extra, "head bytes", w_big.numel() * 2)
+    assert bool(torch.isfinite(out)) and extra < w_big.numel() * 2 // 2
+
+
+def test_dim_first_fallback_shapes_still_use_a_copy(gpu_device):
+    """Shapes the in-place path does not take (float32, V not a multiple of 64) are
+    re-laid once and give the oracle's results."""
+    say("dim-first fallback")
+    torch.manual_seed(21)
+    for dtype, h, v in ((torch.float32, 64, 640), (torch.bfloat16, 128, 1000)):
+        weight = (torch.randn(h, v) * 0.2).to(dtype)
+        assert not native.dim_first_in_place(weight.to(gpu_device), True)
+        hidden = torch.randn(90, h).to(dtype)
+        labels = torch.randint(0, v, (90,))
+        tol = dict(loss_rtol=1e-4, grad_rel=1e-4) if dtype == torch.float32 else {}
+        check_against_oracle(gpu_device, hidden, weight, labels, weight_layout="dim_first", **tol)
+
+
 def test_softcap_with_bias_and_exclusion(gpu_device):
     say("softcap + bias + exclude")
     torch.manual_seed(12)

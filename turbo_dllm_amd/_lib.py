@@ -81,6 +81,28 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_dim_first_supported": (c_int, [c_int64, c_int64, c_int]),
+    "tlce_forward_dim_first": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden weight bias labels row_idx
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m n_out h v dtype
+            c_int64, c_int64, c_float,                          # ignore exclude softcap
+            c_void_p, c_void_p, c_void_p,                       # losses lse valid_count
+            c_void_p, c_int64, c_void_p,                        # workspace bytes stream
+        ],
+    ),
+    "tlce_backward_dim_first": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden weight bias labels row_idx
+            c_void_p, c_void_p, c_void_p,                       # lse valid_count grad_output
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m n_out h v dtype
+            c_int, c_int64, c_int64, c_float,                   # reduction ignore exclude softcap
+            c_void_p, c_void_p, c_void_p,                       # grad_hidden grad_weight grad_bias
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
     "tlce_masked_loss_forward_workspace_bytes": (
         c_int64, [c_int64, c_int64, c_int64, c_int, c_int]
     ),

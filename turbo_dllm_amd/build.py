@@ -32,7 +32,8 @@ _WHOLE_ENGINES = {"staged_bf16": "MfmaEngine<__bf16>", "staged_f16": "MfmaEngine
                   "generic_f32": "SimtEngine<float>", "generic_bf16": "SimtEngine<__bf16>",
                   "generic_f16": "SimtEngine<_Float16>"}
 _PARTS = {2: "grad_logits", 7: "grad_logits_cap", 8: "grad_logits_bias", 9: "grad_logits_cap_bias",
-          1: "forward", 3: "gemm", 4: "kl", 5: "logits", 6: "sequences"}
+          1: "forward", 3: "gemm", 4: "kl", 5: "logits", 6: "sequences",
+          10: "forward_dim_first", 11: "grad_logits_dim_first"}
 UNITS = (
     [(f"engine_{tag}_{name}", "tlce_engine_unit.hip",
       (f"-DTLCE_UNIT_ENGINE={engine}", f"-DTLCE_UNIT_PART={part}"))

@@ -380,9 +380,23 @@ def scatter_rows(src: torch.Tensor, row_idx: torch.Tensor, n_rows: int) -> torch
 
 
 # -------------------------------------------------------------------- forward --
-def _vocab_first(weight: torch.Tensor, weight_dim_first: bool) -> torch.Tensor:
-    # The kernels read the head as [V, H]; a [H, V] head is re-laid once here.
-    return weight.t().contiguous() if weight_dim_first else _dense(weight)
+def dim_first_in_place(weight: torch.Tensor, weight_dim_first: bool) -> bool:
+    """True when a ``[H, V]`` head can be handed to the library as it is stored
+    (``tlce_*_dim_first``: 16-bit dtypes, H and V multiples of 64)."""
+    if not weight_dim_first or weight.dim() != 2 or weight.dtype not in _DTYPE_CODES:
+        return False
+    h, v = weight.shape
+    return bool(_lib.library().tlce_dim_first_supported(int(h), int(v),
+                                                        _DTYPE_CODES[weight.dtype]))
+
+
+def _head_operand(weight: torch.Tensor, weight_dim_first: bool) -> tuple[torch.Tensor, bool]:
+    """The head as the library takes it and whether that is the [H, V] form.  A
+    [H, V] head is read in place where the kernels can (see
+    ``dim_first_in_place``); otherwise it is re-laid to [V, H] once."""
+    if dim_first_in_place(weight, weight_dim_first):
+        return _dense(weight), True
+    return (weight.t().contiguous() if weight_dim_first else _dense(weight)), False
 
 
 def forward(
@@ -416,11 +430,11 @@ def forward(
     if weight.dtype != hidden.dtype:
         raise RuntimeError("native linear CE expects hidden and weight of one dtype")
     hidden = _dense(hidden)
-    weight = _vocab_first(weight, weight_dim_first)
+    weight, in_place = _head_operand(weight, weight_dim_first)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
-    v = weight.shape[0]
-    if weight.shape[1] != h or labels.numel() != m:
+    v = weight.shape[1] if in_place else weight.shape[0]
+    if weight.shape[0 if in_place else 1] != h or labels.numel() != m:
         raise RuntimeError("native linear CE shape mismatch")
     n_out = m if n_out is None else int(n_out)
     bias32 = None if bias is None else bias.to(torch.float32).contiguous()
@@ -433,15 +447,16 @@ def forward(
         lse = torch.empty(m, dtype=torch.float32, device=device)
         valid_count = torch.empty(1, dtype=torch.float32, device=device)
         ws = _workspace(lib.tlce_forward_workspace_bytes(m, h, v, code), device)
+        entry = lib.tlce_forward_dim_first if in_place else lib.tlce_forward
         _lib.check(
-            lib.tlce_forward(
+            entry(
                 _ptr(hidden), _ptr(weight), _ptr(bias32), _ptr(labels), _ptr(row_idx),
                 m, n_out, h, v, code,
                 int(ignore_index), int(exclude_index), float(logit_softcap),
                 _ptr(losses), _ptr(lse), valid_count.data_ptr(),
                 ws.data_ptr(), ws.numel(), _stream(device),
             ),
-            "tlce_forward",
+            "tlce_forward_dim_first" if in_place else "tlce_forward",
         )
     return losses, lse, valid_count
 
@@ -454,10 +469,10 @@ def _backward(
 ):
     device = _require_device(hidden, weight, bias, labels, lse, valid_count, grad_output, row_idx)
     hidden = _dense(hidden)
-    weight_vf = _vocab_first(weight, weight_dim_first)
+    weight_vf, in_place = _head_operand(weight, weight_dim_first)
     labels = labels.reshape(-1).to(torch.long).contiguous()
     m, h = hidden.shape
-    v = weight_vf.shape[0]
+    v = weight_vf.shape[1] if in_place else weight_vf.shape[0]
     n_out = m if n_out is None else int(n_out)
     code = _dtype_code(hidden)
     reduction_code = _reduction_code(reduction)
@@ -471,9 +486,10 @@ def _backward(
     lib = _lib.library()
     with torch.cuda.device(device):
         grad_hidden = torch.empty((n_out, h), dtype=hidden.dtype, device=device)
-        grad_weight = (
-            torch.empty((v, h), dtype=weight.dtype, device=device) if compute_weight_grad else None
-        )
+        grad_weight = None
+        if compute_weight_grad:      # in the layout the library writes: [H, V] in place, else [V, H]
+            grad_weight = torch.empty((h, v) if in_place else (v, h), dtype=weight.dtype,
+                                      device=device)
         grad_bias32 = (
             torch.empty(v, dtype=torch.float32, device=device) if bias is not None else None
         )
@@ -483,8 +499,9 @@ def _backward(
             ),
             device,
         )
+        entry = lib.tlce_backward_dim_first if in_place else lib.tlce_backward
         _lib.check(
-            lib.tlce_backward(
+            entry(
                 _ptr(hidden), _ptr(weight_vf), _ptr(bias32), _ptr(labels), _ptr(row_idx),
                 _ptr(lse), valid_count.data_ptr(), _ptr(grad_output),
                 m, n_out, h, v, code,
@@ -492,11 +509,11 @@ def _backward(
                 _ptr(grad_hidden), _ptr(grad_weight), _ptr(grad_bias32),
                 get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
-            "tlce_backward",
+            "tlce_backward_dim_first" if in_place else "tlce_backward",
         )
     if grad_weight is None:
         grad_weight = torch.empty(0, dtype=weight.dtype, device=device)
-    elif weight_dim_first:
+    elif weight_dim_first and not in_place:
         grad_weight = grad_weight.t().contiguous()
     if grad_bias32 is None:
         grad_bias = torch.empty(0, dtype=torch.float32, device=device)

@@ -56,18 +56,26 @@ __host__ __device__ static inline int forward_vocab_splits(int n_ttiles, int n_v
   return s < n_vtiles ? s : n_vtiles;
 }
 
-// K splits of the grad_hidden contraction (`tiles` output tiles per panel): the
-// smallest factor up to max_split that fills at least 90 % of the last wave of
-// 256 workgroups and gives at least two waves (or max_split itself).  Every
-// split accumulates into a float32 slab of its own.  Shared by the host plan
-// and by the kernels when the row count is known only on the device.
-__host__ __device__ static inline int grad_hidden_k_splits(int64_t tiles, int max_split) {
+// K splits of the grad_hidden contraction: `tiles` output tiles per panel, each a
+// loop of `k_steps` K steps when unsplit; every split accumulates into a float32
+// slab of its own (`slab_elems` elements), summed by the final cast.  Picks the
+// count in [1, max_split] with the least estimated time, in units of one K step:
+//   rounds of 256 workgroups x (K steps per split + 8 for a tile's start and output)
+//   + splits x the time the final cast needs to read one more slab.
+// Ties go to fewer splits.  Integer arithmetic only: the host plan and the
+// kernels that re-plan for a row count known on the device must agree.
+__host__ __device__ static inline int grad_hidden_k_splits(int64_t tiles, int max_split,
+                                                           int64_t k_steps, int64_t slab_elems) {
+  const int64_t per_slab = (slab_elems >> 20) > 1 ? (slab_elems >> 20) : 1;
   int pick = 1;
+  int64_t best = -1;
   for (int ks = 1; ks <= max_split; ++ks) {
-    const int64_t workgroups = tiles * ks;
-    const int64_t rounds = (workgroups + 255) / 256;
-    pick = ks;
-    if (workgroups * 10 >= rounds * 256 * 9 && (workgroups >= 512 || ks == max_split)) break;
+    const int64_t rounds = (tiles * ks + 255) / 256;
+    const int64_t cost = rounds * ((k_steps + ks - 1) / ks + 8) + ks * per_slab;
+    if (best < 0 || cost < best) {
+      best = cost;
+      pick = ks;
+    }
   }
   return pick;
 }

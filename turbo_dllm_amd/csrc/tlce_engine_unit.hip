@@ -7,6 +7,8 @@
 //                        panels without soft cap and bias, gradient contractions,
 //                        KL panels, float32 logits panels), 7..9: the other
 //                        logit-gradient variants (soft cap, bias, both),
+//                        10, 11: the forward statistics and the logit-gradient
+//                        panels over a head stored [h, v],
 //                        6: the launch sequences over them.
 #include "tlce_host.h"
 
@@ -60,6 +62,16 @@ TLCE_LAUNCHERS_KL(extern template, UnitEngine)
 TLCE_LAUNCHERS_LOGITS(template, UnitEngine)
 #else
 TLCE_LAUNCHERS_LOGITS(extern template, UnitEngine)
+#endif
+#if TLCE_UNIT_PART == 10
+TLCE_LAUNCHERS_FORWARD_DIM_FIRST(template, UnitEngine)
+#else
+TLCE_LAUNCHERS_FORWARD_DIM_FIRST(extern template, UnitEngine)
+#endif
+#if TLCE_UNIT_PART == 11
+TLCE_LAUNCHERS_GRAD_LOGITS_DIM_FIRST(template, UnitEngine)
+#else
+TLCE_LAUNCHERS_GRAD_LOGITS_DIM_FIRST(extern template, UnitEngine)
 #endif
 #if TLCE_UNIT_PART == 6
 TLCE_ENGINE_ENTRY_POINTS(template, UnitEngine)

@@ -133,13 +133,14 @@ inline Plan make_plan(int64_t m, int64_t h, int64_t v, int dtype, bool weight_gr
   p.n_panels = (int)ceil_div(p.vp, p.vc);
   // grad_hidden: n_ttiles x n_htiles tiles per panel.  When that is not close
   // to whole waves of 256 workgroups, split K (each split accumulates into its
-  // own float32 slab, summed by the final cast) by the smallest factor that
-  // fills at least 90 % of the last wave.
+  // own float32 slab, summed by the final cast) by the factor with the least
+  // estimated time (grad_hidden_k_splits).
   p.dh_ksplit = 1;
   p.dh_max_ksplit = 1;
   if (p.engine) {
     p.dh_max_ksplit = (int)std::max<int64_t>(1, std::min<int64_t>(16, p.vc / p.bk / 8));
-    p.dh_ksplit = grad_hidden_k_splits((int64_t)p.n_ttiles * p.n_htiles, p.dh_max_ksplit);
+    p.dh_ksplit = grad_hidden_k_splits((int64_t)p.n_ttiles * p.n_htiles, p.dh_max_ksplit,
+                                       p.vc / p.bk, p.mp * h);
   }
   return p;
 }
@@ -154,7 +155,16 @@ struct RowOptions {
   const float* token_weights = nullptr;   // [m] float32, compacted order
   const int64_t* row_count = nullptr;     // device int64
   float* weighted_sum = nullptr;          // forward: [1] float32 out
+  // the head and its gradient are stored [h, v] (weight_dim_first of the reference's
+  // extension, fused_linear_ce.cpp:104,121) and are read / written in place
+  bool weight_dim_first = false;
 };
+
+// A [h, v] head is taken in place by the engine with K-major operand loaders, for
+// vocabularies made of whole 64-row K slabs.
+inline bool dim_first_in_place(int64_t h, int64_t v, int dtype) {
+  return engine_class(h, dtype) == 2 && (v % 64) == 0;
+}
 
 struct ForwardLayout {
   int64_t part_max, part_sum, weighted, total;
@@ -234,10 +244,11 @@ inline int validate_common(const void* hidden, const void* weight, int64_t m, in
 }
 
 // ---------------------------------------------------------------- launches --
-template <class E, bool kSoftcap, bool kBias>
+template <class E, bool kSoftcap, bool kBias, bool kWDimFirst = false>
 int launch_forward_variant(const Plan& p, const ForwardArgs& a, hipStream_t stream) {
   static LdsOptIn lds;
-  if (int rc = enable_large_lds(lce_forward_stats_kernel<E, kSoftcap, kBias>, E::kSmemBytes, lds))
+  if (int rc = enable_large_lds(lce_forward_stats_kernel<E, kSoftcap, kBias, kWDimFirst>,
+                                E::kSmemBytes, lds))
     return rc;
   // with a device-side row count: the most tiles any row count <= m can plan
   const int64_t tiles =
@@ -247,7 +258,8 @@ int launch_forward_variant(const Plan& p, const ForwardArgs& a, hipStream_t stre
                               std::max<int64_t>(kTargetWorkgroups, p.n_ttiles));
   const int grid = xcd_grid(tiles);
   ScopedTimer timer(kClassForwardStats, stream);
-  lce_forward_stats_kernel<E, kSoftcap, kBias><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  lce_forward_stats_kernel<E, kSoftcap, kBias, kWDimFirst>
+      <<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
@@ -261,18 +273,46 @@ int launch_forward(const Plan& p, const ForwardArgs& a, hipStream_t stream) {
   return launch_forward_variant<E, false, false>(p, a, stream);
 }
 
-template <class E, bool kSoftcap, bool kBias>
+// The same over a head stored [h, v] (engines with K-major operand loaders).
+template <class E>
+int launch_forward_dim_first(const Plan& p, const ForwardArgs& a, hipStream_t stream) {
+  if constexpr (E::kHasKMajor) {
+    const bool softcap = a.softcap > 0.0f, bias = a.bias != nullptr;
+    if (softcap && bias) return launch_forward_variant<E, true, true, true>(p, a, stream);
+    if (softcap) return launch_forward_variant<E, true, false, true>(p, a, stream);
+    if (bias) return launch_forward_variant<E, false, true, true>(p, a, stream);
+    return launch_forward_variant<E, false, false, true>(p, a, stream);
+  } else {
+    return fail("this engine cannot read a [h, v] head in place");
+  }
+}
+
+template <class E, bool kSoftcap, bool kBias, bool kWDimFirst = false>
 int launch_grad_logits_variant(const GradLogitsArgs& a, hipStream_t stream) {
   static LdsOptIn lds;
-  if (int rc = enable_large_lds(lce_grad_logits_panel_kernel<E, kSoftcap, kBias>, E::kSmemBytes,
-                                lds))
+  if (int rc = enable_large_lds(lce_grad_logits_panel_kernel<E, kSoftcap, kBias, kWDimFirst>,
+                                E::kSmemBytes, lds))
     return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
   ScopedTimer timer(kClassGradLogits, stream);
-  lce_grad_logits_panel_kernel<E, kSoftcap, kBias>
+  lce_grad_logits_panel_kernel<E, kSoftcap, kBias, kWDimFirst>
       <<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
+}
+
+// The logit-gradient panel over a head stored [h, v] (engines with K-major loaders).
+template <class E>
+int launch_grad_logits_dim_first(const GradLogitsArgs& a, hipStream_t stream) {
+  if constexpr (E::kHasKMajor) {
+    const bool softcap = a.softcap > 0.0f, bias = a.bias != nullptr;
+    if (softcap && bias) return launch_grad_logits_variant<E, true, true, true>(a, stream);
+    if (softcap) return launch_grad_logits_variant<E, true, false, true>(a, stream);
+    if (bias) return launch_grad_logits_variant<E, false, true, true>(a, stream);
+    return launch_grad_logits_variant<E, false, false, true>(a, stream);
+  } else {
+    return fail("this engine cannot read a [h, v] head in place");
+  }
 }
 
 template <class E>
@@ -349,7 +389,11 @@ int forward_impl(const Plan& p, const void* hidden, const void* weight, const fl
   fa.part_max = reinterpret_cast<float*>(ws + l.part_max);
   fa.part_sum = reinterpret_cast<float*>(ws + l.part_sum);
   fa.part_ld = (int)p.mp;
-  if (int rc = launch_forward<E>(p, fa, stream)) return rc;
+  if (opt.weight_dim_first) {
+    if (int rc = launch_forward_dim_first<E>(p, fa, stream)) return rc;
+  } else {
+    if (int rc = launch_forward<E>(p, fa, stream)) return rc;
+  }
 
   CombineArgs ca;
   ca.hidden = hidden; ca.weight = weight; ca.bias = bias; ca.labels = labels;
@@ -364,6 +408,7 @@ int forward_impl(const Plan& p, const void* hidden, const void* weight, const fl
   ca.target_logits = shard.target_logits;
   ca.logit_scale = opt.logit_scale; ca.token_weights = opt.token_weights;
   ca.n_vtiles = p.n_vtiles; ca.tile = p.tile; ca.m_dev = opt.row_count;
+  ca.weight_dim_first = opt.weight_dim_first;
   float* weighted = reinterpret_cast<float*>(ws + l.weighted);
   if (opt.weighted_sum != nullptr) {
     ca.weighted = weighted;
@@ -390,7 +435,7 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
                        int64_t h, int64_t v, int dtype, void* grad_hidden, void* grad_weight,
                        char* ws, hipStream_t stream, Producer&& produce,
                        const std::function<int(float*)>& before_cast = nullptr,
-                       const int64_t* m_dev = nullptr) {
+                       const int64_t* m_dev = nullptr, bool dim_first = false) {
   using T = typename E::T;
   const bool weight_grad = grad_weight != nullptr;
   float* acc32 = reinterpret_cast<float*>(ws + l.acc32);
@@ -437,6 +482,7 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     const int dh_launch_ksplit =
         m_dev == nullptr ? p.dh_ksplit : std::max(p.dh_ksplit, std::min(4, p.dh_max_ksplit));
     dh.slab_budget = (int64_t)p.dh_ksplit * p.mp * h;
+    dh.k_steps_plan = (int)(p.vc / p.bk);
     GemmArgs dw;
     dw.m_dev = m_dev; dw.m_role = kKFollows; dw.m_round = p.bk;
     dw.k_per_split = 0;
@@ -446,6 +492,27 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     dw.c_split_stride = 0;
     dw.mode = kStoreT;
     if constexpr (E::kHasKMajor) {
+      if (p.kmajor && dim_first) {
+        // The head is stored [h, v].  grad_hidden: A = its columns [v0, v0+K), which
+        // are K-contiguous rows of the stored matrix; B = G.
+        dh.a = weight_t + v0; dh.lda = v; dh.a_rows = (int)h;
+        dh.k = (int)round_up(rows_valid, 64);
+        if (int rc = launch_gemm<E, false, false>(dh, dh_launch_ksplit, kClassGradHidden, stream))
+          return rc;
+        if (weight_grad) {
+          // grad_weight [h, v]: the roles of the operands swap so that the hidden axis
+          // becomes the output's rows: A = G (its panel columns), B = hidden, both K-major
+          GemmArgs dwt = dw;
+          dwt.a = g; dwt.lda = p.vc; dwt.a_rows = (int)width;
+          dwt.b = hidden_k; dwt.ldb = h; dwt.b_rows = (int)h;
+          dwt.k = (int)m64;
+          dwt.ni = (int)(width / p.tile); dwt.nj = p.n_htiles;
+          dwt.c = static_cast<T*>(grad_weight) + v0; dwt.ldc = v;
+          dwt.c_rows = (int)h; dwt.c_cols = (int)rows_valid;
+          if (int rc = launch_gemm<E, true, true>(dwt, 1, kClassGradWeight, stream)) return rc;
+        }
+        continue;
+      }
       if (p.kmajor) {
         // grad_hidden: A = weight rows [v0, v0+K) as stored (K-major), B = G
         dh.a = weight_t + v0 * h; dh.lda = h; dh.a_rows = (int)h;
@@ -484,7 +551,8 @@ int panel_contractions(const Plan& p, const BackwardLayout& l, const void* hidde
     ScopedTimer timer(kClassOther, stream);
     lce_finalize_grad_hidden_kernel<T><<<(int)m, 256, 0, stream>>>(
         acc32, p.dh_ksplit, p.mp * h, row_idx, (int)m, (int)h, static_cast<T*>(grad_hidden),
-        m_dev, p.n_htiles, p.tile, std::max(p.dh_ksplit, std::min(4, p.dh_max_ksplit)));
+        m_dev, p.n_htiles, p.tile, std::max(p.dh_ksplit, std::min(4, p.dh_max_ksplit)),
+        (int)(p.vc / p.bk));
   }
   TLCE_LAUNCH_CHECK();
   return 0;
@@ -528,10 +596,12 @@ int backward_impl(const Plan& p, const void* hidden, const void* weight, const f
     ga.n_ttiles = p.n_ttiles; ga.n_ptiles = (int)(width / p.tile);
     ga.g = g; ga.ldg = p.vc; ga.gt = gt; ga.ldgt = p.mp;
     ga.grad_bias = (bias != nullptr) ? grad_bias : nullptr;
+    if (opt.weight_dim_first) return launch_grad_logits_dim_first<E>(ga, stream);
     return launch_grad_logits<E>(ga, stream);
   };
   return panel_contractions<E>(p, l, hidden, weight, row_idx, m, n_out, h, v, dtype, grad_hidden,
-                               grad_weight, ws, stream, produce, nullptr, opt.row_count);
+                               grad_weight, ws, stream, produce, nullptr, opt.row_count,
+                               opt.weight_dim_first);
 }
 
 // -------------------------------------------------------------- frozen KL ----
@@ -862,6 +932,10 @@ int soft_embedding_impl(const Plan& fp, const Plan& bp, const SoftEmbeddingLayou
   X int launch_forward<E>(const Plan&, const ForwardArgs&, hipStream_t);
 #define TLCE_LAUNCHERS_GRAD_LOGITS(X, E, kSoftcap, kBias) \
   X int launch_grad_logits_variant<E, kSoftcap, kBias>(const GradLogitsArgs&, hipStream_t);
+#define TLCE_LAUNCHERS_FORWARD_DIM_FIRST(X, E) \
+  X int launch_forward_dim_first<E>(const Plan&, const ForwardArgs&, hipStream_t);
+#define TLCE_LAUNCHERS_GRAD_LOGITS_DIM_FIRST(X, E) \
+  X int launch_grad_logits_dim_first<E>(const GradLogitsArgs&, hipStream_t);
 #define TLCE_LAUNCHERS_GEMM(X, E)                                         \
   X int launch_gemm<E, false, false>(GemmArgs, int, int, hipStream_t);    \
   X int launch_gemm<E, true, false>(GemmArgs, int, int, hipStream_t);     \

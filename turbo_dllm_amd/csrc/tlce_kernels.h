@@ -12,6 +12,9 @@
 
 namespace tlce {
 
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+
 // ------------------------------------------------------------------ forward --
 // Per (token tile, vocabulary split): stream the split's vocabulary tiles,
 // keeping a running (max, sum-exp) per token in registers (base-2 domain), and
@@ -21,7 +24,7 @@ namespace tlce {
 // logits.
 struct ForwardArgs {
   const void* hidden;   // [m, h]
-  const void* weight;   // [v, h]
+  const void* weight;   // [v, h], or [h, v] for the kernels instantiated with kWDimFirst
   const float* bias;    // [v] or null
   int m, h, v;
   int64_t exclude;
@@ -37,7 +40,10 @@ struct ForwardArgs {
   const int64_t* m_dev = nullptr;
 };
 
-template <class E, bool kSoftcap, bool kBias>
+// kWDimFirst (engines with K-major operands only): the head is stored [h, v]
+// (fused_linear_ce.cpp:104 `weight_dim_first`) and read in place as a K-major
+// operand, K = the hidden axis; v is then a multiple of 8.
+template <class E, bool kSoftcap, bool kBias, bool kWDimFirst = false>
 __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
@@ -77,8 +83,14 @@ __global__ __launch_bounds__(E::kThreads) void lce_forward_stats_kernel(ForwardA
     // reloaded from scratch at the top of every tile (3 % of this kernel).
     eng.forget_lane_invariants();
     typename E::Acc acc;
-    eng.mainloop_set(weight, p.h, vt * E::kTile, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h,
-                     acc, smem);
+    if constexpr (kWDimFirst) {
+      const Operand<T> a = {weight, p.v, vt * E::kTile, p.v};
+      const Operand<T> b = {hidden, p.h, tt * E::kTile, p.m};
+      eng.template mainloop_ex<true, false, true>(a, b, 0, p.h, acc, smem);
+    } else {
+      eng.mainloop_set(weight, p.h, vt * E::kTile, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h,
+                       acc, smem);
+    }
     const int vbase = vt * E::kTile;
     if (kBias) {
 #pragma unroll
@@ -190,6 +202,7 @@ struct CombineArgs {
   int weighted_rows = 0;             // entries of `weighted` to define (rows past m get 0)
   int n_vtiles = 0, tile = 0;        // for the device-side plan when m_dev != null
   const int64_t* m_dev = nullptr;
+  bool weight_dim_first = false;     // weight is [h, v]: the label's column is read with stride v
 };
 
 // Dot product of two rows of length h by one wave (every lane gets the sum):
@@ -261,8 +274,17 @@ __global__ __launch_bounds__(256) void lce_combine_loss_kernel(CombineArgs p) {
     float target = 0.0f;
     if (has_target) {
       const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
-      const T* wrow = static_cast<const T*>(p.weight) + y * (int64_t)p.h;
-      float dot = wave_dot<T>(hrow, wrow, p.h, lane) * p.logit_scale;
+      float dot;
+      if (p.weight_dim_first) {
+        const T* wcol = static_cast<const T*>(p.weight) + y;
+        float part = 0.0f;
+        for (int k = lane; k < p.h; k += 64)
+          part = fmaf(to_float<T>(hrow[k]), to_float<T>(wcol[(int64_t)k * p.v]), part);
+        dot = wave_sum(part) * p.logit_scale;
+      } else {
+        const T* wrow = static_cast<const T*>(p.weight) + y * (int64_t)p.h;
+        dot = wave_dot<T>(hrow, wrow, p.h, lane) * p.logit_scale;
+      }
       if (p.bias != nullptr) dot += p.bias[y];
       if (p.softcap > 0.0f) dot = p.softcap * tanhf(dot / p.softcap);
       target = dot;
@@ -371,7 +393,7 @@ __device__ __forceinline__ void stream_store16(void* dst, uint4 v) {
   __builtin_nontemporal_store(x, reinterpret_cast<u4_t*>(dst));
 }
 
-template <class E, bool kSoftcap, bool kBias>
+template <class E, bool kSoftcap, bool kBias, bool kWDimFirst = false>
 __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(GradLogitsArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
@@ -410,7 +432,13 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
     lse2[j] = p.lse[rc] * TLCE_LOG2E;
     scale[j] = live ? p.scale[rc] : 0.0f;
   }
-  eng.mainloop_set(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+  if constexpr (kWDimFirst) {   // the head as stored, [h, v]: a K-major operand
+    const Operand<T> a = {weight, p.v, vbase, p.v};
+    const Operand<T> b = {hidden, p.h, tt * E::kTile, p.m};
+    eng.template mainloop_ex<true, false, true>(a, b, 0, p.h, acc, smem);
+  } else {
+    eng.mainloop_set(weight, p.h, vbase, p.v, hidden, p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+  }
 
   // the bias add applies the logit multiplier itself (z = multiplier * dot + bias)
   const float raw_scale = kBias ? 1.0f : p.logit_scale;
@@ -1044,16 +1072,17 @@ struct GemmArgs {
   const int64_t* m_dev = nullptr;
   int m_role = 0, m_round = 1;
   int64_t slab_budget = 0;   // kRowsFollow: float32 elements all K-split slabs may take
+  int k_steps_plan = 0;      // kRowsFollow: K steps of a full panel, what the split rule plans on
 };
 
 // K splits and slab stride the grad_hidden contraction uses for a device-side
 // row count: the host plan's rule applied to the real number of token tiles,
 // limited to the splits launched and to the slab memory the plan allocated.
 __device__ __forceinline__ int dynamic_k_splits(int n_ttiles, int n_htiles, int tile, int h,
-                                                int launched, int64_t slab_budget,
+                                                int launched, int64_t slab_budget, int k_steps,
                                                 int64_t* stride) {
   const int64_t slab = (int64_t)n_ttiles * tile * h;
-  int ks = grad_hidden_k_splits((int64_t)n_ttiles * n_htiles, launched);
+  int ks = grad_hidden_k_splits((int64_t)n_ttiles * n_htiles, launched, k_steps, slab);
   while (ks > 1 && ks * slab > slab_budget) --ks;
   *stride = slab;
   return ks;
@@ -1070,8 +1099,6 @@ enum { kRowsFollow = 1, kKFollows = 2 };
 // 1 KiB, 16-byte chunk c of staged row s in slot c ^ (s & 63)).  kAdd: the slab's
 // old values of a half are requested before its rows are staged, so their
 // latency passes under the staging.
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
 
 template <class E, bool kAdd>
 __device__ __forceinline__ void store_tile_f32_by_rows(const E& eng, const typename E::Acc& acc,
@@ -1202,7 +1229,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
       p.c_rows = effective_rows(p.c_rows, p.m_dev);
       p.nj = (p.c_rows + E::kTile - 1) / E::kTile;
       const int ks = dynamic_k_splits(p.nj, p.ni, E::kTile, (int)p.ldc, (int)gridDim.y,
-                                      p.slab_budget, &p.c_split_stride);
+                                      p.slab_budget, p.k_steps_plan, &p.c_split_stride);
       if ((int)blockIdx.y >= ks) return;
       p.k_per_split = (p.k / E::kBK + ks - 1) / ks * E::kBK;
     } else if (p.m_role == kKFollows) {
@@ -1334,18 +1361,30 @@ template <typename T>
 __global__ __launch_bounds__(256) void lce_finalize_grad_hidden_kernel(
     const float* __restrict__ acc32, int n_splits, int64_t split_stride,
     const int64_t* __restrict__ row_idx, int m, int h, T* __restrict__ out,
-    const int64_t* __restrict__ m_dev, int n_htiles, int tile, int launched_splits) {
+    const int64_t* __restrict__ m_dev, int n_htiles, int tile, int launched_splits,
+    int k_steps_plan) {
   const int r = blockIdx.x;
   if (m_dev != nullptr) {
     // the splits and slab stride the contraction derived from the real row count
     m = effective_rows(m, m_dev);
     n_splits = dynamic_k_splits((m + tile - 1) / tile, n_htiles, tile, h, launched_splits,
-                                (int64_t)n_splits * split_stride, &split_stride);
+                                (int64_t)n_splits * split_stride, k_steps_plan, &split_stride);
   }
   if (r >= m) return;
   const int64_t o = (row_idx != nullptr) ? row_idx[r] : (int64_t)r;
   const float* src = acc32 + (int64_t)r * h;
   T* dst = out + o * h;
+  if ((h % 4) == 0 && (split_stride % 4) == 0 &&
+      ((reinterpret_cast<uintptr_t>(acc32) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+    // four hidden entries per thread: 16-byte loads of every slab, one vector store
+    for (int k = threadIdx.x * 4; k < h; k += 256 * 4) {
+      f32x4_t sum = *reinterpret_cast<const f32x4_t*>(src + k);
+      for (int s = 1; s < n_splits; ++s)
+        sum += *reinterpret_cast<const f32x4_t*>(src + (int64_t)s * split_stride + k);
+      store4<T>(dst + k, sum[0], sum[1], sum[2], sum[3]);
+    }
+    return;
+  }
   for (int k = threadIdx.x; k < h; k += 256) {
     float sum = src[k];
     for (int s = 1; s < n_splits; ++s) sum += src[(int64_t)s * split_stride + k];

@@ -140,6 +140,10 @@ int forward_entry(const void* hidden, const void* weight, const float* bias,
   const bool local = shard.local_max != nullptr;
   const bool fused = opt.weighted_sum != nullptr;   // the masked-token loss entry point
   if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  TLCE_REQUIRE(!opt.weight_dim_first || dim_first_in_place(h, v, dtype),
+               "forward: a [h, v] head is read in place only for 16-bit inputs with h and v "
+               "multiples of 64 (h=%lld v=%lld dtype=%d); re-lay it to [v, h] for the other "
+               "entry points", (long long)h, (long long)v, dtype);
   TLCE_REQUIRE(valid_count != nullptr, "forward: valid_count is null");
   TLCE_REQUIRE(opt.logit_scale > 0.0f, "forward: the logit multiplier must be positive");
   TLCE_REQUIRE(n_out >= m, "forward: n_out=%lld < m=%lld", (long long)n_out, (long long)m);
@@ -178,6 +182,25 @@ extern "C" int tlce_forward(const void* hidden, const void* weight, const float*
   return forward_entry(hidden, weight, bias, labels, row_idx, m, n_out, h, v, dtype, ignore_index,
                        exclude_index, logit_softcap, losses, lse, valid_count, ShardStats{},
                        workspace, workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+// ------------------------------------------------ head stored [h, v] ----
+extern "C" int tlce_dim_first_supported(int64_t h, int64_t v, int dtype) {
+  return (h > 0 && v > 0 && dim_first_in_place(h, v, dtype)) ? 1 : 0;
+}
+
+extern "C" int tlce_forward_dim_first(const void* hidden, const void* weight, const float* bias,
+                                      const int64_t* labels, const int64_t* row_idx, int64_t m,
+                                      int64_t n_out, int64_t h, int64_t v, int dtype,
+                                      int64_t ignore_index, int64_t exclude_index,
+                                      float logit_softcap, float* losses, float* lse,
+                                      float* valid_count, void* workspace,
+                                      int64_t workspace_bytes, void* stream) {
+  RowOptions opt;
+  opt.weight_dim_first = true;
+  return forward_entry(hidden, weight, bias, labels, row_idx, m, n_out, h, v, dtype, ignore_index,
+                       exclude_index, logit_softcap, losses, lse, valid_count, ShardStats{},
+                       workspace, workspace_bytes, static_cast<hipStream_t>(stream), opt);
 }
 
 // ------------------------------------------- forward without a workspace ----
@@ -274,6 +297,10 @@ int backward_entry(const void* hidden, const void* weight, const float* bias,
                    void* workspace, int64_t workspace_bytes, hipStream_t stream,
                    const RowOptions& opt = RowOptions{}) {
   if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  TLCE_REQUIRE(!opt.weight_dim_first || dim_first_in_place(h, v, dtype),
+               "backward: a [h, v] head is read in place only for 16-bit inputs with h and v "
+               "multiples of 64 (h=%lld v=%lld dtype=%d); re-lay it to [v, h] for the other "
+               "entry points", (long long)h, (long long)v, dtype);
   TLCE_REQUIRE(opt.logit_scale > 0.0f, "backward: the logit multiplier must be positive");
   TLCE_REQUIRE(reduction_code >= TLCE_REDUCTION_NONE && reduction_code <= TLCE_REDUCTION_MEAN,
                "backward: bad reduction code %d", reduction_code);
@@ -323,6 +350,23 @@ extern "C" int tlce_backward(const void* hidden, const void* weight, const float
                         n_out, h, v, dtype, reduction_code, 0, ignore_index, exclude_index,
                         logit_softcap, grad_hidden, grad_weight, grad_bias, panel_bytes, workspace,
                         workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlce_backward_dim_first(const void* hidden, const void* weight, const float* bias,
+                                       const int64_t* labels, const int64_t* row_idx,
+                                       const float* lse, const float* valid_count,
+                                       const float* grad_output, int64_t m, int64_t n_out,
+                                       int64_t h, int64_t v, int dtype, int reduction_code,
+                                       int64_t ignore_index, int64_t exclude_index,
+                                       float logit_softcap, void* grad_hidden, void* grad_weight,
+                                       float* grad_bias, int64_t panel_bytes, void* workspace,
+                                       int64_t workspace_bytes, void* stream) {
+  RowOptions opt;
+  opt.weight_dim_first = true;
+  return backward_entry(hidden, weight, bias, labels, row_idx, lse, valid_count, grad_output, m,
+                        n_out, h, v, dtype, reduction_code, 0, ignore_index, exclude_index,
+                        logit_softcap, grad_hidden, grad_weight, grad_bias, panel_bytes, workspace,
+                        workspace_bytes, static_cast<hipStream_t>(stream), opt);
 }
 
 extern "C" int tlce_backward_local(const void* hidden, const void* weight, const float* bias,

@@ -243,22 +243,38 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
 
     hidden_flat = hidden.reshape(-1, hidden.shape[-1]).contiguous()
     labels_flat = labels.reshape(-1).to(torch.long).contiguous()
-    # the kernels read the head as [V, H]: a [H, V] head is re-laid once here and
-    # the copy is kept for the backward
-    weight_vf = weight.t().contiguous() if weight_dim_first else weight.contiguous()
+    n = hidden_flat.shape[0]
+    # A [H, V] head is read in place where the library can (16-bit inputs, H and V
+    # multiples of 64) and the row count is read back or rows stay in place; otherwise
+    # it is re-laid to [V, H] once here and the copy is kept for the backward.
+    in_place = mode != "device" and native.dim_first_in_place(weight, weight_dim_first)
+    if in_place or not weight_dim_first:
+        weight_vf = weight.contiguous()
+    else:
+        weight_vf = weight.t().contiguous()
     if bias is not None:
         bias = bias.contiguous()
-    n = hidden_flat.shape[0]
 
-    rows, targets, _, row_idx, row_count, m = native.compact_loss_rows(
-        hidden_flat, labels_flat, None, ignore_index, mode)
+    if in_place and mode == "sync":
+        # the entry points that take a device-side row count read a [V, H] head only:
+        # compact with the count read back, as the reference's call sites do
+        row_idx, m = native.compact_rows(labels_flat, ignore_index)
+        row_count = None
+        if m == n:
+            rows, targets, row_idx = hidden_flat, labels_flat, None
+        else:
+            rows = native.gather_rows(hidden_flat, row_idx)
+            targets = native.gather_rows(labels_flat, row_idx)
+    else:
+        rows, targets, _, row_idx, row_count, m = native.compact_loss_rows(
+            hidden_flat, labels_flat, None, ignore_index, mode)
 
     if row_count is None:
         losses, lse, valid_count = native.forward(
             rows, weight_vf, bias, targets,
             row_block_size=0, ignore_index=ignore_index, exclude_index=exclude_index,
             logit_softcap=float(logit_softcap), compute_dtype=compute_dtype,
-            weight_dim_first=False, row_idx=row_idx, n_out=n,
+            weight_dim_first=in_place, row_idx=row_idx, n_out=n,
         )
     else:
         losses, lse, valid_count, _ = native.masked_loss_forward(
@@ -274,6 +290,7 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
     ctx.exclude_index = int(exclude_index)
     ctx.compute_dtype = compute_dtype
     ctx.weight_dim_first = weight_dim_first
+    ctx.in_place = in_place
     ctx.logit_softcap = float(logit_softcap)
     # the backward may run on an autograd worker thread, which does not see this
     # thread's context: the panel budget in force now travels with the node
@@ -296,7 +313,7 @@ def _device_backward(ctx, grad_output, frozen: bool):
                 rows, weight_vf, bias, targets, lse, valid_count, grad_output,
                 row_block_size=0, reduction=ctx.reduction, ignore_index=ctx.ignore_index,
                 exclude_index=ctx.exclude_index, logit_softcap=ctx.logit_softcap,
-                compute_dtype=ctx.compute_dtype, weight_dim_first=False,
+                compute_dtype=ctx.compute_dtype, weight_dim_first=ctx.in_place,
                 row_idx=row_idx, n_out=ctx.n_rows,
             )
         else:
@@ -306,7 +323,7 @@ def _device_backward(ctx, grad_output, frozen: bool):
                 n_out=ctx.n_rows, ignore_index=ctx.ignore_index, exclude_index=ctx.exclude_index,
                 logit_softcap=ctx.logit_softcap, compute_weight_grad=not frozen,
             )
-    if not frozen and ctx.weight_dim_first:
+    if not frozen and ctx.weight_dim_first and not ctx.in_place:
         grad_weight = grad_weight.t().contiguous()
     return (
         grad_hidden.reshape(ctx.hidden_shape),
