@@ -404,14 +404,21 @@ def masked_token_loss(
     logit_softcap: Optional[float] = None,
     loss_scale: float = 1.0,
     dtype: torch.dtype = torch.float64,
+    round_scaled_hidden: bool = False,
 ):
     """``sum_r CE_r * w_r / valid_token_count * loss_scale`` over the rows whose
     label is not -100, CE taken on ``hidden * output_multiplier``
     (nemotron/model.py:2084-2086, :2099-2151).  The multiplication is done in
-    ``dtype`` (the reference rounds the product to the hidden dtype first)."""
-    h = hidden.reshape(-1, hidden.shape[-1]).to(dtype)
-    if output_multiplier is not None:
-        h = h * float(output_multiplier)
+    ``dtype``; with ``round_scaled_hidden`` the product is first rounded to the
+    dtype of ``hidden``, which is where the reference rounds it
+    (``compact_hidden * float(multiplier)`` on the 16-bit tensor)."""
+    h = hidden.reshape(-1, hidden.shape[-1])
+    if output_multiplier is not None and round_scaled_hidden:
+        h = (h * float(output_multiplier)).to(hidden.dtype).to(dtype)
+    else:
+        h = h.to(dtype)
+        if output_multiplier is not None:
+            h = h * float(output_multiplier)
     token_losses = dense_linear_ce(h, weight, labels.reshape(-1), bias=bias, reduction="none",
                                    exclude_index=exclude_index, logit_softcap=logit_softcap,
                                    dtype=dtype)

@@ -259,3 +259,40 @@ def test_non_positive_multiplier_takes_the_reference_sequence(gpu_device):
     wl = workloads.small_head(seed=12, scale=16)
     say("masked_token_loss, multiplier -0.5", "N", wl.n_rows, "M", wl.n_loss_rows)
     check_masked_loss(gpu_device, wl, mode="sync", multiplier=-0.5)
+
+
+def test_multiplier_rounding_point_against_the_reference_order(gpu_device):
+    """The fused path multiplies the float32 dot product by output_multiplier; the
+    reference multiplies the 16-bit hidden states first and rounds them
+    (nemotron/model.py:2084-2086).  For a multiplier that is not a power of two the
+    two differ by the bf16 rounding of hidden * multiplier: the gap is measured
+    here against an oracle that rounds where the reference does, and bounded."""
+    from turbo_dllm_amd.layers import VocabParallelLinear
+
+    dev = gpu_device
+    gen = torch.Generator().manual_seed(77)
+    n, h, v = 600, 256, 3000
+    hidden = torch.randn(n, h, generator=gen).bfloat16()
+    weight = (torch.randn(v, h, generator=gen) * 0.1).bfloat16()
+    labels = torch.randint(0, v, (n,), generator=gen)
+    labels[torch.rand(n, generator=gen) < 0.3] = -100
+    weights = torch.rand(n, generator=gen) + 0.5
+    count = float((labels != -100).sum())
+    head = VocabParallelLinear(h, v, bias=False).to(device=dev, dtype=torch.bfloat16)
+    with torch.no_grad():
+        head.weight.copy_(weight.to(dev))
+    for multiplier in (0.5, 1.75, 0.3):
+        got = float(masked_token_loss(hidden.to(dev), labels.to(dev), weights.to(dev), head,
+                                      valid_token_count=count, output_multiplier=multiplier))
+        exact = float(oracle.masked_token_loss(hidden, weight, labels, weights, count,
+                                               output_multiplier=multiplier))
+        rounded = float(oracle.masked_token_loss(hidden, weight, labels, weights, count,
+                                                 output_multiplier=multiplier,
+                                                 round_scaled_hidden=True))
+        print("[case] multiplier", multiplier, "fused", got, "float product", exact,
+              "rounded product (reference order)", rounded,
+              "gap to the reference order", abs(got - rounded) / abs(rounded), flush=True)
+        assert abs(got - exact) <= 1e-3 * abs(exact)
+        assert abs(got - rounded) <= 1e-3 * abs(rounded)     # inside the loss bar either way
+        if multiplier == 0.5:                                # a power of two rounds nothing
+            assert rounded == exact

@@ -545,3 +545,30 @@ def test_dflash_loss_oracle_per_sample_loop_and_empty_batch():
     assert torch.count_nonzero(dh) == 0 and dw is None
     with pytest.raises(ValueError):
         oracle.dflash_token_loss(hidden, targets, mask, weights, draft_w, counts, loss_kind="kl")
+
+
+def test_masked_token_loss_oracle_rounding_point_of_the_scaled_hidden_states():
+    """round_scaled_hidden=True rounds hidden * multiplier to the 16-bit dtype before the
+    projection, the order of the reference's loss method (nemotron/model.py:2084-2086):
+    pinned against the library expression on the rounded product."""
+    gen = torch.Generator().manual_seed(5)
+    hidden = torch.randn(9, 16, generator=gen).bfloat16()
+    weight = (torch.randn(23, 16, generator=gen) * 0.3).bfloat16()
+    labels = torch.randint(0, 23, (9,), generator=gen)
+    labels[2] = -100
+    weights = torch.rand(9, generator=gen) + 0.5
+    scaled = (hidden * 1.75)                      # bf16 tensor times a Python float: rounds to bf16
+    assert scaled.dtype == torch.bfloat16
+    logits = F.linear(scaled.double(), weight.double())
+    token = F.cross_entropy(logits, labels, reduction="none", ignore_index=-100)
+    expect = (token * weights.double()).sum() / 8.0
+    got = oracle.masked_token_loss(hidden, weight, labels, weights, 8.0, output_multiplier=1.75,
+                                   round_scaled_hidden=True)
+    torch.testing.assert_close(got, expect, rtol=1e-12, atol=1e-12)
+    plain = oracle.masked_token_loss(hidden, weight, labels, weights, 8.0, output_multiplier=1.75)
+    assert float(plain) != float(got) and abs(float(plain) - float(got)) < 1e-2 * float(got)
+    # a power of two rounds nothing
+    a = oracle.masked_token_loss(hidden, weight, labels, weights, 8.0, output_multiplier=0.5)
+    b = oracle.masked_token_loss(hidden, weight, labels, weights, 8.0, output_multiplier=0.5,
+                                 round_scaled_hidden=True)
+    assert float(a) == float(b)
