@@ -445,7 +445,13 @@ def main() -> int:
                          "set_compaction_mode): exact launches after one host read-back of "
                          "the row count, no read-back (device-side count), or no compaction")
     ap.add_argument("--panel-mib", type=int, default=0,
-                    help="budget of the backward's logit-gradient panel in MiB (0: 1 GiB default)")
+                    help="budget of the staging panel between the contractions in MiB (0: the "
+                         "library's default, 2.5 GiB with --gradients forward, 1 GiB with "
+                         "recompute)")
+    ap.add_argument("--gradients", choices=("forward", "recompute"), default="forward",
+                    help="form the gradients in the forward while a block's logits exist "
+                         "(3 contractions per step; the package default) or in a backward "
+                         "that recomputes the logits (4)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain row copy of the weight matrix (known HBM bytes) "
                          "so rocprofv3 FETCH_SIZE / WRITE_SIZE readings can be scaled")
@@ -470,6 +476,7 @@ def main() -> int:
         return 1
     set_compaction_mode(args.compaction_mode)
     options.set_panel_bytes(args.panel_mib << 20)
+    options.set_gradient_mode(args.gradients)
     if args.objective == "masked_loss":
         return bench_masked_loss(args)
     if args.objective != "ce":
@@ -517,7 +524,18 @@ def main() -> int:
         # the same operands and entry points the loss API uses for this compaction mode
         rows, targets, _, row_idx, count, m_rows = native.compact_loss_rows(
             hidden.detach(), labels, None, -100, args.compaction_mode)
-        if count is not None:
+        fused = (args.gradients == "forward" and args.compaction_mode != "device"
+                 and native.fused_gradients_supported(rows, weight.detach(), None, False))
+        if fused:
+            with _lib.kernel_profile() as prof:
+                out = native.forward_with_gradients(
+                    rows[:m_rows], weight.detach(), targets[:m_rows], ignore_index=-100,
+                    exclude_index=-1, logit_softcap=softcap, compute_weight_grad=True,
+                    row_idx=row_idx, n_out=n)
+                native.apply_grad_output(out[3], out[4], go, out[2], reduction="mean",
+                                         dtype=hidden.dtype, row_idx=row_idx, n_out=n)
+            del out
+        elif count is not None:
             kw = dict(m=m_rows, row_idx=row_idx, row_count=count, n_out=n, ignore_index=-100,
                       exclude_index=-1, logit_softcap=softcap)
             with _lib.kernel_profile() as prof:
@@ -551,6 +569,10 @@ def main() -> int:
         "lce_forward_stats_kernel": (prof.ms["forward_stats"], prof.launches["forward_stats"], 1),
         "lce_grad_logits_panel_kernel": (prof.ms["grad_logits_panel"],
                                          prof.launches["grad_logits_panel"], 1),
+        # every block of rows launches this kernel twice; the second launch is the
+        # second try, which exits at once unless the block asked for it
+        "lce_exp_logits_panel_kernel": (prof.ms["exp_logits_panel"],
+                                        prof.launches["exp_logits_panel"] // 2, 1),
         "lce_gemm_nt_kernel": (prof.ms["grad_hidden_gemm"] + prof.ms["grad_weight_gemm"],
                                prof.launches["grad_hidden_gemm"]
                                + prof.launches["grad_weight_gemm"], 2),
@@ -561,12 +583,17 @@ def main() -> int:
     avg_ms = total_ms / launches
     flops_per_launch = contractions * contraction_tflop * 1e12 / launches
     achieved = flops_per_launch / 1e12 / (avg_ms / 1e3)
+    executed_contractions = 3 if fused else 4
     useful_tflops = 3.0 * contraction_tflop / (ms_per_step / 1e3)
-    executed_tflops = 4.0 * contraction_tflop / (ms_per_step / 1e3)
+    executed_tflops = executed_contractions * contraction_tflop / (ms_per_step / 1e3)
     # launches are sized for the loss-bearing rows, or for all rows when the count is not
     # read back / rows are not compacted
     plan_rows = m if args.compaction_mode == "sync" else n
-    plan = _lib.query_plan(plan_rows, h, v, _lib.DTYPE_BF16, True, options.get_panel_bytes())
+    if fused:
+        plan = {"engine": "mfma_direct", "tile": 256,
+                **_lib.query_fused_plan(plan_rows, h, v, _lib.DTYPE_BF16, options.get_panel_bytes())}
+    else:
+        plan = _lib.query_plan(plan_rows, h, v, _lib.DTYPE_BF16, True, options.get_panel_bytes())
     traffic, traffic_note = measured_traffic(wl.name, dominant)
 
     result = {
@@ -587,19 +614,18 @@ def main() -> int:
                         f"softcap={wl.logit_softcap}, seed={args.seed}",
             "input_rows_per_s": n / (ms_per_step / 1e3),
             "compaction_mode": args.compaction_mode,
-            "panel_bytes": options.get_panel_bytes() or (1 << 30),
+            "gradients": "forward" if fused else "recompute",
+            "panel_bytes": options.get_panel_bytes() or ((5 << 29) if fused else (1 << 30)),
             "plan": plan,
             "sources": source_fingerprint(),
         },
         "loss": loss_value,
         "tflops_useful_6MHV": useful_tflops,
-        "tflops_executed_8MHV": executed_tflops,
+        "contractions_executed": executed_contractions,
+        "tflops_executed": executed_tflops,
         "frac_of_bf16_peak_useful": useful_tflops / PEAK_BF16_TFLOPS,
         "mfma_util_executed": executed_tflops / PEAK_BF16_TFLOPS,
         "ms_per_step_median": ms_median,
-        "forward_only_ms": round(prof.ms["forward_stats"] + prof.ms["combine_loss"], 3),
-        "backward_only_ms": round(sum(x for k, x in prof.ms.items()
-                                      if k not in ("forward_stats", "combine_loss")), 3),
         "kernel_ms": {k: round(x, 3) for k, x in prof.ms.items()},
         "kernel_launches": prof.launches,
         "roofline": {

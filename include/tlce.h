@@ -427,6 +427,59 @@ int tlce_segment_weighted_sum(const float* values, const float* weights,
                               int64_t m, int64_t segment_length, int64_t n_segments,
                               float* out, void* stream);
 
+/* ---- forward that also leaves the gradients: 3 contractions, not 4 ---------
+ * Replaces the pair fused_linear_ce_forward + fused_linear_ce_backward
+ * (dllm_parallel/csrc/fused_linear_ce.cpp:94-207) for callers whose upstream
+ * gradient is one number (reduction "sum" / "mean", or a weighted sum of the
+ * token losses): the reference's backward recomputes the logits of every block
+ * (fused_linear_ce_cuda.cu:618-791), the plain entry points here do the same
+ * by vocabulary panels.  This entry point forms the gradients of
+ *     S = sum_r token_weights[r] * loss[r]
+ * while the logits of a block of rows exist:
+ *     grad_hidden_f32[r, :]  = dS / d hidden[r, :]      [m, h] float32, compact rows
+ *     grad_weight_f32[v, :]  = dS / d weight[v, :]      [v, h] float32 (NULL: frozen head)
+ * and writes losses / lse / valid_count as tlce_forward does (losses unweighted).
+ * tlce_apply_grad_output then multiplies both by the upstream gradient
+ * (grad_output[0], divided by valid_count[0] for TLCE_REDUCTION_MEAN), rounds
+ * them once to the input dtype, and un-compacts grad_hidden through row_idx
+ * into [n_out, h] (other rows zero).  No bias, head stored [v, h], 16-bit inputs
+ * with h and v multiples of 64 (tlce_fused_gradients_supported); everything else
+ * goes through tlce_forward / tlce_backward.
+ *
+ * Rows are taken in blocks of as many rows as a panel of panel_bytes (0: 2.5 GiB)
+ * holds over the whole vocabulary (tlce_query_fused_plan); the panel holds
+ * exp(logit - reference) in the input dtype, the reference being the label's
+ * logit of the row.  A block in which some row's largest logit lies more than
+ * 40 (8 for f16) above its reference is produced a second time with the exact
+ * row maxima as references; the decision is taken on the device, the second
+ * try's launches are always made and do nothing otherwise.
+ * logit_multiplier > 0 scales the raw dot products (1: plain operator). */
+int tlce_fused_gradients_supported(int64_t h, int64_t v, int dtype);
+
+int tlce_query_fused_plan(int64_t m, int64_t h, int64_t v, int dtype,
+                          int64_t panel_bytes, int64_t* block_rows, int* n_blocks,
+                          int* grad_hidden_k_splits);
+
+int64_t tlce_forward_with_gradients_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                                    int dtype, int compute_weight_grad,
+                                                    int64_t panel_bytes);
+
+int tlce_forward_with_gradients(const void* hidden, const void* weight,
+                                const int64_t* labels, const int64_t* row_idx,
+                                const float* token_weights, int64_t m, int64_t n_out,
+                                int64_t h, int64_t v, int dtype, int64_t ignore_index,
+                                int64_t exclude_index, float logit_softcap,
+                                float logit_multiplier, float* losses, float* lse,
+                                float* valid_count, float* grad_hidden_f32,
+                                float* grad_weight_f32, int64_t panel_bytes,
+                                void* workspace, int64_t workspace_bytes, void* stream);
+
+int tlce_apply_grad_output(const float* grad_hidden_f32, const float* grad_weight_f32,
+                           const int64_t* row_idx, const float* grad_output,
+                           const float* valid_count, int64_t m, int64_t n_out,
+                           int64_t h, int64_t v, int dtype, int reduction_code,
+                           void* grad_hidden, void* grad_weight, void* stream);
+
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be
  * NULL.  `engine` is 2 for the bf16/f16 MFMA kernels with direct-to-LDS loads
@@ -446,9 +499,9 @@ int tlce_query_plan(int64_t m, int64_t h, int64_t v, int dtype,
  *   0 forward logits+softmax-stats tiles   1 per-row loss merge
  *   2 backward logit-gradient panel tiles  3 grad_hidden contraction
  *   4 grad_weight contraction              5 operand transposes
- *   6 fills, scales and casts
+ *   6 fills, scales and casts             7 exponentiated-logits panel tiles
  * The events allocate driver resources: not for use under graph capture. */
-#define TLCE_PROFILE_CLASSES 7
+#define TLCE_PROFILE_CLASSES 8
 int tlce_profile_begin(void);
 int tlce_profile_end(double* class_ms, int64_t* class_launches, int n_classes);
 

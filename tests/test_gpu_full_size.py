@@ -28,14 +28,20 @@ def say(*parts):
     print("[case]", *parts, flush=True)
 
 
-def run(dev, wl, grad_scale=1.0):
+def run(dev, wl, grad_scale=1.0, reduction="none"):
+    """Forward + backward through the public operator.  reduction "none" with a
+    per-row upstream gradient goes through the backward that recomputes the logits;
+    "mean" through the forward that forms the gradients while the logits exist."""
     hidden = wl.hidden.to(dev).requires_grad_(True)
     weight = wl.weight.to(dev).requires_grad_(True)
-    losses = tiled_linear_cross_entropy(hidden, weight, wl.labels.to(dev), reduction="none",
+    losses = tiled_linear_cross_entropy(hidden, weight, wl.labels.to(dev), reduction=reduction,
                                         logit_softcap=wl.logit_softcap, dtype=hidden.dtype,
                                         weight_layout="vocab_first")
     m = max(wl.n_loss_rows, 1)
-    losses.backward(torch.full_like(losses, grad_scale / m))
+    if reduction == "none":
+        losses.backward(torch.full_like(losses, grad_scale / m))
+    else:
+        (losses * grad_scale).backward()
     torch.cuda.synchronize()
     return losses.detach().cpu(), hidden.grad.cpu(), weight.grad.cpu()
 
@@ -100,7 +106,7 @@ def test_block_diffusion_labels_compaction_full_size(gpu_device):
 
 # ------------------------------------------------- remaining configurations ----
 def check_configuration_full_size(dev, wl, *, check_column_sums=True, token_rows=None,
-                                  vocab_rows=None):
+                                  vocab_rows=None, reduction="none"):
     """One benchmark configuration at full size against the float32 oracle.
 
     The oracle's per-row loss and lse are computed for every loss-bearing row (in
@@ -114,18 +120,23 @@ def check_configuration_full_size(dev, wl, *, check_column_sums=True, token_rows
     h, v = wl.hidden.shape[1], wl.weight.shape[0]
     cap = wl.logit_softcap
     say(wl.name, "N", n, "M", m, "H", h, "V", v, "softcap", cap)
-    losses, dh, dw = run(dev, wl)
+    losses, dh, dw = run(dev, wl, reduction=reduction)
     say("device done")
     keep = wl.labels != -100
     rows = torch.nonzero(keep).flatten()
-    assert torch.count_nonzero(losses[~keep]) == 0
     assert torch.count_nonzero(dh[~keep]) == 0
     assert bool(torch.isfinite(losses).all()) and bool(torch.isfinite(dh.float()).all())
     assert bool(torch.isfinite(dw.float()).all())
 
     ref_loss, ref_lse = oracle_lse_in_chunks(wl, rows)
-    torch.testing.assert_close(losses[rows], ref_loss, rtol=1e-3, atol=1e-4)
-    say("losses on all", rows.numel(), "loss-bearing rows ok")
+    if reduction == "none":
+        assert torch.count_nonzero(losses[~keep]) == 0
+        torch.testing.assert_close(losses[rows], ref_loss, rtol=1e-3, atol=1e-4)
+        say("losses on all", rows.numel(), "loss-bearing rows ok")
+    else:
+        ref_mean = float(ref_loss.double().mean())
+        say("mean loss", float(losses), "oracle", ref_mean)
+        assert abs(float(losses) - ref_mean) <= 1e-3 * abs(ref_mean)
 
     gen = torch.Generator().manual_seed(1)
     if token_rows is None:
@@ -167,6 +178,47 @@ def check_configuration_full_size(dev, wl, *, check_column_sums=True, token_rows
 
 def test_block_diffusion_shard_full_size(gpu_device):
     check_configuration_full_size(gpu_device, workloads.block_diffusion_shard(seed=6))
+
+
+# The same configurations with the loss reduced to its mean: the gradients are formed
+# in the forward, in blocks of rows over the whole vocabulary (three contractions).
+def test_headline_shape_gradients_formed_in_the_forward(gpu_device):
+    """The shape and path the benchmark times: 32768 loss-bearing rows in four blocks
+    of 8192, grad_weight accumulated in float32 over the blocks.  Token rows on block
+    and tile edges, vocabulary rows at both ends, labels and random ones."""
+    from turbo_dllm_amd import _lib
+    wl = workloads.block_diffusion_shard(seed=0, all_rows_loss_bearing=True)
+    n, v = wl.n_rows, wl.weight.shape[0]
+    plan = _lib.query_fused_plan(n, 4096, v, _lib.DTYPE_BF16)
+    say("plan", plan)
+    block_rows = plan["block_rows"]
+    assert plan["n_blocks"] == 4 and block_rows == 8192
+    gen = torch.Generator().manual_seed(3)
+    token_rows = torch.cat([torch.tensor([0, 255, 256, block_rows - 1, block_rows,
+                                          3 * block_rows - 1, 3 * block_rows, n - 1]),
+                            torch.randperm(n, generator=gen)[:40]])
+    vocab_rows = torch.cat([torch.tensor([0, 1, 255, 256, v - 256, v - 1]),
+                            torch.randint(0, v, (34,), generator=gen)])
+    _, dh, dw = check_configuration_full_size(gpu_device, wl, token_rows=token_rows,
+                                              vocab_rows=vocab_rows, reduction="mean")
+    _, dh2, dw2 = run(gpu_device, wl, grad_scale=2.0, reduction="mean")
+    assert torch.equal(dh2.float(), dh.float() * 2.0)
+    assert torch.equal(dw2.float(), dw.float() * 2.0)
+
+
+def test_block_diffusion_shard_full_size_gradients_formed_in_the_forward(gpu_device):
+    check_configuration_full_size(gpu_device, workloads.block_diffusion_shard(seed=6),
+                                  reduction="mean")
+
+
+def test_gemma_softcap_head_full_size_gradients_formed_in_the_forward(gpu_device):
+    check_configuration_full_size(gpu_device, workloads.gemma_softcap_head(seed=7),
+                                  check_column_sums=False, reduction="mean")
+
+
+def test_sparse_drafter_head_full_size_gradients_formed_in_the_forward(gpu_device):
+    check_configuration_full_size(gpu_device, workloads.sparse_drafter_head(seed=8),
+                                  reduction="mean")
 
 
 def test_gemma_softcap_head_full_size(gpu_device):
@@ -213,11 +265,12 @@ def test_block_diffusion_shard_full_size_without_host_read_back(gpu_device):
         torch.cuda.synchronize()
         results[mode] = (loss.detach().cpu(), hidden.grad.cpu(), head.weight.grad.cpu())
         say(mode, "loss", float(loss.detach()))
-    # same forward plan in both modes -> identical loss; gradients differ only in the
-    # order the vocabulary panels are accumulated
-    assert torch.equal(results["sync"][0], results["device"][0])
+    # "sync" forms the gradients in the forward (three contractions), "device" in a
+    # backward that recomputes the logits: the same loss up to summation order, and
+    # gradients that differ by the rounding of two different 16-bit panels
+    torch.testing.assert_close(results["sync"][0], results["device"][0], rtol=1e-5, atol=0)
     for a, b in zip(results["sync"][1:], results["device"][1:]):
-        assert oracle.relative_max_error(b, a.float()) <= 5e-3
+        assert oracle.relative_max_error(b, a.float()) <= 1e-2
     keep = wl.labels != -100
     rows = torch.nonzero(keep).flatten()
     pick = rows[torch.randperm(m, generator=gen)[:256]]

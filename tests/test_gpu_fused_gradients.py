@@ -1,0 +1,244 @@
+"""GPU parity of the forward that also leaves the gradients
+(``tlce_forward_with_gradients`` + ``tlce_apply_grad_output``: three contractions
+instead of the four of forward + recomputing backward).
+
+It replaces the pair fused_linear_ce_forward / fused_linear_ce_backward
+(dllm_parallel/csrc/fused_linear_ce.cpp:94-207) for scalar reductions, so the
+checks are the operator's: loss within 1e-3 relative and gradients within 2e-2
+relative max-norm of the float32 oracle (bf16 / f16 inputs), through the ctypes
+binding of the C ABI and through the public loss API.
+"""
+
+import pytest
+import torch
+
+import linear_ce_oracle as oracle
+from turbo_dllm_amd import _lib, options
+from turbo_dllm_amd import chunked_linear_ce_native as native
+from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL = 1e-3
+GRAD_REL_MAX = 2e-2
+
+
+def say(*parts):
+    print("[case]", *parts, flush=True)
+
+
+def make_case(m, h, v, *, seed, dtype=torch.bfloat16, ignored=0.0, std=0.05):
+    gen = torch.Generator().manual_seed(seed)
+    hidden = torch.randn(m, h, generator=gen).to(dtype)
+    weight = (torch.randn(v, h, generator=gen) * std).to(dtype)
+    labels = torch.randint(0, v, (m,), generator=gen)
+    if ignored > 0:
+        labels[torch.rand(m, generator=gen) < ignored] = -100
+    return hidden, weight, labels
+
+
+def run_fused(dev, hidden, weight, labels, *, reduction="mean", exclude=-1, softcap=0.0,
+              grad_output=0.7, weight_grad=True, token_weights=None, multiplier=1.0,
+              row_idx=None, n_out=None):
+    out = native.forward_with_gradients(
+        hidden.to(dev), weight.to(dev), labels.to(dev), ignore_index=-100, exclude_index=exclude,
+        logit_softcap=softcap, compute_weight_grad=weight_grad,
+        token_weights=None if token_weights is None else token_weights.to(dev),
+        logit_multiplier=multiplier, row_idx=row_idx, n_out=n_out)
+    losses, lse, valid, dh32, dw32 = out
+    go = torch.tensor([grad_output], device=dev)
+    dh, dw = native.apply_grad_output(dh32, dw32, go, valid, reduction=reduction,
+                                      dtype=hidden.dtype, row_idx=row_idx, n_out=n_out,
+                                      vocab=weight.shape[0])
+    torch.cuda.synchronize()
+    return losses.cpu(), lse.cpu(), float(valid), dh.cpu(), None if dw is None else dw.cpu()
+
+
+@pytest.mark.parametrize("m,h,v,kw", [
+    (300, 256, 1024, {}),
+    (1, 64, 64, {}),
+    (257, 128, 4160, dict(softcap=30.0, exclude=17, ignored=0.3)),
+    (1000, 512, 2048 + 64, dict(exclude=5)),
+    (520, 192, 8192, dict(reduction="sum", ignored=0.5)),
+    (700, 256, 3072, dict(dtype=torch.float16, softcap=15.0)),
+    (2048, 1024, 32000, dict(panel=40 << 20)),          # 2 blocks of rows
+    (1500, 256, 5120, dict(panel=1, ignored=0.2)),        # one token tile per block, 6 blocks
+])
+def test_fused_gradients_match_the_oracle(gpu_device, m, h, v, kw):
+    say("fused gradients", m, h, v, kw)
+    kw = dict(kw)
+    dtype = kw.pop("dtype", torch.bfloat16)
+    reduction = kw.pop("reduction", "mean")
+    exclude = kw.pop("exclude", None)
+    softcap = kw.pop("softcap", None)
+    panel = kw.pop("panel", 0)
+    hidden, weight, labels = make_case(m, h, v, seed=m + v, dtype=dtype, ignored=kw.pop("ignored", 0.0))
+    if exclude is not None:
+        labels[::7] = exclude          # rows whose label is the excluded column
+    with options.panel_budget(panel):
+        losses, lse, valid, dh, dw = run_fused(
+            gpu_device, hidden, weight, labels, reduction=reduction,
+            exclude=-1 if exclude is None else exclude, softcap=softcap or 0.0)
+    okw = dict(exclude_index=exclude, logit_softcap=softcap, dtype=torch.float32)
+    ref_losses, ref_lse = oracle.dense_linear_ce(hidden, weight, labels, reduction="none",
+                                                 return_lse=True, **okw)
+    keep = labels != -100
+    if exclude is not None:
+        # a row labelled with the excluded column: loss = lse (its logit is not defined)
+        on_excluded = labels == exclude
+        ref_losses = torch.where(on_excluded, ref_lse, ref_losses)
+    assert valid == float(keep.sum())
+    torch.testing.assert_close(losses[keep], ref_losses[keep], rtol=LOSS_RTOL, atol=1e-3)
+    assert torch.all(losses[~keep] == 0)
+    torch.testing.assert_close(lse[keep], ref_lse[keep], rtol=LOSS_RTOL, atol=1e-3)
+    go = torch.tensor(0.7)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, go, reduction=reduction, **okw)
+    err_h = oracle.relative_max_error(dh, rdh)
+    err_w = oracle.relative_max_error(dw, rdw)
+    say(f"  dH {err_h:.2e} dW {err_w:.2e}")
+    assert err_h <= GRAD_REL_MAX and err_w <= GRAD_REL_MAX
+    assert torch.all(dh[~keep] == 0)
+
+
+def test_rows_far_from_their_reference_take_the_second_try(gpu_device):
+    """Rows whose largest logit lies more than the window above the label's logit
+    (losses above 40 nats) are produced a second time with the exact maximum as
+    reference; losses and gradients must come out as for any other row."""
+    say("second try")
+    m, h, v = 600, 128, 2048
+    hidden, weight, labels = make_case(m, h, v, seed=5, std=0.05)
+    # every third row points along a weight row other than its label's, scaled so that
+    # this logit is ~100-200 while the label's stays near 0
+    for r in range(0, m, 3):
+        other = (int(labels[r]) + 1) % v
+        direction = weight[other].float()
+        hidden[r] = (direction * (150.0 / float(direction @ direction))).to(hidden.dtype)
+    losses, lse, valid, dh, dw = run_fused(gpu_device, hidden, weight, labels)
+    okw = dict(dtype=torch.float32)
+    ref_losses = oracle.dense_linear_ce(hidden, weight, labels, reduction="none", **okw)
+    assert float(ref_losses.max()) > 60.0     # the case does leave the window
+    torch.testing.assert_close(losses, ref_losses, rtol=LOSS_RTOL, atol=1e-3)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, torch.tensor(0.7), **okw)
+    err_h = oracle.relative_max_error(dh, rdh)
+    err_w = oracle.relative_max_error(dw, rdw)
+    say(f"  max loss {float(ref_losses.max()):.1f} dH {err_h:.2e} dW {err_w:.2e}")
+    assert err_h <= GRAD_REL_MAX and err_w <= GRAD_REL_MAX
+    assert torch.isfinite(dh.float()).all() and torch.isfinite(dw.float()).all()
+
+
+def test_frozen_head_weights_and_multiplier(gpu_device):
+    """No grad_weight when the head is frozen; per-row loss weights and the logit
+    multiplier enter the gradients as in the masked-token loss
+    (nemotron/model.py:2084-2151)."""
+    say("frozen head, token weights, multiplier")
+    m, h, v = 900, 256, 4096
+    hidden, weight, labels = make_case(m, h, v, seed=11, ignored=0.25)
+    gen = torch.Generator().manual_seed(3)
+    weights = torch.rand(m, generator=gen) + 0.25
+    multiplier = 0.5
+    losses, lse, valid, dh, dw = run_fused(gpu_device, hidden, weight, labels, reduction="sum",
+                                           weight_grad=False, token_weights=weights,
+                                           multiplier=multiplier, grad_output=1.0)
+    assert dw is None
+    keep = labels != -100
+    count = float(keep.sum())
+    ref = oracle.masked_token_loss(hidden, weight, labels, weights, count,
+                                   output_multiplier=multiplier, dtype=torch.float32)
+    mine = float((losses * weights).sum()) / count
+    assert abs(mine - float(ref)) <= LOSS_RTOL * abs(float(ref))
+    rdh, _, _ = oracle.masked_token_loss_grads(hidden, weight, labels, weights, count,
+                                               output_multiplier=multiplier, dtype=torch.float32)
+    err_h = oracle.relative_max_error(dh / count, rdh)
+    say(f"  dH {err_h:.2e}")
+    assert err_h <= GRAD_REL_MAX
+
+
+def test_uncompaction_through_row_idx(gpu_device):
+    say("row_idx scatter")
+    n, h, v = 1200, 128, 1024
+    hidden, weight, labels = make_case(n, h, v, seed=21, ignored=0.6)
+    dev = gpu_device
+    row_idx, m = native.compact_rows(labels.to(dev), -100)
+    rows = native.gather_rows(hidden.to(dev), row_idx)
+    targets = native.gather_rows(labels.to(dev), row_idx)
+    losses, _, valid, dh, dw = run_fused(dev, rows, weight, targets, row_idx=row_idx, n_out=n)
+    assert valid == m and losses.shape == (n,) and dh.shape == (n, h)
+    okw = dict(dtype=torch.float32)
+    ref_losses = oracle.dense_linear_ce(hidden, weight, labels, reduction="none", **okw)
+    torch.testing.assert_close(losses, ref_losses, rtol=LOSS_RTOL, atol=1e-3)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, torch.tensor(0.7), **okw)
+    assert oracle.relative_max_error(dh, rdh) <= GRAD_REL_MAX
+    assert oracle.relative_max_error(dw, rdw) <= GRAD_REL_MAX
+    assert torch.all(dh[labels == -100] == 0)
+
+
+@pytest.mark.parametrize("reduction", ["mean", "sum"])
+@pytest.mark.parametrize("frozen", [False, True])
+def test_loss_api_takes_the_fused_path_and_agrees_with_recompute(gpu_device, reduction, frozen):
+    """The public operator: the default gradient mode forms the gradients in the
+    forward (its kernels show up in the library's per-class launch counts instead of
+    the plain forward's), "recompute" keeps the four-contraction path;
+    both agree with each other far inside the oracle's bars."""
+    say("loss API", reduction, frozen)
+    m, h, v = 1100, 256, 4096
+    hidden, weight, labels = make_case(m, h, v, seed=31, ignored=0.3)
+    dev = gpu_device
+    results = {}
+    for mode in options.GRADIENT_MODES:
+        x = hidden.to(dev).requires_grad_(True)
+        w = weight.to(dev).requires_grad_(not frozen)
+        with options.gradient_mode(mode), _lib.kernel_profile() as prof:
+            loss = tiled_linear_cross_entropy(x, w, labels.to(dev), reduction=reduction,
+                                              dtype=torch.bfloat16, weight_layout="vocab_first")
+            (loss * 1.5).backward()
+            torch.cuda.synchronize()
+        results[mode] = (float(loss.detach()), x.grad.cpu(), None if frozen else w.grad.cpu())
+        # (the profile sees this thread's launches: the forward's)
+        if mode == "forward":
+            assert prof.launches["exp_logits_panel"] > 0 and prof.launches["forward_stats"] == 0
+        else:
+            assert prof.launches["exp_logits_panel"] == 0 and prof.launches["forward_stats"] > 0
+    a, b = results["forward"], results["recompute"]
+    assert abs(a[0] - b[0]) <= 1e-5 * abs(b[0])
+    assert oracle.relative_max_error(a[1], b[1].float()) <= 1e-2
+    if not frozen:
+        assert oracle.relative_max_error(a[2], b[2].float()) <= 1e-2
+    ref = oracle.dense_linear_ce(hidden, weight, labels, reduction=reduction, dtype=torch.float32)
+    assert abs(a[0] - float(ref)) <= LOSS_RTOL * abs(float(ref))
+
+
+def test_no_gradient_needed_means_plain_forward(gpu_device):
+    say("no grad")
+    hidden, weight, labels = make_case(300, 128, 1024, seed=41)
+    dev = gpu_device
+    with _lib.kernel_profile() as prof, torch.no_grad():
+        tiled_linear_cross_entropy(hidden.to(dev), weight.to(dev), labels.to(dev),
+                                   dtype=torch.bfloat16, weight_layout="vocab_first")
+        torch.cuda.synchronize()
+    assert prof.launches["exp_logits_panel"] == 0 and prof.launches["forward_stats"] > 0
+
+
+def test_linear_in_the_upstream_gradient_and_repeatable(gpu_device):
+    """apply_grad_output is linear in grad_output bit for bit (a power of two), and the
+    whole path gives the same bits on every run (no float atomics on the gradients)."""
+    say("linearity / determinism")
+    hidden, weight, labels = make_case(777, 256, 3072, seed=51, ignored=0.1)
+    a = run_fused(gpu_device, hidden, weight, labels, grad_output=0.5)
+    b = run_fused(gpu_device, hidden, weight, labels, grad_output=1.0)
+    c = run_fused(gpu_device, hidden, weight, labels, grad_output=1.0)
+    assert torch.equal(b[3], c[3]) and torch.equal(b[4], c[4]) and torch.equal(b[0], c[0])
+    assert torch.equal(a[3].float() * 2, b[3].float()) and torch.equal(a[4].float() * 2, b[4].float())
+
+
+def test_unsupported_operands_are_rejected_before_any_launch(gpu_device):
+    dev = gpu_device
+    hidden = torch.zeros(8, 96, dtype=torch.bfloat16, device=dev)     # h not a multiple of 64
+    weight = torch.zeros(128, 96, dtype=torch.bfloat16, device=dev)
+    labels = torch.zeros(8, dtype=torch.long, device=dev)
+    assert not native.fused_gradients_supported(hidden, weight, None, False)
+    with pytest.raises(RuntimeError, match="multiples"):
+        native.forward_with_gradients(hidden, weight, labels, ignore_index=-100, exclude_index=-1,
+                                      logit_softcap=0.0, compute_weight_grad=True)
+    h32 = torch.zeros(8, 64, dtype=torch.float32, device=dev)
+    w32 = torch.zeros(128, 64, dtype=torch.float32, device=dev)
+    assert not native.fused_gradients_supported(h32, w32, None, False)

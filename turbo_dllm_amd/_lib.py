@@ -103,6 +103,32 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_fused_gradients_supported": (c_int, [c_int64, c_int64, c_int]),
+    "tlce_query_fused_plan": (
+        c_int, [c_int64, c_int64, c_int64, c_int, c_int64, c_void_p, c_void_p, c_void_p]
+    ),
+    "tlce_forward_with_gradients_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int, c_int, c_int64]
+    ),
+    "tlce_forward_with_gradients": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden weight labels row_idx weights
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m n_out h v dtype
+            c_int64, c_int64, c_float, c_float,                 # ignore exclude softcap multiplier
+            c_void_p, c_void_p, c_void_p,                       # losses lse valid_count
+            c_void_p, c_void_p,                                 # grad_hidden_f32 grad_weight_f32
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
+    "tlce_apply_grad_output": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # dh32 dw32 row_idx grad_output valid
+            c_int64, c_int64, c_int64, c_int64, c_int, c_int,   # m n_out h v dtype reduction
+            c_void_p, c_void_p, c_void_p,                       # grad_hidden grad_weight stream
+        ],
+    ),
     "tlce_masked_loss_forward_workspace_bytes": (
         c_int64, [c_int64, c_int64, c_int64, c_int, c_int]
     ),
@@ -290,9 +316,25 @@ def query_plan(m: int, h: int, v: int, dtype_code: int, compute_weight_grad: boo
     }
 
 
+def query_fused_plan(m: int, h: int, v: int, dtype_code: int, panel_bytes: int = 0) -> dict:
+    """How the forward that leaves the gradients would take ``m`` rows: rows per
+    block, blocks, and K splits of the grad_hidden contraction (no GPU needed)."""
+    block_rows = c_int64()
+    n_blocks, ksplits = c_int(), c_int()
+    check(
+        library().tlce_query_fused_plan(
+            m, h, v, dtype_code, panel_bytes, ctypes.byref(block_rows), ctypes.byref(n_blocks),
+            ctypes.byref(ksplits),
+        ),
+        "tlce_query_fused_plan",
+    )
+    return {"block_rows": block_rows.value, "n_blocks": n_blocks.value,
+            "grad_hidden_k_splits": ksplits.value}
+
+
 PROFILE_CLASSES = (
     "forward_stats", "combine_loss", "grad_logits_panel", "grad_hidden_gemm",
-    "grad_weight_gemm", "transpose", "other",
+    "grad_weight_gemm", "transpose", "other", "exp_logits_panel",
 )
 
 

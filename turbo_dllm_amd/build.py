@@ -33,7 +33,7 @@ _WHOLE_ENGINES = {"staged_bf16": "MfmaEngine<__bf16>", "staged_f16": "MfmaEngine
                   "generic_f16": "SimtEngine<_Float16>"}
 _PARTS = {2: "grad_logits", 7: "grad_logits_cap", 8: "grad_logits_bias", 9: "grad_logits_cap_bias",
           1: "forward", 3: "gemm", 4: "kl", 5: "logits", 6: "sequences",
-          10: "forward_dim_first", 11: "grad_logits_dim_first"}
+          10: "forward_dim_first", 11: "grad_logits_dim_first", 12: "exp_panel"}
 UNITS = (
     [(f"engine_{tag}_{name}", "tlce_engine_unit.hip",
       (f"-DTLCE_UNIT_ENGINE={engine}", f"-DTLCE_UNIT_PART={part}"))

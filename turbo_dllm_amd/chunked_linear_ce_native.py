@@ -461,6 +461,135 @@ def forward(
     return losses, lse, valid_count
 
 
+# ------------------------------------------- forward that leaves the gradients --
+def fused_gradients_supported(hidden: torch.Tensor, weight: torch.Tensor,
+                              bias: torch.Tensor | None, weight_dim_first: bool) -> bool:
+    """Whether ``forward_with_gradients`` takes these operands: 16-bit inputs on
+    the GPU, head stored [V, H], no bias, H and V multiples of 64."""
+    if bias is not None or weight_dim_first or not hidden.is_cuda:
+        return False
+    if hidden.dtype not in (torch.bfloat16, torch.float16) or weight.dtype != hidden.dtype:
+        return False
+    if hidden.dim() != 2 or weight.dim() != 2 or weight.shape[1] != hidden.shape[1]:
+        return False
+    return bool(_lib.library().tlce_fused_gradients_supported(
+        hidden.shape[1], weight.shape[0], _dtype_code(hidden)))
+
+
+def forward_with_gradients(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    ignore_index: int,
+    exclude_index: int,
+    logit_softcap: float,
+    compute_weight_grad: bool,
+    token_weights: torch.Tensor | None = None,
+    logit_multiplier: float = 1.0,
+    row_idx: torch.Tensor | None = None,
+    n_out: int | None = None,
+):
+    """The forward and, in the same pass over the logits, the float32 gradients of
+    ``sum_r token_weights[r] * loss[r]`` (three contractions instead of the four
+    of ``forward`` + ``backward``).
+
+    Returns ``(losses [n_out] f32, lse [m] f32, valid_count [1] f32,
+    grad_hidden_f32 [m, H], grad_weight_f32 [V, H] or None)``;
+    ``apply_grad_output`` turns the last two into the gradients of the reduced
+    loss once the upstream gradient is known.
+    """
+    device = _require_device(hidden, weight, labels, row_idx, token_weights)
+    if not fused_gradients_supported(hidden, weight, None, False):
+        raise RuntimeError(
+            "forward_with_gradients needs bf16/f16 operands, a [V, H] head and H, V multiples "
+            "of 64; use forward / backward for other inputs"
+        )
+    hidden = _dense(hidden)
+    weight = _dense(weight)
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v = weight.shape[0]
+    if labels.numel() != m:
+        raise RuntimeError("native linear CE shape mismatch")
+    if row_idx is not None and row_idx.numel() != m:
+        raise RuntimeError("row_idx must have one entry per row")
+    if token_weights is not None:
+        token_weights = token_weights.reshape(-1).to(torch.float32).contiguous()
+        if token_weights.numel() != m:
+            raise RuntimeError("token_weights must have one entry per row")
+    n_out = m if n_out is None else int(n_out)
+    lib = _lib.library()
+    code = _dtype_code(hidden)
+    panel = get_panel_bytes()
+    with torch.cuda.device(device):
+        losses = torch.empty(n_out, dtype=torch.float32, device=device)
+        lse = torch.empty(m, dtype=torch.float32, device=device)
+        valid_count = torch.empty(1, dtype=torch.float32, device=device)
+        grad_hidden32 = torch.empty((m, h), dtype=torch.float32, device=device)
+        grad_weight32 = (torch.empty((v, h), dtype=torch.float32, device=device)
+                         if compute_weight_grad else None)
+        ws = _workspace(
+            lib.tlce_forward_with_gradients_workspace_bytes(
+                m, h, v, code, int(compute_weight_grad), panel),
+            device,
+        )
+        _lib.check(
+            lib.tlce_forward_with_gradients(
+                _ptr(hidden), _ptr(weight), _ptr(labels), _ptr(row_idx), _ptr(token_weights),
+                m, n_out, h, v, code,
+                int(ignore_index), int(exclude_index), float(logit_softcap),
+                float(logit_multiplier),
+                _ptr(losses), _ptr(lse), valid_count.data_ptr(),
+                _ptr(grad_hidden32), _ptr(grad_weight32),
+                panel, ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_forward_with_gradients",
+        )
+    return losses, lse, valid_count, grad_hidden32, grad_weight32
+
+
+def apply_grad_output(
+    grad_hidden32: torch.Tensor,
+    grad_weight32: torch.Tensor | None,
+    grad_output: torch.Tensor,
+    valid_count: torch.Tensor,
+    *,
+    reduction: str,
+    dtype: torch.dtype,
+    row_idx: torch.Tensor | None = None,
+    n_out: int | None = None,
+    vocab: int | None = None,
+) -> tuple[torch.Tensor, torch.Tensor | None]:
+    """``(grad_hidden [n_out, H], grad_weight [V, H] or None)`` in ``dtype``: the
+    float32 gradients ``forward_with_gradients`` left, times the upstream gradient
+    (over ``valid_count`` for the mean), each entry rounded once."""
+    device = _require_device(grad_hidden32, grad_weight32, grad_output, valid_count, row_idx)
+    reduction_code = _reduction_code(reduction)
+    if reduction_code == _lib.REDUCTION_NONE:
+        raise RuntimeError("apply_grad_output needs a scalar upstream gradient (sum or mean)")
+    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
+    if grad_output.numel() != 1:
+        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected 1")
+    m, h = grad_hidden32.shape
+    v = grad_weight32.shape[0] if grad_weight32 is not None else int(vocab or 1)
+    n_out = m if n_out is None else int(n_out)
+    code = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}[dtype]
+    with torch.cuda.device(device):
+        grad_hidden = torch.empty((n_out, h), dtype=dtype, device=device)
+        grad_weight = (torch.empty((v, h), dtype=dtype, device=device)
+                       if grad_weight32 is not None else None)
+        _lib.check(
+            _lib.library().tlce_apply_grad_output(
+                _ptr(grad_hidden32), _ptr(grad_weight32), _ptr(row_idx), _ptr(grad_output),
+                _ptr(valid_count), m, n_out, h, v, code, reduction_code,
+                _ptr(grad_hidden), _ptr(grad_weight), _stream(device),
+            ),
+            "tlce_apply_grad_output",
+        )
+    return grad_hidden, grad_weight
+
+
 # ------------------------------------------------------------------- backward --
 def _backward(
     hidden, weight, bias, labels, lse, valid_count, grad_output, *,

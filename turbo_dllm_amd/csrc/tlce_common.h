@@ -127,6 +127,31 @@ __device__ __forceinline__ void grouped_tile(int logical, int ni, int nj, int gr
   *tj = within / gsize;
 }
 
+// The same order with the groups along i balanced: ceil(ni / group) groups whose
+// sizes differ by at most one (13 tiles in groups of at most 4: 4, 3, 3, 3 instead
+// of 4, 4, 4, 1), for launches whose ni is small and not a multiple of the group.
+__device__ __forceinline__ void balanced_grouped_tile(int logical, int ni, int nj, int group,
+                                                      int* ti, int* tj) {
+  const int n_groups = (ni + group - 1) / group;
+  const int base = ni / n_groups, extra = ni % n_groups;   // the first `extra` groups hold base + 1
+  const int big = (base + 1) * nj;
+  int first, gsize, within;
+  if (logical < extra * big) {
+    const int g = logical / big;
+    gsize = base + 1;
+    first = g * gsize;
+    within = logical - g * big;
+  } else {
+    const int rest = logical - extra * big;
+    const int g = rest / (base * nj);
+    gsize = base;
+    first = extra * (base + 1) + g * base;
+    within = rest - g * base * nj;
+  }
+  *ti = first + within % gsize;
+  *tj = within / gsize;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }

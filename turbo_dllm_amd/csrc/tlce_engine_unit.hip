@@ -9,8 +9,11 @@
 //                        logit-gradient variants (soft cap, bias, both),
 //                        10, 11: the forward statistics and the logit-gradient
 //                        panels over a head stored [h, v],
+//                        12: the exponentiated-logits panel of the forward that
+//                        leaves the gradients (direct engines only),
 //                        6: the launch sequences over them.
 #include "tlce_host.h"
+#include "tlce_fused.h"
 
 #ifndef TLCE_UNIT_ENGINE
 #error "define TLCE_UNIT_ENGINE and TLCE_UNIT_PART (see turbo_dllm_amd/build.py)"
@@ -73,8 +76,14 @@ TLCE_LAUNCHERS_GRAD_LOGITS_DIM_FIRST(template, UnitEngine)
 #else
 TLCE_LAUNCHERS_GRAD_LOGITS_DIM_FIRST(extern template, UnitEngine)
 #endif
+#if TLCE_UNIT_PART == 12
+TLCE_LAUNCHERS_EXP_PANEL(template, UnitEngine)
+#else
+TLCE_LAUNCHERS_EXP_PANEL(extern template, UnitEngine)
+#endif
 #if TLCE_UNIT_PART == 6
 TLCE_ENGINE_ENTRY_POINTS(template, UnitEngine)
+TLCE_FUSED_ENTRY_POINTS(template, UnitEngine)
 #endif
 #endif
 

@@ -1,0 +1,466 @@
+// Forward that also leaves the gradients: three contractions instead of four.
+//
+// The plain forward keeps no logits, so the backward has to recompute them
+// (ce_grad_logits_kernel works on stored logits, fused_linear_ce_cuda.cu:240-290;
+// the reference's blocks hold float32 logits between its forward and backward
+// halves, :618-791).  When the loss is reduced to a scalar ("mean" / "sum") the
+// upstream gradient is one number, and the gradients of the loss SUM can be
+// formed while the logits of a block of rows exist, then scaled by that number
+// afterwards.  Rows are taken in blocks of as many rows as a bounded panel holds
+// over the WHOLE vocabulary; per block:
+//
+//   1. lce_exp_logits_panel_kernel: one contraction; the panel receives
+//      e[r, v] = exp(z[r, v] - c[r]) * cap'(z) rounded to the input dtype, where
+//      c[r] is a per-row reference logit known beforehand (the label's logit, a
+//      one-row dot product).  Any c within ~80 of the row maximum keeps e inside
+//      the 16-bit formats' exponent range with full relative precision.  The
+//      tile sums of exp(z - c) and the tile maxima go out as per-tile partials.
+//   2. lce_fused_rows_kernel: lse[r] = c[r] + log(sum), loss, the row factor
+//      s[r] = weight[r] / sum (softmax = s * e), the label's panel entry replaced
+//      by (e_label - sum) * cap' so that s * entry = (p_label - 1) * cap', and
+//      hidden rows scaled by s for the grad_weight contraction.  A row whose
+//      maximum lies outside [c - 40, c + 40] marks the block; steps 1-2 are
+//      launched a second time and run only for marked blocks, with c = the exact
+//      row maximum found by the first try (cannot fail again).
+//   3. grad_hidden[r, :] = s[r] * (panel . weight)[r, :]   (K = the vocabulary,
+//      complete for the block: no read-modify-write of a slab across panels)
+//   4. grad_weight += panel^T . (s * hidden)   (float32 accumulator [v, h], one
+//      read-modify-write per block of rows)
+//
+// Both gradients stay float32 until the upstream gradient arrives
+// (lce_scale_cast_rows_kernel), so each is rounded once.
+#pragma once
+
+#include "tlce_host.h"
+
+namespace tlce {
+
+// The row offset beyond which the first try is redone with the exact maximum
+// (natural-log units).  exp(40) ~ 2e17 and its reciprocal are far inside the
+// bf16 / float32 exponent range, also after a multiplication by a hidden entry
+// or a loss weight; f16 panels (max 65504) are kept to +-8.
+// Default bound of the panel of exponentiated logits: 32 token tiles over a
+// 152 K vocabulary in 16-bit.  Per block of rows the grad_weight accumulator
+// [v, h] float32 is read and written once, so fewer, larger blocks cost less
+// (measured at 32768 x 4096 x 151936: 1 GiB 106.7 ms per step, 1.2 GiB 101.5,
+// 2.4 GiB 96.9).
+constexpr int64_t kDefaultFusedPanelBytes = 5ll << 29;
+constexpr float kRefWindowWide = 40.0f;
+constexpr float kRefWindowF16 = 8.0f;
+
+struct ExpPanelArgs {
+  const void* hidden;   // [m, h] the rows of this block
+  const void* weight;   // [v, h]
+  const float* ref;     // [m] reference logit per row (natural units); +inf: row without loss
+  int m, h, v;
+  int64_t exclude;
+  float softcap;
+  float logit_scale;    // logits = cap(logit_scale * hidden . weight^T)
+  int n_ttiles, n_vtiles;
+  void* panel;          // [n_ttiles * tile, ld]
+  int64_t ld;
+  float* part_sum;      // [n_vtiles, part_ld] sum over the tile of exp(z - ref)
+  float* part_max;      // [n_vtiles, part_ld] tile maximum of z in base-2 units
+  int part_ld;
+  const int* run_flag;  // non-null: the launch does nothing unless *run_flag != 0
+};
+
+template <class E, bool kSoftcap>
+__global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPanelArgs p) {
+  extern __shared__ __align__(16) char smem[];
+  using T = typename E::T;
+  static_assert(E::kHasKMajor && sizeof(T) == 2 && E::kCols == 4,
+                "written for the four-wave direct-to-LDS engine");
+  if (p.run_flag != nullptr && *p.run_flag == 0) return;
+  const int logical = xcd_logical_block_of(blockIdx.x, p.n_ttiles * p.n_vtiles);
+  if (logical < 0) return;
+  int tt, vt;
+  balanced_grouped_tile(logical, p.n_ttiles, p.n_vtiles, 4, &tt, &vt);
+
+  E eng;
+  typename E::Acc acc;
+  const int vbase = vt * E::kTile;
+  // reference logit of each owned token column in base-2 units; +inf for rows
+  // past the block and rows without loss, whose whole column of e becomes 0
+  float ref2[E::kCols];
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    const int r = tt * E::kTile + eng.col(j);
+    ref2[j] = (r < p.m) ? p.ref[r] * TLCE_LOG2E : INFINITY;
+  }
+  eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
+                   static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+
+  const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
+  const float to_base2 = kSoftcap ? p.softcap * TLCE_LOG2E : p.logit_scale * TLCE_LOG2E;
+  const bool edge = (vbase + E::kTile > p.v) ||
+                    (p.exclude >= vbase && p.exclude < vbase + E::kTile);
+  const int excluded = (int)p.exclude;
+  float col_sum[E::kCols], col_max[E::kCols];
+  T* panel = static_cast<T*>(p.panel);
+  const int pcol = vt * E::kTile;   // first panel column of this tile
+
+  // The tile is staged in LDS (free after the main loop) as [token][vocab]:
+  // 512-byte rows, 16-byte chunk c of token t in slot c ^ (t & 31), and leaves in
+  // whole rows, a quarter of the tokens (one owned column index) at a time.
+  auto emit = [&](auto edge_tag) {
+    constexpr bool kEdge = decltype(edge_tag)::value;
+    asm volatile("" ::: "memory");   // one real branch per variant
+#pragma unroll
+    for (int j = 0; j < E::kCols; ++j) {
+      const int tok = eng.col(j);
+      float s = 0.0f, mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < E::kRows; i += 4) {
+        float e4[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int row = eng.row(i + q);
+          float z2, dcap = 1.0f;
+          if (kSoftcap) {
+            const float t = tanh_of<E::kPrecise>(E::get(acc, j, i + q) * inv_cap);
+            z2 = t * to_base2;
+            dcap = 1.0f - t * t;
+          } else {
+            z2 = E::get(acc, j, i + q) * to_base2;
+          }
+          float e = exp2_of<E::kPrecise>(z2 - ref2[j]);
+          if (kEdge) {
+            const bool ok = (vbase + row < p.v) && (vbase + row != excluded);
+            e = ok ? e : 0.0f;
+            z2 = ok ? z2 : -INFINITY;
+          }
+          mx = fmaxf(mx, z2);
+          s += e;
+          e4[q] = kSoftcap ? e * dcap : e;
+        }
+        const int vq = eng.row(i) >> 2;
+        T* dst = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
+                                      (vq & 1) * 8);
+        store4<T>(dst, e4[0], e4[1], e4[2], e4[3]);
+      }
+      col_sum[j] = s;
+      col_max[j] = mx;
+      __syncthreads();
+      constexpr int kPieces = E::kTokensPerIndex * 32;   // 16-byte pieces of this quarter
+#pragma unroll
+      for (int it = 0; it < kPieces / E::kThreads; ++it) {
+        const int c = it * E::kThreads + threadIdx.x;
+        const int t = E::token_of_index(j, c >> 5);
+        const int ch = c & 31;
+        const uint4 val = *reinterpret_cast<const uint4*>(smem + t * 512 + ((ch ^ (t & 31)) * 16));
+        stream_store16(panel + ((int64_t)tt * E::kTile + t) * p.ld + pcol + ch * 8, val);
+      }
+    }
+  };
+  if (edge) {
+    emit(std::true_type{});
+  } else {
+    emit(std::false_type{});
+  }
+
+  // merge the kShare threads that hold the same token column, in a fixed order
+  __syncthreads();   // the last quarter has been read out of the stage
+  float* sh_sum = reinterpret_cast<float*>(smem);
+  float* sh_max = sh_sum + E::kShare * E::kTile;
+  const int slot = eng.share_slot();
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) {
+    sh_sum[slot * E::kTile + eng.col(j)] = col_sum[j];
+    sh_max[slot * E::kTile + eng.col(j)] = col_max[j];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < E::kTile; c += E::kThreads) {
+    float sum = 0.0f, mx = -INFINITY;
+#pragma unroll
+    for (int sl = 0; sl < E::kShare; ++sl) {
+      sum += sh_sum[sl * E::kTile + c];
+      mx = fmaxf(mx, sh_max[sl * E::kTile + c]);
+    }
+    const int64_t o = (int64_t)vt * p.part_ld + tt * E::kTile + c;
+    p.part_sum[o] = sum;
+    p.part_max[o] = mx;
+  }
+}
+
+template <class E, bool kSoftcap>
+int launch_exp_panel_variant(const ExpPanelArgs& a, hipStream_t stream) {
+  static LdsOptIn lds;
+  if (int rc = enable_large_lds(lce_exp_logits_panel_kernel<E, kSoftcap>, E::kSmemBytes, lds))
+    return rc;
+  const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_vtiles);
+  ScopedTimer timer(kClassExpPanel, stream);
+  lce_exp_logits_panel_kernel<E, kSoftcap><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------------------------------- row kernels --
+// (engine-independent; compiled beside the C ABI, reached through launch_*)
+
+// Before the blocks: the label's logit of every row by a one-row dot product,
+// which is both the loss's target term and the reference logit of the row.
+struct LabelLogitArgs {
+  const void* hidden;   // [m, h]
+  const void* weight;   // [v, h]
+  const int64_t* labels;
+  int m, h, v;
+  int64_t ignore, exclude;
+  float softcap, logit_scale;
+  float* target;        // [m] cap(scale * h . w[label]); 0 when the label has no logit
+  float* ref;           // [m] reference logit; +inf for rows without loss
+  float* valid_count;   // [1] += rows with a label other than `ignore`
+  int dtype;
+};
+
+struct FusedRowsArgs {
+  const void* hidden;          // [m, h] rows of the block
+  const int64_t* labels;       // [m]
+  const float* ref;            // [m] the reference the panel was produced with
+  const float* target;         // [m]
+  const float* token_weights;  // [m] or null
+  const int64_t* row_idx;      // [m] or null: where the row's loss goes
+  int64_t loss_row0;           // row_idx == null: index of the block's first row in `losses`
+  const float* part_sum;
+  const float* part_max;
+  int part_ld, n_vtiles;
+  int m, m_pad;                // rows of the block; rows of `scaled_hidden` to define (zeros past m)
+  int h, v;
+  int64_t ignore, exclude;
+  float softcap, logit_scale, window;
+  void* panel;                 // [.., ld]
+  int64_t ld;
+  float* lse;                  // [m]
+  float* losses;               // scattered, or null
+  float* row_scale;            // [m_pad]
+  void* scaled_hidden;         // [m_pad, h] or null (no grad_weight)
+  float* ref_next;             // [m] reference of the second try
+  int* redo;                   // [1] set when some row needs the second try
+  const int* run_flag;         // non-null: run only when *run_flag != 0
+  int dtype;
+};
+
+// grad_hidden32[r, :] = row_scale[r] * sum over K splits of slab[s][r, :]
+struct ReduceSlabsArgs {
+  const float* slabs;
+  int n_splits;
+  int64_t split_stride;
+  const float* row_scale;
+  int m, h;
+  float* out;   // [m, h]
+};
+
+// out[row_idx[r], :] = dtype(g * in[r, :]) with g = grad_output[0] (/ valid_count[0]
+// for the mean): the upstream gradient applied to the float32 gradients the
+// forward left, rounding each entry once.
+struct ScaleCastArgs {
+  const float* in;          // [rows, h]
+  const int64_t* row_idx;   // or null
+  const float* grad_output; // [1]
+  const float* valid_count; // [1], read for the mean reduction only
+  int reduction;
+  int64_t rows;
+  int h;
+  void* out;
+  int dtype;
+};
+
+int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream);
+int launch_fused_rows(const FusedRowsArgs& a, hipStream_t stream);
+int launch_reduce_slabs(const ReduceSlabsArgs& a, hipStream_t stream);
+int launch_scale_cast(const ScaleCastArgs& a, hipStream_t stream);
+
+// ------------------------------------------------------------------- plan ----
+struct FusedPlan {
+  int64_t vp;           // panel columns: the vocabulary rounded up to whole tiles
+  int n_vtiles, n_htiles;
+  int64_t block_rows;   // rows per block, a multiple of the tile
+  int n_blocks;
+  int dh_ksplit;        // K splits of the grad_hidden contraction of a full block
+};
+
+inline bool fused_gradients_supported(int64_t h, int64_t v, int dtype) {
+  return engine_class(h, dtype) == 2 && (v % 64) == 0;
+}
+
+inline FusedPlan make_fused_plan(int64_t m, int64_t h, int64_t v, int dtype, int64_t panel_bytes) {
+  FusedPlan p;
+  const int64_t tile = 256;
+  p.vp = round_up(v, tile);
+  p.n_vtiles = (int)(p.vp / tile);
+  p.n_htiles = (int)ceil_div(h, tile);
+  if (panel_bytes <= 0) panel_bytes = kDefaultFusedPanelBytes;
+  const int64_t total = ceil_div(std::max<int64_t>(m, 1), tile);   // token tiles
+  const int64_t budget =
+      std::max<int64_t>(1, panel_bytes / (p.vp * dtype_bytes(dtype) * tile));
+  p.n_blocks = (int)ceil_div(total, budget);
+  int64_t per = ceil_div(total, p.n_blocks);   // balanced blocks
+  // several blocks: 16 token tiles x 16 hidden tiles make whole rounds of 256
+  // workgroups in the grad_hidden contraction
+  if (p.n_blocks > 1 && round_up(per, 16) <= budget) per = round_up(per, 16);
+  p.block_rows = per * tile;
+  p.n_blocks = (int)ceil_div(total, per);
+  const int64_t k_steps = p.vp / 64;
+  const int max_split = (int)std::max<int64_t>(1, std::min<int64_t>(16, k_steps / 8));
+  p.dh_ksplit = grad_hidden_k_splits((p.block_rows / tile) * p.n_htiles, max_split, k_steps,
+                                     p.block_rows * h);
+  return p;
+}
+
+struct FusedLayout {
+  int64_t panel, part_sum, part_max, target, ref, ref_next, row_scale, scaled_hidden, slabs,
+      redo, total;
+};
+
+inline FusedLayout fused_layout(const FusedPlan& p, int64_t m, int64_t h, int dtype,
+                                bool weight_grad) {
+  FusedLayout l;
+  const int64_t es = dtype_bytes(dtype);
+  const int64_t mp = round_up(std::max<int64_t>(m, 1), 256);
+  int64_t off = 0;
+  l.panel = off;      off += align256(p.block_rows * p.vp * es);
+  l.part_sum = off;   off += align256((int64_t)p.n_vtiles * p.block_rows * 4);
+  l.part_max = off;   off += align256((int64_t)p.n_vtiles * p.block_rows * 4);
+  l.target = off;     off += align256(mp * 4);
+  l.ref = off;        off += align256(mp * 4);
+  l.ref_next = off;   off += align256(p.block_rows * 4);
+  l.row_scale = off;  off += align256(p.block_rows * 4);
+  l.scaled_hidden = off;
+  if (weight_grad) off += align256(p.block_rows * h * es);
+  l.slabs = off;      off += align256((int64_t)p.dh_ksplit * p.block_rows * h * 4);
+  l.redo = off;       off += align256((int64_t)p.n_blocks * 4);
+  l.total = off;
+  return l;
+}
+
+// Options of the fused sequence beyond the operator's own arguments.
+struct FusedOptions {
+  float logit_scale = 1.0f;
+  const float* token_weights = nullptr;   // [m] per-row loss weights or null
+};
+
+template <class E>
+int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* weight,
+                         const int64_t* labels, const int64_t* row_idx, int64_t m, int64_t h,
+                         int64_t v, int dtype, int64_t ignore, int64_t exclude, float softcap,
+                         float* losses, float* lse, float* valid_count, float* grad_hidden32,
+                         float* grad_weight32, char* ws, hipStream_t stream,
+                         const FusedOptions& opt) {
+  using T = typename E::T;
+  const bool weight_grad = grad_weight32 != nullptr;
+  const FusedLayout l = fused_layout(p, m, h, dtype, weight_grad);
+  T* panel = reinterpret_cast<T*>(ws + l.panel);
+  float* part_sum = reinterpret_cast<float*>(ws + l.part_sum);
+  float* part_max = reinterpret_cast<float*>(ws + l.part_max);
+  float* target = reinterpret_cast<float*>(ws + l.target);
+  float* ref = reinterpret_cast<float*>(ws + l.ref);
+  float* ref_next = reinterpret_cast<float*>(ws + l.ref_next);
+  float* row_scale = reinterpret_cast<float*>(ws + l.row_scale);
+  T* scaled_hidden = weight_grad ? reinterpret_cast<T*>(ws + l.scaled_hidden) : nullptr;
+  float* slabs = reinterpret_cast<float*>(ws + l.slabs);
+  int* redo = reinterpret_cast<int*>(ws + l.redo);
+  const T* hidden_t = static_cast<const T*>(hidden);
+
+  if (int rc = fill_zero(redo, (int64_t)p.n_blocks * 4, stream)) return rc;
+  LabelLogitArgs la;
+  la.hidden = hidden; la.weight = weight; la.labels = labels;
+  la.m = (int)m; la.h = (int)h; la.v = (int)v;
+  la.ignore = ignore; la.exclude = exclude; la.softcap = softcap; la.logit_scale = opt.logit_scale;
+  la.target = target; la.ref = ref; la.valid_count = valid_count; la.dtype = dtype;
+  if (int rc = launch_label_logit(la, stream)) return rc;
+
+  for (int block = 0; block < p.n_blocks; ++block) {
+    const int64_t r0 = (int64_t)block * p.block_rows;
+    const int64_t rows = std::min<int64_t>(p.block_rows, m - r0);
+    if (rows <= 0) break;
+    const int n_ttiles = (int)ceil_div(rows, E::kTile);
+    const int64_t rows_p = (int64_t)n_ttiles * E::kTile;
+    const int64_t rows64 = round_up(rows, 64);
+
+    ExpPanelArgs ea;
+    ea.hidden = hidden_t + r0 * h; ea.weight = weight;
+    ea.m = (int)rows; ea.h = (int)h; ea.v = (int)v;
+    ea.exclude = exclude; ea.softcap = softcap; ea.logit_scale = opt.logit_scale;
+    ea.n_ttiles = n_ttiles; ea.n_vtiles = p.n_vtiles;
+    ea.panel = panel; ea.ld = p.vp;
+    ea.part_sum = part_sum; ea.part_max = part_max; ea.part_ld = (int)p.block_rows;
+
+    FusedRowsArgs ra;
+    ra.hidden = hidden_t + r0 * h; ra.labels = labels + r0;
+    ra.target = target + r0;
+    ra.token_weights = opt.token_weights ? opt.token_weights + r0 : nullptr;
+    ra.row_idx = row_idx ? row_idx + r0 : nullptr; ra.loss_row0 = r0;
+    ra.part_sum = part_sum; ra.part_max = part_max;
+    ra.part_ld = (int)p.block_rows; ra.n_vtiles = p.n_vtiles;
+    ra.m = (int)rows; ra.m_pad = (int)rows_p; ra.h = (int)h; ra.v = (int)v;
+    ra.ignore = ignore; ra.exclude = exclude; ra.softcap = softcap;
+    ra.logit_scale = opt.logit_scale;
+    ra.window = (dtype == TLCE_DTYPE_F16) ? kRefWindowF16 : kRefWindowWide;
+    ra.panel = panel; ra.ld = p.vp;
+    ra.lse = lse + r0; ra.losses = losses;
+    ra.row_scale = row_scale; ra.scaled_hidden = scaled_hidden;
+    ra.ref_next = ref_next; ra.redo = redo + block; ra.dtype = dtype;
+
+    for (int attempt = 0; attempt < 2; ++attempt) {
+      ea.ref = attempt ? ref_next : ref + r0;
+      ea.run_flag = attempt ? redo + block : nullptr;
+      if (softcap > 0.0f) {
+        if (int rc = launch_exp_panel_variant<E, true>(ea, stream)) return rc;
+      } else {
+        if (int rc = launch_exp_panel_variant<E, false>(ea, stream)) return rc;
+      }
+      ra.ref = ea.ref;
+      ra.run_flag = ea.run_flag;
+      // the second try must not mark the block again: it reads the flag the first set
+      if (int rc = launch_fused_rows(ra, stream)) return rc;
+    }
+
+    // grad_hidden of the block: A = weight as stored (K-major, K = vocabulary), B = panel
+    GemmArgs dh;
+    dh.a = weight; dh.lda = h; dh.a_rows = (int)h;
+    dh.b = panel; dh.ldb = p.vp; dh.b_rows = (int)rows_p;
+    dh.k = (int)round_up(v, 64);
+    dh.k_per_split = 0;
+    dh.ni = p.n_htiles; dh.nj = n_ttiles;
+    dh.c = slabs; dh.ldc = h; dh.c_rows = (int)rows_p; dh.c_cols = (int)h;
+    dh.c_split_stride = p.block_rows * h;
+    dh.mode = kStoreF32;
+    const int ksplit = (rows_p == p.block_rows)
+                           ? p.dh_ksplit
+                           : std::min(p.dh_ksplit,
+                                      grad_hidden_k_splits((int64_t)n_ttiles * p.n_htiles,
+                                                           p.dh_ksplit, p.vp / 64, rows_p * h));
+    if (int rc = launch_gemm<E, true, false>(dh, ksplit, kClassGradHidden, stream)) return rc;
+    ReduceSlabsArgs rs;
+    rs.slabs = slabs; rs.n_splits = ksplit; rs.split_stride = p.block_rows * h;
+    rs.row_scale = row_scale; rs.m = (int)rows; rs.h = (int)h;
+    rs.out = grad_hidden32 + r0 * h;
+    if (int rc = launch_reduce_slabs(rs, stream)) return rc;
+
+    if (weight_grad) {
+      // grad_weight += panel^T . (s * hidden): both operands K-major, K = the block's rows
+      GemmArgs dw;
+      dw.a = scaled_hidden; dw.lda = h; dw.a_rows = (int)h;
+      dw.b = panel; dw.ldb = p.vp; dw.b_rows = (int)p.vp;
+      dw.k = (int)rows64;
+      dw.k_per_split = 0;
+      dw.ni = p.n_htiles; dw.nj = p.n_vtiles;
+      dw.c = grad_weight32; dw.ldc = h; dw.c_rows = (int)v; dw.c_cols = (int)h;
+      dw.c_split_stride = 0;
+      dw.mode = block == 0 ? kStoreF32 : kAddF32;
+      if (int rc = launch_gemm<E, true, true>(dw, 1, kClassGradWeight, stream)) return rc;
+    }
+  }
+  return 0;
+}
+
+#define TLCE_LAUNCHERS_EXP_PANEL(X, E)                                            \
+  X int launch_exp_panel_variant<E, false>(const ExpPanelArgs&, hipStream_t);     \
+  X int launch_exp_panel_variant<E, true>(const ExpPanelArgs&, hipStream_t);
+#define TLCE_FUSED_ENTRY_POINTS(X, E)                                                            \
+  X int fused_gradients_impl<E>(const FusedPlan&, const void*, const void*, const int64_t*,      \
+                                const int64_t*, int64_t, int64_t, int64_t, int, int64_t,         \
+                                int64_t, float, float*, float*, float*, float*, float*, char*,   \
+                                hipStream_t, const FusedOptions&);
+
+}  // namespace tlce

@@ -1,0 +1,168 @@
+// Row kernels of the forward that leaves the gradients (tlce_fused.h): the
+// label-logit pass before the blocks, the per-block statistics / row-factor pass,
+// the K-split reduction of grad_hidden and the final scale-and-cast.  Engine
+// independent; compiled beside the C ABI.
+#pragma once
+
+#include "tlce_fused.h"
+
+namespace tlce {
+
+// One wave per row, 16 rows per workgroup (one atomic per workgroup for the count
+// of rows with a loss).
+template <typename T>
+__global__ __launch_bounds__(256) void lce_label_logit_kernel(LabelLogitArgs p) {
+  __shared__ int block_valid;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) block_valid = 0;
+  __syncthreads();
+  int wave_valid = 0;
+  for (int i = 0; i < 4; ++i) {
+    const int r = blockIdx.x * 16 + wave * 4 + i;
+    if (r >= p.m) continue;
+    const int64_t label = p.labels[r];
+    const bool valid = label != p.ignore;
+    const bool here = valid && label >= 0 && label < p.v;
+    float z = 0.0f;
+    if (here) {
+      const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
+      const T* wrow = static_cast<const T*>(p.weight) + label * (int64_t)p.h;
+      z = wave_dot<T>(hrow, wrow, p.h, lane) * p.logit_scale;
+      if (p.softcap > 0.0f) z = p.softcap * tanhf(z / p.softcap);
+    }
+    if (lane == 0) {
+      // a label on the excluded column or outside the vocabulary has no logit in the
+      // loss (ce_forward_kernel, fused_linear_ce_cuda.cu:199-219); as a reference any
+      // real column's logit serves
+      p.target[r] = (here && label != p.exclude) ? z : 0.0f;
+      p.ref[r] = valid ? z : INFINITY;
+    }
+    wave_valid += valid ? 1 : 0;
+  }
+  if (lane == 0 && wave_valid != 0) atomicAdd(&block_valid, wave_valid);
+  __syncthreads();
+  if (threadIdx.x == 0 && block_valid != 0) atomicAdd(p.valid_count, (float)block_valid);
+}
+
+// 64 rows per workgroup.  First the per-tile partials of the 64 rows are added up
+// with the rows across the lanes (coalesced: partials are stored [tile][row]), each
+// quarter of the workgroup taking every fourth vocabulary tile in order and the
+// four quarter sums merged in a fixed order; then each wave finishes 16 rows (rows
+// past m only get their zero row of scaled_hidden and a zero row factor).
+constexpr int kFusedRowsPerBlock = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void lce_fused_rows_kernel(FusedRowsArgs p) {
+  if (p.run_flag != nullptr && *p.run_flag == 0) return;
+  __shared__ float sh_sum[4][kFusedRowsPerBlock];
+  __shared__ float sh_max[4][kFusedRowsPerBlock];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int row0 = blockIdx.x * kFusedRowsPerBlock;
+  {
+    const int r = row0 + lane;
+    float sum = 0.0f, mx2 = -INFINITY;
+    if (r < p.m) {
+      for (int t = wave; t < p.n_vtiles; t += 4) {
+        sum += p.part_sum[(int64_t)t * p.part_ld + r];
+        mx2 = fmaxf(mx2, p.part_max[(int64_t)t * p.part_ld + r]);
+      }
+    }
+    sh_sum[wave][lane] = sum;
+    sh_max[wave][lane] = mx2;
+  }
+  __syncthreads();
+  T* scaled = static_cast<T*>(p.scaled_hidden);
+  for (int i = 0; i < kFusedRowsPerBlock / 4; ++i) {
+    const int rr = wave * (kFusedRowsPerBlock / 4) + i;
+    const int r = row0 + rr;
+    if (r >= p.m_pad) return;
+    float factor = 0.0f;
+    if (r < p.m) {
+      const float c = p.ref[r];
+      const bool live = c < INFINITY;   // rows without loss carry +inf
+      const float sum = ((sh_sum[0][rr] + sh_sum[1][rr]) + sh_sum[2][rr]) + sh_sum[3][rr];
+      const float mx = fmaxf(fmaxf(sh_max[0][rr], sh_max[1][rr]),
+                             fmaxf(sh_max[2][rr], sh_max[3][rr])) * TLCE_LN2;
+      const bool in_window = (mx - c <= p.window) && (mx - c >= -1.0f) && (sum > 0.0f) &&
+                             (sum < 3.0e38f);
+      const float lse = live ? c + logf(sum) : 0.0f;
+      const float target = p.target[r];
+      const float w = (p.token_weights != nullptr) ? p.token_weights[r] : 1.0f;
+      const int64_t label = p.labels[r];
+      if (live) factor = w * p.logit_scale / sum;
+      if (lane == 0) {
+        p.lse[r] = lse;
+        if (p.losses != nullptr) {
+          const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : p.loss_row0 + r;
+          p.losses[o] = live ? lse - target : 0.0f;
+        }
+        p.ref_next[r] = (live && !in_window) ? mx : c;
+        if (live && !in_window) atomicOr(p.redo, 1);
+        // the label's entry: s * entry = (softmax - 1) * cap'
+        if (live && label >= 0 && label < p.v && label != p.exclude) {
+          float dcap = 1.0f;
+          if (p.softcap > 0.0f) {
+            const float t = target / p.softcap;
+            dcap = 1.0f - t * t;
+          }
+          const float entry = (expf(target - c) - sum) * dcap;
+          static_cast<T*>(p.panel)[(int64_t)r * p.ld + label] = from_float<T>(entry);
+        }
+        p.row_scale[r] = factor;
+      }
+    } else if (lane == 0) {
+      p.row_scale[r] = 0.0f;
+    }
+    if (scaled != nullptr) {
+      const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)min(r, p.m - 1) * p.h;
+      T* out = scaled + (int64_t)r * p.h;
+      if ((p.h % 8) == 0) {
+        typedef T v8_t __attribute__((ext_vector_type(8)));
+        for (int k = lane * 8; k < p.h; k += 64 * 8) {
+          const v8_t x = *reinterpret_cast<const v8_t*>(hrow + k);
+          v8_t y;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) y[e] = from_float<T>(to_float<T>(x[e]) * factor);
+          *reinterpret_cast<v8_t*>(out + k) = y;
+        }
+      } else {
+        for (int k = lane; k < p.h; k += 64) out[k] = from_float<T>(to_float<T>(hrow[k]) * factor);
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void lce_reduce_scaled_slabs_kernel(ReduceSlabsArgs p) {
+  const int r = blockIdx.x;
+  const float s = p.row_scale[r];
+  const float* src = p.slabs + (int64_t)r * p.h;
+  float* dst = p.out + (int64_t)r * p.h;
+  for (int k = threadIdx.x * 4; k < p.h; k += 256 * 4) {
+    f32x4_t sum = *reinterpret_cast<const f32x4_t*>(src + k);
+    for (int q = 1; q < p.n_splits; ++q)
+      sum += *reinterpret_cast<const f32x4_t*>(src + (int64_t)q * p.split_stride + k);
+    *reinterpret_cast<f32x4_t*>(dst + k) = sum * s;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void lce_scale_cast_rows_kernel(ScaleCastArgs p) {
+  float g = p.grad_output[0];
+  if (p.reduction == TLCE_REDUCTION_MEAN) {
+    // no row with a loss: every gradient entry is zero and stays zero
+    const float count = p.valid_count[0];
+    g = count > 0.0f ? g / count : 0.0f;
+  }
+  const int64_t r = blockIdx.x;
+  const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : r;
+  const float* src = p.in + r * p.h;
+  T* dst = static_cast<T*>(p.out) + o * p.h;
+  for (int k = threadIdx.x * 4; k < p.h; k += 256 * 4) {
+    const f32x4_t x = *reinterpret_cast<const f32x4_t*>(src + k);
+    store4<T>(dst + k, x[0] * g, x[1] * g, x[2] * g, x[3] * g);
+  }
+}
+
+}  // namespace tlce

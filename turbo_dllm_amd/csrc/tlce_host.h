@@ -44,7 +44,8 @@ enum KernelClass {
   kClassGradWeight = 4,
   kClassTranspose = 5,
   kClassOther = 6,
-  kNumClasses = 7
+  kClassExpPanel = 7,
+  kNumClasses = 8
 };
 
 struct Profiler {

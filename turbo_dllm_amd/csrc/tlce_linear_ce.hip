@@ -5,6 +5,7 @@
 // kernels that do not depend on an engine (tlce_row_kernels.h).
 #include "tlce_host.h"
 #include "tlce_row_kernels.h"
+#include "tlce_fused_rows.h"
 
 namespace tlce {
 
@@ -65,6 +66,48 @@ int launch_sum(const float* x, int64_t n, float* out, hipStream_t stream) {
   return 0;
 }
 
+// ---- row kernels of the forward that leaves the gradients (tlce_fused_rows.h) ----
+#define TLCE_BY_16BIT_DTYPE(dtype, CALL)                          \
+  do {                                                            \
+    if ((dtype) == TLCE_DTYPE_BF16) { using T = __bf16; CALL; }   \
+    else { using T = _Float16; CALL; }                            \
+  } while (0)
+
+int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassCombine, stream);
+  TLCE_BY_16BIT_DTYPE(a.dtype,
+                      (lce_label_logit_kernel<T><<<(int)ceil_div(a.m, 16), 256, 0, stream>>>(a)));
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_fused_rows(const FusedRowsArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassCombine, stream);
+  TLCE_BY_16BIT_DTYPE(
+      a.dtype, (lce_fused_rows_kernel<T><<<(int)ceil_div(a.m_pad, kFusedRowsPerBlock), 256, 0,
+                                           stream>>>(a)));
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_reduce_slabs(const ReduceSlabsArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_reduce_scaled_slabs_kernel<<<a.m, 256, 0, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_scale_cast(const ScaleCastArgs& a, hipStream_t stream) {
+  if (a.rows <= 0) return 0;
+  ScopedTimer timer(kClassOther, stream);
+  TLCE_BY_16BIT_DTYPE(a.dtype,
+                      (lce_scale_cast_rows_kernel<T><<<(unsigned)a.rows, 256, 0, stream>>>(a)));
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+TLCE_FUSED_ENTRY_POINTS(extern template, MfmaDirect4Engine<__bf16>)
+TLCE_FUSED_ENTRY_POINTS(extern template, MfmaDirect4Engine<_Float16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaDirect4Engine<__bf16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaDirect4Engine<_Float16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaEngine<__bf16>)
@@ -640,6 +683,127 @@ extern "C" int tlce_segment_weighted_sum(const float* values, const float* weigh
   lce_segment_weighted_sum_kernel<<<(int)n_segments, 256, 0, stream>>>(
       values, weights, row_idx, row_count, m, segment_length, out);
   TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+// ------------------------------------ forward that leaves the gradients ----
+extern "C" int tlce_fused_gradients_supported(int64_t h, int64_t v, int dtype) {
+  return (h > 0 && v > 0 && fused_gradients_supported(h, v, dtype)) ? 1 : 0;
+}
+
+extern "C" int tlce_query_fused_plan(int64_t m, int64_t h, int64_t v, int dtype,
+                                     int64_t panel_bytes, int64_t* block_rows, int* n_blocks,
+                                     int* grad_hidden_k_splits) {
+  TLCE_REQUIRE(m >= 0 && h > 0 && v > 0, "query_fused_plan: bad shape");
+  TLCE_REQUIRE(fused_gradients_supported(h, v, dtype),
+               "query_fused_plan: needs 16-bit inputs with h and v multiples of 64");
+  const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
+  if (block_rows) *block_rows = p.block_rows;
+  if (n_blocks) *n_blocks = p.n_blocks;
+  if (grad_hidden_k_splits) *grad_hidden_k_splits = p.dh_ksplit;
+  return 0;
+}
+
+extern "C" int64_t tlce_forward_with_gradients_workspace_bytes(int64_t m, int64_t h, int64_t v,
+                                                               int dtype, int compute_weight_grad,
+                                                               int64_t panel_bytes) {
+  if (m < 0 || h <= 0 || v <= 0 || !fused_gradients_supported(h, v, dtype)) return -1;
+  return fused_layout(make_fused_plan(m, h, v, dtype, panel_bytes), m, h, dtype,
+                      compute_weight_grad != 0).total;
+}
+
+extern "C" int tlce_forward_with_gradients(
+    const void* hidden, const void* weight, const int64_t* labels, const int64_t* row_idx,
+    const float* token_weights, int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
+    int64_t ignore_index, int64_t exclude_index, float logit_softcap, float logit_multiplier,
+    float* losses, float* lse, float* valid_count, float* grad_hidden_f32, float* grad_weight_f32,
+    int64_t panel_bytes, void* workspace, int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
+  TLCE_REQUIRE(fused_gradients_supported(h, v, dtype),
+               "forward_with_gradients: needs 16-bit inputs with h and v multiples of 64 "
+               "(h=%lld v=%lld dtype=%d)", (long long)h, (long long)v, dtype);
+  TLCE_REQUIRE(valid_count != nullptr, "forward_with_gradients: valid_count is null");
+  TLCE_REQUIRE(logit_multiplier > 0.0f,
+               "forward_with_gradients: the logit multiplier must be positive");
+  TLCE_REQUIRE(n_out >= m, "forward_with_gradients: n_out=%lld < m=%lld", (long long)n_out,
+               (long long)m);
+  TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
+               "forward_with_gradients: n_out != m without row_idx");
+  TLCE_REQUIRE(((uintptr_t)grad_hidden_f32 & 15) == 0 && ((uintptr_t)grad_weight_f32 & 15) == 0,
+               "forward_with_gradients: gradients must be 16-byte aligned");
+  if (int rc = fill_zero(valid_count, 4, stream)) return rc;
+  if (losses != nullptr && (row_idx != nullptr || m == 0)) {
+    if (int rc = fill_zero(losses, n_out * 4, stream)) return rc;
+  }
+  if (m == 0) {
+    if (grad_weight_f32 != nullptr) return fill_zero(grad_weight_f32, v * h * 4, stream);
+    return 0;
+  }
+  TLCE_REQUIRE(labels && lse && grad_hidden_f32 && workspace,
+               "forward_with_gradients: null pointer");
+  const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
+  const int64_t need = fused_layout(p, m, h, dtype, grad_weight_f32 != nullptr).total;
+  TLCE_REQUIRE(workspace_bytes >= need,
+               "forward_with_gradients: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+               "forward_with_gradients: workspace must be 256-byte aligned");
+  FusedOptions opt;
+  opt.logit_scale = logit_multiplier;
+  opt.token_weights = token_weights;
+  if (dtype == TLCE_DTYPE_BF16) {
+    return fused_gradients_impl<MfmaDirect4Engine<__bf16>>(
+        p, hidden, weight, labels, row_idx, m, h, v, dtype, ignore_index, exclude_index,
+        logit_softcap, losses, lse, valid_count, grad_hidden_f32, grad_weight_f32,
+        static_cast<char*>(workspace), stream, opt);
+  }
+  return fused_gradients_impl<MfmaDirect4Engine<_Float16>>(
+      p, hidden, weight, labels, row_idx, m, h, v, dtype, ignore_index, exclude_index,
+      logit_softcap, losses, lse, valid_count, grad_hidden_f32, grad_weight_f32,
+      static_cast<char*>(workspace), stream, opt);
+}
+
+extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float* grad_weight_f32,
+                                      const int64_t* row_idx, const float* grad_output,
+                                      const float* valid_count, int64_t m, int64_t n_out,
+                                      int64_t h, int64_t v, int dtype, int reduction_code,
+                                      void* grad_hidden, void* grad_weight, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  TLCE_REQUIRE(dtype == TLCE_DTYPE_BF16 || dtype == TLCE_DTYPE_F16,
+               "apply_grad_output: unsupported dtype code %d", dtype);
+  TLCE_REQUIRE(m >= 0 && h > 0 && v > 0 && (h % 4) == 0, "apply_grad_output: bad shape");
+  TLCE_REQUIRE(reduction_code == TLCE_REDUCTION_SUM || reduction_code == TLCE_REDUCTION_MEAN,
+               "apply_grad_output: the upstream gradient must be a scalar (sum or mean)");
+  TLCE_REQUIRE(n_out >= m, "apply_grad_output: n_out=%lld < m=%lld", (long long)n_out,
+               (long long)m);
+  TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
+               "apply_grad_output: n_out != m without row_idx");
+  TLCE_REQUIRE(grad_hidden != nullptr || n_out == 0, "apply_grad_output: grad_hidden is null");
+  TLCE_REQUIRE(grad_output != nullptr, "apply_grad_output: grad_output is null");
+  TLCE_REQUIRE(valid_count != nullptr || reduction_code != TLCE_REDUCTION_MEAN,
+               "apply_grad_output: the mean reduction needs valid_count");
+  TLCE_REQUIRE((grad_weight == nullptr) == (grad_weight_f32 == nullptr),
+               "apply_grad_output: grad_weight and its float32 source go together");
+  TLCE_REQUIRE((((uintptr_t)grad_hidden | (uintptr_t)grad_weight | (uintptr_t)grad_hidden_f32 |
+                 (uintptr_t)grad_weight_f32) & 15) == 0,
+               "apply_grad_output: gradients must be 16-byte aligned");
+  const int64_t es = dtype_bytes(dtype);
+  if (row_idx != nullptr || m == 0) {
+    if (int rc = fill_zero(grad_hidden, n_out * h * es, stream)) return rc;
+  }
+  ScaleCastArgs a;
+  a.grad_output = grad_output; a.valid_count = valid_count; a.reduction = reduction_code;
+  a.h = (int)h; a.dtype = dtype;
+  if (m > 0) {
+    TLCE_REQUIRE(grad_hidden_f32 != nullptr, "apply_grad_output: null pointer");
+    a.in = grad_hidden_f32; a.row_idx = row_idx; a.rows = m; a.out = grad_hidden;
+    if (int rc = launch_scale_cast(a, stream)) return rc;
+  }
+  if (grad_weight != nullptr) {
+    a.in = grad_weight_f32; a.row_idx = nullptr; a.rows = v; a.out = grad_weight;
+    if (int rc = launch_scale_cast(a, stream)) return rc;
+  }
   return 0;
 }
 

@@ -28,7 +28,7 @@ import torch
 from torch import nn
 
 from .compaction import compact_valid_loss_rows, gather_rows
-from .options import resolve_compaction
+from .options import get_gradient_mode, resolve_compaction
 from .tiled_linear_cross_entropy import tiled_linear_cross_entropy
 
 _DEVICE_DTYPES = (torch.float16, torch.bfloat16, torch.float32)
@@ -64,6 +64,27 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
 
         rows, targets, token_weights, row_idx, row_count, m = native.compact_loss_rows(
             hidden_flat, labels_flat, weights_flat, -100, mode)
+        # gradients while the logits exist (3 contractions instead of 4), where the
+        # library takes the operands and the row count is known to the host
+        ctx.fused = (
+            bool(ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) and mode != "device"
+            and get_gradient_mode() == "forward"
+            and native.fused_gradients_supported(rows, weight, bias, False)
+        )
+        if ctx.fused:
+            losses, _, valid_count, grad_rows32, grad_weight32 = native.forward_with_gradients(
+                rows[:m], weight, targets[:m], ignore_index=-100, exclude_index=exclude_index,
+                logit_softcap=logit_softcap, compute_weight_grad=bool(ctx.needs_input_grad[1]),
+                token_weights=None if token_weights is None else token_weights[:m],
+                logit_multiplier=multiplier,
+                row_idx=row_idx, n_out=n,
+            )
+            ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx)
+            ctx.hidden_shape = hidden.shape
+            ctx.n_rows, ctx.m = n, m
+            ctx.grad_dtype, ctx.vocab = hidden.dtype, weight.shape[0]
+            # losses holds the unweighted token losses at their positions, zeros elsewhere
+            return torch.dot(losses, weights_flat)
         _, lse, _, weighted_sum = native.masked_loss_forward(
             rows, weight, bias, targets, token_weights, m=m, row_idx=row_idx,
             row_count=row_count, n_out=n, ignore_index=-100, exclude_index=exclude_index,
@@ -81,6 +102,13 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
     def backward(ctx, grad_output):  # type: ignore[override]
         from . import chunked_linear_ce_native as native
 
+        if ctx.fused:
+            grad_rows32, grad_weight32, valid_count, row_idx = ctx.saved_tensors
+            grad_hidden, grad_weight = native.apply_grad_output(
+                grad_rows32, grad_weight32, grad_output, valid_count, reduction="sum",
+                dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows, vocab=ctx.vocab,
+            )
+            return (grad_hidden.reshape(ctx.hidden_shape), grad_weight, None) + (None,) * 6
         rows, weight, bias, targets, token_weights, lse, row_idx, row_count = ctx.saved_tensors
         with native.panel_budget(ctx.panel_bytes):
             grad_hidden, grad_weight, grad_bias = native.masked_loss_backward(

@@ -1,8 +1,10 @@
 """Context-local options of the device path.
 
-Two settings steer how the HIP library is driven: how rows whose label is
-``ignore_index`` are compacted away, and how many bytes the backward's staging
-panel of rounded logit gradients may take.  Both are ``contextvars``: a value
+Three settings steer how the HIP library is driven: how rows whose label is
+``ignore_index`` are compacted away, how many bytes the staging panel between
+the contractions may take, and whether the gradients are formed during the
+forward (three contractions) or by a backward that recomputes the logits
+(four).  All are ``contextvars``: a value
 set with the context managers below (or passed per call where a function takes
 the keyword) is seen by the calling thread / task only, so two trainers in one
 process can choose differently.  The reference's extension has no such
@@ -32,6 +34,47 @@ COMPACTION_MODES = ("sync", "device", "none")
 _compaction = contextvars.ContextVar("tlce_compaction_mode", default="sync")
 # 0 selects the library default (1 GiB)
 _panel_bytes = contextvars.ContextVar("tlce_panel_bytes", default=0)
+
+
+# When the gradients of a scalar-reduced loss ("mean" / "sum") are formed:
+#   "forward"   (default) during the forward, while the logits of a block of rows
+#               exist: 3 contractions per step instead of 4.  Taken where the
+#               library supports it (16-bit inputs, no bias, H and V multiples of
+#               64, the row count known to the host) and a gradient is required;
+#               other calls fall back to "recompute".  The forward then holds the
+#               float32 gradients ([M, H] and [V, H]) until the backward scales
+#               and rounds them;
+#   "recompute" by a backward that recomputes the logits in vocabulary panels, as
+#               the reference's backward does block by block
+#               (fused_linear_ce_cuda.cu:618-791).
+GRADIENT_MODES = ("forward", "recompute")
+_gradients = contextvars.ContextVar("tlce_gradient_mode", default="forward")
+
+
+def get_gradient_mode() -> str:
+    return _gradients.get()
+
+
+def _checked_gradient_mode(mode: str) -> str:
+    if mode not in GRADIENT_MODES:
+        raise ValueError(f"gradient mode must be one of {GRADIENT_MODES}")
+    return mode
+
+
+def set_gradient_mode(mode: str) -> str:
+    """Sets the mode for the current context (thread / task); returns the old one."""
+    old = _gradients.get()
+    _gradients.set(_checked_gradient_mode(mode))
+    return old
+
+
+@contextlib.contextmanager
+def gradient_mode(mode: str):
+    token = _gradients.set(_checked_gradient_mode(mode))
+    try:
+        yield
+    finally:
+        _gradients.reset(token)
 
 
 def _checked_mode(mode: str) -> str:

@@ -26,6 +26,7 @@ from typing import Optional
 
 import torch
 
+from . import options
 from .options import (COMPACTION_MODES, compaction_mode, get_compaction_mode,  # noqa: F401
                       resolve_compaction, set_compaction_mode)
 
@@ -269,6 +270,31 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
         rows, targets, _, row_idx, row_count, m = native.compact_loss_rows(
             hidden_flat, labels_flat, None, ignore_index, mode)
 
+    # Gradients while the logits exist (3 contractions instead of 4): when the loss
+    # is reduced to a scalar, some input needs a gradient, and the library takes the
+    # operands (options.GRADIENT_MODES).
+    wants_grad = bool(ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+    ctx.fused = (
+        wants_grad and mode != "device" and reduction in ("mean", "sum")
+        and options.get_gradient_mode() == "forward"
+        and native.fused_gradients_supported(rows, weight_vf, bias, in_place or weight_dim_first)
+    )
+    if ctx.fused:
+        # (rows compacted with the count read back carry up to 63 zero rows of padding)
+        losses, lse, valid_count, grad_rows32, grad_weight32 = native.forward_with_gradients(
+            rows[:m], weight_vf, targets[:m], ignore_index=ignore_index, exclude_index=exclude_index,
+            logit_softcap=float(logit_softcap),
+            compute_weight_grad=bool(ctx.needs_input_grad[1]), row_idx=row_idx, n_out=n,
+        )
+        ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx)
+        ctx.hidden_shape = hidden.shape
+        ctx.n_rows, ctx.m = n, m
+        ctx.reduction = reduction
+        ctx.grad_dtype = hidden.dtype
+        ctx.vocab = weight_vf.shape[0]
+        if reduction == "sum":
+            return losses.sum()
+        return losses.sum() / valid_count.squeeze(0)
     if row_count is None:
         losses, lse, valid_count = native.forward(
             rows, weight_vf, bias, targets,
@@ -305,6 +331,14 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
 def _device_backward(ctx, grad_output, frozen: bool):
     from . import chunked_linear_ce_native as native
 
+    if ctx.fused:
+        grad_rows32, grad_weight32, valid_count, row_idx = ctx.saved_tensors
+        grad_hidden, grad_weight = native.apply_grad_output(
+            grad_rows32, grad_weight32, grad_output, valid_count, reduction=ctx.reduction,
+            dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows, vocab=ctx.vocab,
+        )
+        return (grad_hidden.reshape(ctx.hidden_shape), None if frozen else grad_weight,
+                None) + (None,) * 9
     rows, weight_vf, bias, targets, lse, valid_count, row_idx, row_count = ctx.saved_tensors
     with native.panel_budget(ctx.panel_bytes):
         if row_count is None:
