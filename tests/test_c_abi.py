@@ -136,3 +136,58 @@ def test_dim_first_entry_points_validate_before_touching_a_gpu():
                                      _lib.DTYPE_F32, _lib.REDUCTION_SUM, -100, -1, 0.0, fake,
                                      fake, None, 0, fake, 1 << 30, None)
     assert rc != 0 and "read in place only" in _lib.last_error()
+
+
+def test_fused_gradient_entry_points_validate_before_touching_a_gpu():
+    lib = _lib.library()
+    assert lib.tlce_fused_gradients_supported(4096, 151936, _lib.DTYPE_BF16) == 1
+    assert lib.tlce_fused_gradients_supported(4096, 151936, _lib.DTYPE_F16) == 1
+    assert lib.tlce_fused_gradients_supported(4096, 151936, _lib.DTYPE_F32) == 0
+    assert lib.tlce_fused_gradients_supported(4096, 151937, _lib.DTYPE_BF16) == 0
+    assert lib.tlce_fused_gradients_supported(72, 1024, _lib.DTYPE_BF16) == 0
+    assert lib.tlce_forward_with_gradients_workspace_bytes(8, 72, 1024, _lib.DTYPE_BF16, 1, 0) == -1
+    fake = 4096          # aligned, never dereferenced: validation fails first
+
+    def forward(h=64, v=128, dtype=_lib.DTYPE_BF16, multiplier=1.0, ws_bytes=1 << 30, n_out=8,
+                row_idx=None):
+        return lib.tlce_forward_with_gradients(
+            fake, fake, fake, row_idx, None, 8, n_out, h, v, dtype, -100, -1, 0.0, multiplier,
+            fake, fake, fake, fake, fake, 0, fake, ws_bytes, None)
+
+    assert forward(h=72) != 0 and "multiples of 64" in _lib.last_error()
+    assert forward(dtype=_lib.DTYPE_F32) != 0 and "multiples of 64" in _lib.last_error()
+    assert forward(multiplier=0.0) != 0 and "multiplier must be positive" in _lib.last_error()
+    assert forward(ws_bytes=16) != 0 and "workspace too small" in _lib.last_error()
+    assert forward(n_out=4) != 0 and "n_out" in _lib.last_error()
+    assert forward(n_out=16) != 0 and "without row_idx" in _lib.last_error()
+    # the upstream gradient must be one number
+    rc = lib.tlce_apply_grad_output(fake, fake, None, fake, fake, 8, 8, 64, 128, _lib.DTYPE_BF16,
+                                    _lib.REDUCTION_NONE, fake, fake, None)
+    assert rc != 0 and "scalar" in _lib.last_error()
+    rc = lib.tlce_apply_grad_output(fake, None, None, fake, fake, 8, 8, 64, 128, _lib.DTYPE_BF16,
+                                    _lib.REDUCTION_SUM, fake, fake, None)
+    assert rc != 0 and "go together" in _lib.last_error()
+    rc = lib.tlce_apply_grad_output(fake, fake, None, fake, None, 8, 8, 64, 128, _lib.DTYPE_BF16,
+                                    _lib.REDUCTION_MEAN, fake, fake, None)
+    assert rc != 0 and "valid_count" in _lib.last_error()
+
+
+def test_fused_plan_blocks():
+    # the benchmark's shape: 2.5 GiB hold 34 token tiles over 594 vocabulary tiles; four
+    # balanced blocks of 32 tiles (whole rounds of 256 workgroups for grad_hidden)
+    plan = _lib.query_fused_plan(32768, 4096, 151936, _lib.DTYPE_BF16)
+    assert plan == {"block_rows": 8192, "n_blocks": 4, "grad_hidden_k_splits": 1}
+    # a 1 GiB panel: 13 tiles fit, ten balanced blocks
+    plan = _lib.query_fused_plan(32768, 4096, 151936, _lib.DTYPE_BF16, 1 << 30)
+    assert plan["block_rows"] == 13 * 256 and plan["n_blocks"] == 10
+    # everything in one block when it fits; the K split then fills the chip
+    plan = _lib.query_fused_plan(1610, 4096, 151936, _lib.DTYPE_BF16)
+    assert plan["n_blocks"] == 1 and plan["block_rows"] == 1792
+    assert plan["grad_hidden_k_splits"] > 1
+    # a budget below one tile still makes progress, one token tile at a time
+    plan = _lib.query_fused_plan(1000, 256, 5120, _lib.DTYPE_BF16, 1)
+    assert plan["block_rows"] == 256 and plan["n_blocks"] == 4
+    bytes_needed = _lib.library().tlce_forward_with_gradients_workspace_bytes(
+        32768, 4096, 151936, _lib.DTYPE_BF16, 1, 0)
+    panel = 8192 * 152064 * 2
+    assert panel < bytes_needed < panel + (1 << 30)

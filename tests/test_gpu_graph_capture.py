@@ -181,3 +181,64 @@ def test_frozen_kl_graph_replays_match_eager(gpu_device, n, hd, ht, v, softcap, 
         for name, a, b, c in zip(("losses", "grad_hidden"), got, eager, again):
             assert torch.equal(a, b), (replay, name)
             assert torch.equal(b, c), (replay, name, "eager runs differ")
+
+
+@pytest.mark.parametrize("n,h,v", [(700, 128, 1536)])
+def test_gradients_formed_in_the_forward_graph_replays_match_eager(gpu_device, n, h, v,
+                                                                   set_panel_budget):
+    """The forward that leaves the gradients, and the scaling by the upstream
+    gradient, from one graph: the decision to redo a block of rows with exact row
+    maxima is taken on the device (the second try's launches are recorded and do
+    nothing unless asked), so one graph serves inputs that need it and inputs that
+    do not."""
+    print("[case] fused-gradient graph capture", n, h, v, flush=True)
+    dev = gpu_device
+    set_panel_budget(256 * v * 2)          # one token tile per block: three blocks
+    gen = torch.Generator().manual_seed(n)
+    weight = (torch.randn(v, h, generator=gen) * 0.2).bfloat16().to(dev)
+
+    def make(far_rows):
+        hidden = torch.randn(n, h, generator=gen).bfloat16()
+        labels = torch.randint(0, v, (n,), generator=gen)
+        labels[torch.rand(n, generator=gen) < 0.2] = -100
+        for r in range(0, n, 5) if far_rows else ():
+            # a logit ~120 on another column than the label's: outside the window
+            w = weight[(int(labels[r]) + 1) % v].float().cpu()
+            hidden[r] = (w * (120.0 / float(w @ w))).bfloat16()
+        return hidden, labels
+
+    go = torch.full((1,), 0.75, device=dev)
+
+    def run(hidden, labels):
+        losses, lse, count, dh32, dw32 = native.forward_with_gradients(
+            hidden, weight, labels, ignore_index=-100, exclude_index=-1, logit_softcap=0.0,
+            compute_weight_grad=True)
+        dh, dw = native.apply_grad_output(dh32, dw32, go, count, reduction="mean",
+                                          dtype=torch.bfloat16)
+        return losses, dh, dw
+
+    static_hidden = torch.zeros(n, h, dtype=torch.bfloat16, device=dev)
+    static_labels = torch.zeros(n, dtype=torch.long, device=dev)
+    first = make(False)
+    static_hidden.copy_(first[0])
+    static_labels.copy_(first[1])
+    run(static_hidden, static_labels)            # warm-up: one-time kernel attributes
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outputs = run(static_hidden, static_labels)
+    torch.cuda.synchronize()
+
+    for replay in range(5):
+        hidden, labels = first if replay == 0 else make(far_rows=replay in (2, 3))
+        static_hidden.copy_(hidden)
+        static_labels.copy_(labels)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outputs]
+        eager = run(hidden.to(dev), labels.to(dev))      # eager work between replays
+        torch.cuda.synchronize()
+        for name, a, b in zip(("losses", "grad_hidden", "grad_weight"), got, eager):
+            assert torch.equal(a, b), (replay, name)
+        assert torch.isfinite(got[0]).all() and torch.isfinite(got[1].float()).all()

@@ -80,16 +80,22 @@ __global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPa
   E eng;
   typename E::Acc acc;
   const int vbase = vt * E::kTile;
-  // reference logit of each owned token column in base-2 units; +inf for rows
-  // past the block and rows without loss, whose whole column of e becomes 0
-  float ref2[E::kCols];
-#pragma unroll
-  for (int j = 0; j < E::kCols; ++j) {
-    const int r = tt * E::kTile + eng.col(j);
-    ref2[j] = (r < p.m) ? p.ref[r] * TLCE_LOG2E : INFINITY;
+  // Reference logit of every token column of the tile in base-2 units; +inf for
+  // rows past the block and rows without loss, whose whole column of e becomes 0.
+  // Fetched before the contraction so that the latency passes under it, and parked
+  // in the LDS beyond the engine's stages: during the main loop every register
+  // of the wave is taken.
+  float* ref_stash = reinterpret_cast<float*>(smem + E::kSmemBytes);
+  for (int c = threadIdx.x; c < E::kTile; c += E::kThreads) {
+    const int r = tt * E::kTile + c;
+    ref_stash[c] = (r < p.m) ? p.ref[r] * TLCE_LOG2E : INFINITY;
   }
   eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
                    static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
+  // (the main loop's barriers have made the stash visible to every wave)
+  float ref2[E::kCols];
+#pragma unroll
+  for (int j = 0; j < E::kCols; ++j) ref2[j] = ref_stash[eng.col(j)];
 
   const float inv_cap = kSoftcap ? p.logit_scale / p.softcap : 0.0f;
   const float to_base2 = kSoftcap ? p.softcap * TLCE_LOG2E : p.logit_scale * TLCE_LOG2E;
@@ -186,11 +192,12 @@ __global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPa
 template <class E, bool kSoftcap>
 int launch_exp_panel_variant(const ExpPanelArgs& a, hipStream_t stream) {
   static LdsOptIn lds;
-  if (int rc = enable_large_lds(lce_exp_logits_panel_kernel<E, kSoftcap>, E::kSmemBytes, lds))
+  constexpr int kLdsBytes = E::kSmemBytes + E::kTile * (int)sizeof(float);   // stages + stash
+  if (int rc = enable_large_lds(lce_exp_logits_panel_kernel<E, kSoftcap>, kLdsBytes, lds))
     return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_vtiles);
   ScopedTimer timer(kClassExpPanel, stream);
-  lce_exp_logits_panel_kernel<E, kSoftcap><<<grid, E::kThreads, E::kSmemBytes, stream>>>(a);
+  lce_exp_logits_panel_kernel<E, kSoftcap><<<grid, E::kThreads, kLdsBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }

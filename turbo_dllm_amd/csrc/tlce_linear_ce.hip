@@ -732,6 +732,18 @@ extern "C" int tlce_forward_with_gradients(
                "forward_with_gradients: n_out != m without row_idx");
   TLCE_REQUIRE(((uintptr_t)grad_hidden_f32 & 15) == 0 && ((uintptr_t)grad_weight_f32 & 15) == 0,
                "forward_with_gradients: gradients must be 16-byte aligned");
+  // everything that can be refused is refused before the first launch
+  const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
+  if (m > 0) {
+    TLCE_REQUIRE(labels && lse && grad_hidden_f32 && workspace,
+                 "forward_with_gradients: null pointer");
+    const int64_t need = fused_layout(p, m, h, dtype, grad_weight_f32 != nullptr).total;
+    TLCE_REQUIRE(workspace_bytes >= need,
+                 "forward_with_gradients: workspace too small (%lld < %lld)",
+                 (long long)workspace_bytes, (long long)need);
+    TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+                 "forward_with_gradients: workspace must be 256-byte aligned");
+  }
   if (int rc = fill_zero(valid_count, 4, stream)) return rc;
   if (losses != nullptr && (row_idx != nullptr || m == 0)) {
     if (int rc = fill_zero(losses, n_out * 4, stream)) return rc;
@@ -740,15 +752,6 @@ extern "C" int tlce_forward_with_gradients(
     if (grad_weight_f32 != nullptr) return fill_zero(grad_weight_f32, v * h * 4, stream);
     return 0;
   }
-  TLCE_REQUIRE(labels && lse && grad_hidden_f32 && workspace,
-               "forward_with_gradients: null pointer");
-  const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
-  const int64_t need = fused_layout(p, m, h, dtype, grad_weight_f32 != nullptr).total;
-  TLCE_REQUIRE(workspace_bytes >= need,
-               "forward_with_gradients: workspace too small (%lld < %lld)",
-               (long long)workspace_bytes, (long long)need);
-  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
-               "forward_with_gradients: workspace must be 256-byte aligned");
   FusedOptions opt;
   opt.logit_scale = logit_multiplier;
   opt.token_weights = token_weights;
