@@ -442,15 +442,16 @@ int tlce_segment_weighted_sum(const float* values, const float* weights,
  * tlce_apply_grad_output then multiplies both by the upstream gradient
  * (grad_output[0], divided by valid_count[0] for TLCE_REDUCTION_MEAN), rounds
  * them once to the input dtype, and un-compacts grad_hidden through row_idx
- * into [n_out, h] (other rows zero).  No bias, head stored [v, h], 16-bit inputs
+ * into [n_out, h] (other rows zero).  No bias, head stored [v, h], bf16 inputs
  * with h and v multiples of 64 (tlce_fused_gradients_supported); everything else
- * goes through tlce_forward / tlce_backward.
+ * goes through tlce_forward / tlce_backward (f16 included: its exponent range
+ * cannot hold exp(logit - reference) and the row sums of it).
  *
  * Rows are taken in blocks of as many rows as a panel of panel_bytes (0: 2.5 GiB)
  * holds over the whole vocabulary (tlce_query_fused_plan); the panel holds
- * exp(logit - reference) in the input dtype, the reference being the label's
+ * exp(logit - reference) in bf16, the reference being the label's
  * logit of the row.  A block in which some row's largest logit lies more than
- * 40 (8 for f16) above its reference is produced a second time with the exact
+ * 40 above its reference is produced a second time with the exact
  * row maxima as references; the decision is taken on the device, the second
  * try's launches are always made and do nothing otherwise.
  * logit_multiplier > 0 scales the raw dot products (1: plain operator). */

@@ -141,7 +141,7 @@ def test_dim_first_entry_points_validate_before_touching_a_gpu():
 def test_fused_gradient_entry_points_validate_before_touching_a_gpu():
     lib = _lib.library()
     assert lib.tlce_fused_gradients_supported(4096, 151936, _lib.DTYPE_BF16) == 1
-    assert lib.tlce_fused_gradients_supported(4096, 151936, _lib.DTYPE_F16) == 1
+    assert lib.tlce_fused_gradients_supported(4096, 151936, _lib.DTYPE_F16) == 0    # bf16 only
     assert lib.tlce_fused_gradients_supported(4096, 151936, _lib.DTYPE_F32) == 0
     assert lib.tlce_fused_gradients_supported(4096, 151937, _lib.DTYPE_BF16) == 0
     assert lib.tlce_fused_gradients_supported(72, 1024, _lib.DTYPE_BF16) == 0

@@ -34,10 +34,14 @@ _WHOLE_ENGINES = {"staged_bf16": "MfmaEngine<__bf16>", "staged_f16": "MfmaEngine
 _PARTS = {2: "grad_logits", 7: "grad_logits_cap", 8: "grad_logits_bias", 9: "grad_logits_cap_bias",
           1: "forward", 3: "gemm", 4: "kl", 5: "logits", 6: "sequences",
           10: "forward_dim_first", 11: "grad_logits_dim_first", 12: "exp_panel"}
+# the forward that leaves the gradients (part 12 and its launch sequence) exists for bf16 only
+_FUSED_ENGINES = ("direct_bf16",)
 UNITS = (
     [(f"engine_{tag}_{name}", "tlce_engine_unit.hip",
-      (f"-DTLCE_UNIT_ENGINE={engine}", f"-DTLCE_UNIT_PART={part}"))
-     for tag, engine in _SPLIT_ENGINES.items() for part, name in _PARTS.items()]
+      (f"-DTLCE_UNIT_ENGINE={engine}", f"-DTLCE_UNIT_PART={part}")
+      + (("-DTLCE_UNIT_FUSED=1",) if tag in _FUSED_ENGINES else ()))
+     for tag, engine in _SPLIT_ENGINES.items() for part, name in _PARTS.items()
+     if part != 12 or tag in _FUSED_ENGINES]
     + [(f"engine_{tag}", "tlce_engine_unit.hip",
         (f"-DTLCE_UNIT_ENGINE={engine}", "-DTLCE_UNIT_PART=0"))
        for tag, engine in _WHOLE_ENGINES.items()]

@@ -464,11 +464,12 @@ def forward(
 # ------------------------------------------- forward that leaves the gradients --
 def fused_gradients_supported(hidden: torch.Tensor, weight: torch.Tensor,
                               bias: torch.Tensor | None, weight_dim_first: bool) -> bool:
-    """Whether ``forward_with_gradients`` takes these operands: 16-bit inputs on
-    the GPU, head stored [V, H], no bias, H and V multiples of 64."""
+    """Whether ``forward_with_gradients`` takes these operands: bf16 inputs on the
+    GPU, head stored [V, H], no bias, H and V multiples of 64.  (f16's exponent
+    range cannot hold exp(logit - reference) and its row sums.)"""
     if bias is not None or weight_dim_first or not hidden.is_cuda:
         return False
-    if hidden.dtype not in (torch.bfloat16, torch.float16) or weight.dtype != hidden.dtype:
+    if hidden.dtype != torch.bfloat16 or weight.dtype != hidden.dtype:
         return False
     if hidden.dim() != 2 or weight.dim() != 2 or weight.shape[1] != hidden.shape[1]:
         return False
@@ -502,7 +503,7 @@ def forward_with_gradients(
     device = _require_device(hidden, weight, labels, row_idx, token_weights)
     if not fused_gradients_supported(hidden, weight, None, False):
         raise RuntimeError(
-            "forward_with_gradients needs bf16/f16 operands, a [V, H] head and H, V multiples "
+            "forward_with_gradients needs bf16 operands, a [V, H] head and H, V multiples "
             "of 64; use forward / backward for other inputs"
         )
     hidden = _dense(hidden)
@@ -574,7 +575,9 @@ def apply_grad_output(
     m, h = grad_hidden32.shape
     v = grad_weight32.shape[0] if grad_weight32 is not None else int(vocab or 1)
     n_out = m if n_out is None else int(n_out)
-    code = {torch.bfloat16: _lib.DTYPE_BF16, torch.float16: _lib.DTYPE_F16}[dtype]
+    if dtype != torch.bfloat16:
+        raise RuntimeError("apply_grad_output writes bf16 gradients only")
+    code = _lib.DTYPE_BF16
     with torch.cuda.device(device):
         grad_hidden = torch.empty((n_out, h), dtype=dtype, device=device)
         grad_weight = (torch.empty((v, h), dtype=dtype, device=device)

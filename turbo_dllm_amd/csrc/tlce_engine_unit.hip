@@ -10,7 +10,8 @@
 //                        10, 11: the forward statistics and the logit-gradient
 //                        panels over a head stored [h, v],
 //                        12: the exponentiated-logits panel of the forward that
-//                        leaves the gradients (direct engines only),
+//                        leaves the gradients (with TLCE_UNIT_FUSED, which also adds
+//                        that sequence to part 6: the bf16 direct engine only),
 //                        6: the launch sequences over them.
 #include "tlce_host.h"
 #include "tlce_fused.h"
@@ -76,14 +77,18 @@ TLCE_LAUNCHERS_GRAD_LOGITS_DIM_FIRST(template, UnitEngine)
 #else
 TLCE_LAUNCHERS_GRAD_LOGITS_DIM_FIRST(extern template, UnitEngine)
 #endif
+#ifdef TLCE_UNIT_FUSED   // the engine the forward that leaves the gradients is built for
 #if TLCE_UNIT_PART == 12
 TLCE_LAUNCHERS_EXP_PANEL(template, UnitEngine)
 #else
 TLCE_LAUNCHERS_EXP_PANEL(extern template, UnitEngine)
 #endif
+#endif
 #if TLCE_UNIT_PART == 6
 TLCE_ENGINE_ENTRY_POINTS(template, UnitEngine)
+#ifdef TLCE_UNIT_FUSED
 TLCE_FUSED_ENTRY_POINTS(template, UnitEngine)
+#endif
 #endif
 #endif
 

@@ -10,10 +10,10 @@
 // over the WHOLE vocabulary; per block:
 //
 //   1. lce_exp_logits_panel_kernel: one contraction; the panel receives
-//      e[r, v] = exp(z[r, v] - c[r]) * cap'(z) rounded to the input dtype, where
+//      e[r, v] = exp(z[r, v] - c[r]) * cap'(z) rounded to bf16, where
 //      c[r] is a per-row reference logit known beforehand (the label's logit, a
 //      one-row dot product).  Any c within ~80 of the row maximum keeps e inside
-//      the 16-bit formats' exponent range with full relative precision.  The
+//      bf16's exponent range (float32's) with full relative precision.  The
 //      tile sums of exp(z - c) and the tile maxima go out as per-tile partials.
 //   2. lce_fused_rows_kernel: lse[r] = c[r] + log(sum), loss, the row factor
 //      s[r] = weight[r] / sum (softmax = s * e), the label's panel entry replaced
@@ -38,15 +38,16 @@ namespace tlce {
 // The row offset beyond which the first try is redone with the exact maximum
 // (natural-log units).  exp(40) ~ 2e17 and its reciprocal are far inside the
 // bf16 / float32 exponent range, also after a multiplication by a hidden entry
-// or a loss weight; f16 panels (max 65504) are kept to +-8.
+// or a loss weight.  f16 (largest number 65504) has no such room: the label's
+// panel entry alone is of the size of sum_v exp(z - c) = 1 / softmax(label), so
+// the sequence is built for bf16 only and f16 inputs keep the recomputing backward.
 // Default bound of the panel of exponentiated logits: 32 token tiles over a
 // 152 K vocabulary in 16-bit.  Per block of rows the grad_weight accumulator
 // [v, h] float32 is read and written once, so fewer, larger blocks cost less
 // (measured at 32768 x 4096 x 151936: 1 GiB 106.7 ms per step, 1.2 GiB 101.5,
 // 2.4 GiB 96.9).
 constexpr int64_t kDefaultFusedPanelBytes = 5ll << 29;
-constexpr float kRefWindowWide = 40.0f;
-constexpr float kRefWindowF16 = 8.0f;
+constexpr float kRefWindow = 40.0f;
 
 struct ExpPanelArgs {
   const void* hidden;   // [m, h] the rows of this block
@@ -217,7 +218,6 @@ struct LabelLogitArgs {
   float* target;        // [m] cap(scale * h . w[label]); 0 when the label has no logit
   float* ref;           // [m] reference logit; +inf for rows without loss
   float* valid_count;   // [1] += rows with a label other than `ignore`
-  int dtype;
 };
 
 struct FusedRowsArgs {
@@ -244,7 +244,6 @@ struct FusedRowsArgs {
   float* ref_next;             // [m] reference of the second try
   int* redo;                   // [1] set when some row needs the second try
   const int* run_flag;         // non-null: run only when *run_flag != 0
-  int dtype;
 };
 
 // grad_hidden32[r, :] = row_scale[r] * sum over K splits of slab[s][r, :]
@@ -269,7 +268,6 @@ struct ScaleCastArgs {
   int64_t rows;
   int h;
   void* out;
-  int dtype;
 };
 
 int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream);
@@ -287,7 +285,7 @@ struct FusedPlan {
 };
 
 inline bool fused_gradients_supported(int64_t h, int64_t v, int dtype) {
-  return engine_class(h, dtype) == 2 && (v % 64) == 0;
+  return dtype == TLCE_DTYPE_BF16 && engine_class(h, dtype) == 2 && (v % 64) == 0;
 }
 
 inline FusedPlan make_fused_plan(int64_t m, int64_t h, int64_t v, int dtype, int64_t panel_bytes) {
@@ -373,7 +371,7 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
   la.hidden = hidden; la.weight = weight; la.labels = labels;
   la.m = (int)m; la.h = (int)h; la.v = (int)v;
   la.ignore = ignore; la.exclude = exclude; la.softcap = softcap; la.logit_scale = opt.logit_scale;
-  la.target = target; la.ref = ref; la.valid_count = valid_count; la.dtype = dtype;
+  la.target = target; la.ref = ref; la.valid_count = valid_count;
   if (int rc = launch_label_logit(la, stream)) return rc;
 
   for (int block = 0; block < p.n_blocks; ++block) {
@@ -402,11 +400,11 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
     ra.m = (int)rows; ra.m_pad = (int)rows_p; ra.h = (int)h; ra.v = (int)v;
     ra.ignore = ignore; ra.exclude = exclude; ra.softcap = softcap;
     ra.logit_scale = opt.logit_scale;
-    ra.window = (dtype == TLCE_DTYPE_F16) ? kRefWindowF16 : kRefWindowWide;
+    ra.window = kRefWindow;
     ra.panel = panel; ra.ld = p.vp;
     ra.lse = lse + r0; ra.losses = losses;
     ra.row_scale = row_scale; ra.scaled_hidden = scaled_hidden;
-    ra.ref_next = ref_next; ra.redo = redo + block; ra.dtype = dtype;
+    ra.ref_next = ref_next; ra.redo = redo + block;
 
     for (int attempt = 0; attempt < 2; ++attempt) {
       ea.ref = attempt ? ref_next : ref + r0;

@@ -67,25 +67,17 @@ int launch_sum(const float* x, int64_t n, float* out, hipStream_t stream) {
 }
 
 // ---- row kernels of the forward that leaves the gradients (tlce_fused_rows.h) ----
-#define TLCE_BY_16BIT_DTYPE(dtype, CALL)                          \
-  do {                                                            \
-    if ((dtype) == TLCE_DTYPE_BF16) { using T = __bf16; CALL; }   \
-    else { using T = _Float16; CALL; }                            \
-  } while (0)
-
 int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassCombine, stream);
-  TLCE_BY_16BIT_DTYPE(a.dtype,
-                      (lce_label_logit_kernel<T><<<(int)ceil_div(a.m, 16), 256, 0, stream>>>(a)));
+  lce_label_logit_kernel<__bf16><<<(int)ceil_div(a.m, 16), 256, 0, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
 
 int launch_fused_rows(const FusedRowsArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassCombine, stream);
-  TLCE_BY_16BIT_DTYPE(
-      a.dtype, (lce_fused_rows_kernel<T><<<(int)ceil_div(a.m_pad, kFusedRowsPerBlock), 256, 0,
-                                           stream>>>(a)));
+  lce_fused_rows_kernel<__bf16>
+      <<<(int)ceil_div(a.m_pad, kFusedRowsPerBlock), 256, 0, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
@@ -100,14 +92,12 @@ int launch_reduce_slabs(const ReduceSlabsArgs& a, hipStream_t stream) {
 int launch_scale_cast(const ScaleCastArgs& a, hipStream_t stream) {
   if (a.rows <= 0) return 0;
   ScopedTimer timer(kClassOther, stream);
-  TLCE_BY_16BIT_DTYPE(a.dtype,
-                      (lce_scale_cast_rows_kernel<T><<<(unsigned)a.rows, 256, 0, stream>>>(a)));
+  lce_scale_cast_rows_kernel<__bf16><<<(unsigned)a.rows, 256, 0, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
 
 TLCE_FUSED_ENTRY_POINTS(extern template, MfmaDirect4Engine<__bf16>)
-TLCE_FUSED_ENTRY_POINTS(extern template, MfmaDirect4Engine<_Float16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaDirect4Engine<__bf16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaDirect4Engine<_Float16>)
 TLCE_ENGINE_ENTRY_POINTS(extern template, MfmaEngine<__bf16>)
@@ -696,7 +686,7 @@ extern "C" int tlce_query_fused_plan(int64_t m, int64_t h, int64_t v, int dtype,
                                      int* grad_hidden_k_splits) {
   TLCE_REQUIRE(m >= 0 && h > 0 && v > 0, "query_fused_plan: bad shape");
   TLCE_REQUIRE(fused_gradients_supported(h, v, dtype),
-               "query_fused_plan: needs 16-bit inputs with h and v multiples of 64");
+               "query_fused_plan: needs bf16 inputs with h and v multiples of 64");
   const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
   if (block_rows) *block_rows = p.block_rows;
   if (n_blocks) *n_blocks = p.n_blocks;
@@ -721,7 +711,7 @@ extern "C" int tlce_forward_with_gradients(
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (int rc = validate_common(hidden, weight, m, h, v, dtype)) return rc;
   TLCE_REQUIRE(fused_gradients_supported(h, v, dtype),
-               "forward_with_gradients: needs 16-bit inputs with h and v multiples of 64 "
+               "forward_with_gradients: needs bf16 inputs with h and v multiples of 64 "
                "(h=%lld v=%lld dtype=%d)", (long long)h, (long long)v, dtype);
   TLCE_REQUIRE(valid_count != nullptr, "forward_with_gradients: valid_count is null");
   TLCE_REQUIRE(logit_multiplier > 0.0f,
@@ -755,13 +745,7 @@ extern "C" int tlce_forward_with_gradients(
   FusedOptions opt;
   opt.logit_scale = logit_multiplier;
   opt.token_weights = token_weights;
-  if (dtype == TLCE_DTYPE_BF16) {
-    return fused_gradients_impl<MfmaDirect4Engine<__bf16>>(
-        p, hidden, weight, labels, row_idx, m, h, v, dtype, ignore_index, exclude_index,
-        logit_softcap, losses, lse, valid_count, grad_hidden_f32, grad_weight_f32,
-        static_cast<char*>(workspace), stream, opt);
-  }
-  return fused_gradients_impl<MfmaDirect4Engine<_Float16>>(
+  return fused_gradients_impl<MfmaDirect4Engine<__bf16>>(
       p, hidden, weight, labels, row_idx, m, h, v, dtype, ignore_index, exclude_index,
       logit_softcap, losses, lse, valid_count, grad_hidden_f32, grad_weight_f32,
       static_cast<char*>(workspace), stream, opt);
@@ -773,8 +757,8 @@ extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float*
                                       int64_t h, int64_t v, int dtype, int reduction_code,
                                       void* grad_hidden, void* grad_weight, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
-  TLCE_REQUIRE(dtype == TLCE_DTYPE_BF16 || dtype == TLCE_DTYPE_F16,
-               "apply_grad_output: unsupported dtype code %d", dtype);
+  TLCE_REQUIRE(dtype == TLCE_DTYPE_BF16, "apply_grad_output: unsupported dtype code %d (bf16 only)",
+               dtype);
   TLCE_REQUIRE(m >= 0 && h > 0 && v > 0 && (h % 4) == 0, "apply_grad_output: bad shape");
   TLCE_REQUIRE(reduction_code == TLCE_REDUCTION_SUM || reduction_code == TLCE_REDUCTION_MEAN,
                "apply_grad_output: the upstream gradient must be a scalar (sum or mean)");
@@ -797,7 +781,7 @@ extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float*
   }
   ScaleCastArgs a;
   a.grad_output = grad_output; a.valid_count = valid_count; a.reduction = reduction_code;
-  a.h = (int)h; a.dtype = dtype;
+  a.h = (int)h;
   if (m > 0) {
     TLCE_REQUIRE(grad_hidden_f32 != nullptr, "apply_grad_output: null pointer");
     a.in = grad_hidden_f32; a.row_idx = row_idx; a.rows = m; a.out = grad_hidden;
