@@ -524,16 +524,18 @@ def main() -> int:
         # the same operands and entry points the loss API uses for this compaction mode
         rows, targets, _, row_idx, count, m_rows = native.compact_loss_rows(
             hidden.detach(), labels, None, -100, args.compaction_mode)
-        fused = (args.gradients == "forward" and args.compaction_mode != "device"
+        fused = (args.gradients == "forward"
                  and native.fused_gradients_supported(rows, weight.detach(), None, False))
+        on_device = count if args.compaction_mode == "device" else None
         if fused:
             with _lib.kernel_profile() as prof:
                 out = native.forward_with_gradients(
                     rows[:m_rows], weight.detach(), targets[:m_rows], ignore_index=-100,
                     exclude_index=-1, logit_softcap=softcap, compute_weight_grad=True,
-                    row_idx=row_idx, n_out=n)
+                    row_idx=row_idx, n_out=n, row_count=on_device)
                 native.apply_grad_output(out[3], out[4], go, out[2], reduction="mean",
-                                         dtype=hidden.dtype, row_idx=row_idx, n_out=n)
+                                         dtype=hidden.dtype, row_idx=row_idx, n_out=n,
+                                         row_count=on_device)
             del out
         elif count is not None:
             kw = dict(m=m_rows, row_idx=row_idx, row_count=count, n_out=n, ignore_index=-100,

@@ -454,7 +454,12 @@ int tlce_segment_weighted_sum(const float* values, const float* weights,
  * 40 above its reference is produced a second time with the exact
  * row maxima as references; the decision is taken on the device, the second
  * try's launches are always made and do nothing otherwise.
- * logit_multiplier > 0 scales the raw dot products (1: plain operator). */
+ * logit_multiplier > 0 scales the raw dot products (1: plain operator).
+ * row_count (device int64, optional, needs row_idx): the real number of rows
+ * when m is only the capacity the launches and buffers are sized for; as in
+ * tlce_masked_loss_*, workgroups past the count exit at once and nothing needs
+ * the host, so compaction, this call and tlce_apply_grad_output record into one
+ * HIP graph that serves any mask. */
 int tlce_fused_gradients_supported(int64_t h, int64_t v, int dtype);
 
 int tlce_query_fused_plan(int64_t m, int64_t h, int64_t v, int dtype,
@@ -467,7 +472,8 @@ int64_t tlce_forward_with_gradients_workspace_bytes(int64_t m, int64_t h, int64_
 
 int tlce_forward_with_gradients(const void* hidden, const void* weight,
                                 const int64_t* labels, const int64_t* row_idx,
-                                const float* token_weights, int64_t m, int64_t n_out,
+                                const float* token_weights, const int64_t* row_count,
+                                int64_t m, int64_t n_out,
                                 int64_t h, int64_t v, int dtype, int64_t ignore_index,
                                 int64_t exclude_index, float logit_softcap,
                                 float logit_multiplier, float* losses, float* lse,
@@ -476,7 +482,8 @@ int tlce_forward_with_gradients(const void* hidden, const void* weight,
                                 void* workspace, int64_t workspace_bytes, void* stream);
 
 int tlce_apply_grad_output(const float* grad_hidden_f32, const float* grad_weight_f32,
-                           const int64_t* row_idx, const float* grad_output,
+                           const int64_t* row_idx, const int64_t* row_count,
+                           const float* grad_output,
                            const float* valid_count, int64_t m, int64_t n_out,
                            int64_t h, int64_t v, int dtype, int reduction_code,
                            void* grad_hidden, void* grad_weight, void* stream);

@@ -149,10 +149,10 @@ def test_fused_gradient_entry_points_validate_before_touching_a_gpu():
     fake = 4096          # aligned, never dereferenced: validation fails first
 
     def forward(h=64, v=128, dtype=_lib.DTYPE_BF16, multiplier=1.0, ws_bytes=1 << 30, n_out=8,
-                row_idx=None):
+                row_idx=None, row_count=None):
         return lib.tlce_forward_with_gradients(
-            fake, fake, fake, row_idx, None, 8, n_out, h, v, dtype, -100, -1, 0.0, multiplier,
-            fake, fake, fake, fake, fake, 0, fake, ws_bytes, None)
+            fake, fake, fake, row_idx, None, row_count, 8, n_out, h, v, dtype, -100, -1, 0.0,
+            multiplier, fake, fake, fake, fake, fake, 0, fake, ws_bytes, None)
 
     assert forward(h=72) != 0 and "multiples of 64" in _lib.last_error()
     assert forward(dtype=_lib.DTYPE_F32) != 0 and "multiples of 64" in _lib.last_error()
@@ -160,15 +160,16 @@ def test_fused_gradient_entry_points_validate_before_touching_a_gpu():
     assert forward(ws_bytes=16) != 0 and "workspace too small" in _lib.last_error()
     assert forward(n_out=4) != 0 and "n_out" in _lib.last_error()
     assert forward(n_out=16) != 0 and "without row_idx" in _lib.last_error()
+    assert forward(row_count=fake) != 0 and "needs row_idx" in _lib.last_error()
     # the upstream gradient must be one number
-    rc = lib.tlce_apply_grad_output(fake, fake, None, fake, fake, 8, 8, 64, 128, _lib.DTYPE_BF16,
-                                    _lib.REDUCTION_NONE, fake, fake, None)
+    rc = lib.tlce_apply_grad_output(fake, fake, None, None, fake, fake, 8, 8, 64, 128,
+                                    _lib.DTYPE_BF16, _lib.REDUCTION_NONE, fake, fake, None)
     assert rc != 0 and "scalar" in _lib.last_error()
-    rc = lib.tlce_apply_grad_output(fake, None, None, fake, fake, 8, 8, 64, 128, _lib.DTYPE_BF16,
-                                    _lib.REDUCTION_SUM, fake, fake, None)
+    rc = lib.tlce_apply_grad_output(fake, None, None, None, fake, fake, 8, 8, 64, 128,
+                                    _lib.DTYPE_BF16, _lib.REDUCTION_SUM, fake, fake, None)
     assert rc != 0 and "go together" in _lib.last_error()
-    rc = lib.tlce_apply_grad_output(fake, fake, None, fake, None, 8, 8, 64, 128, _lib.DTYPE_BF16,
-                                    _lib.REDUCTION_MEAN, fake, fake, None)
+    rc = lib.tlce_apply_grad_output(fake, fake, None, None, fake, None, 8, 8, 64, 128,
+                                    _lib.DTYPE_BF16, _lib.REDUCTION_MEAN, fake, fake, None)
     assert rc != 0 and "valid_count" in _lib.last_error()
 
 

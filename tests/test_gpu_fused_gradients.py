@@ -174,6 +174,49 @@ def test_uncompaction_through_row_idx(gpu_device):
     assert torch.all(dh[labels == -100] == 0)
 
 
+@pytest.mark.parametrize("keep_fraction", [0.0, 0.002, 0.25, 0.6, 1.0])
+@pytest.mark.parametrize("tiles_per_block", [0, 1, 2])
+def test_row_count_kept_on_the_device(gpu_device, keep_fraction, tiles_per_block):
+    """Operands sized for all rows, the count of loss-bearing rows only in device
+    memory (the "device" compaction mode): every launch is sized for the capacity,
+    workgroups and whole blocks of rows past the count do nothing, and an
+    accumulating grad_weight launch with no rows leaves the accumulator alone."""
+    say("device row count", keep_fraction, tiles_per_block)
+    n, h, v = 1100, 128, 2112
+    hidden, weight, labels = make_case(n, h, v, seed=61, ignored=1.0 - keep_fraction)
+    if keep_fraction == 0.0:
+        labels[:] = -100
+    dev = gpu_device
+    vp = (v + 255) // 256 * 256
+    with options.panel_budget(tiles_per_block * 256 * vp * 2):
+        rows, targets, _, row_idx, row_count, m = native.compact_loss_rows(
+            hidden.to(dev), labels.to(dev), None, -100, "device")
+        assert m == n and row_count is not None
+        out = native.forward_with_gradients(
+            rows[:n], weight.to(dev), targets[:n], ignore_index=-100, exclude_index=-1,
+            logit_softcap=0.0, compute_weight_grad=True, row_idx=row_idx, n_out=n,
+            row_count=row_count)
+        losses, _, valid, dh32, dw32 = out
+        go = torch.tensor([0.7], device=dev)
+        dh, dw = native.apply_grad_output(dh32, dw32, go, valid, reduction="sum",
+                                          dtype=torch.bfloat16, row_idx=row_idx, n_out=n,
+                                          row_count=row_count)
+    torch.cuda.synchronize()
+    keep = labels != -100
+    assert float(valid) == float(keep.sum()) == float(row_count)
+    okw = dict(dtype=torch.float32)
+    ref_losses = oracle.dense_linear_ce(hidden, weight, labels, reduction="none", **okw)
+    torch.testing.assert_close(losses.cpu(), ref_losses, rtol=LOSS_RTOL, atol=1e-3)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, torch.tensor(0.7),
+                                               reduction="sum", **okw)
+    if keep.any():
+        assert oracle.relative_max_error(dh.cpu(), rdh) <= GRAD_REL_MAX
+        assert oracle.relative_max_error(dw.cpu(), rdw) <= GRAD_REL_MAX
+    else:
+        assert torch.all(dw == 0)
+    assert torch.all(dh.cpu()[~keep] == 0)
+
+
 @pytest.mark.parametrize("reduction", ["mean", "sum"])
 @pytest.mark.parametrize("frozen", [False, True])
 def test_loss_api_takes_the_fused_path_and_agrees_with_recompute(gpu_device, reduction, frozen):

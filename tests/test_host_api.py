@@ -326,6 +326,46 @@ def test_options_are_local_to_the_calling_thread():
     options.set_panel_bytes(old)
 
 
+def test_gradient_mode_option_and_host_tensors():
+    """The gradient mode is a context-local option like the others; host tensors
+    never take the library's forward-with-gradients path, whatever the mode."""
+    import threading
+
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    from turbo_dllm_amd import options
+    from turbo_dllm_amd.tiled_linear_cross_entropy import tiled_linear_cross_entropy
+
+    assert options.GRADIENT_MODES == ("forward", "recompute")
+    assert options.get_gradient_mode() == "forward"
+    seen = {}
+    with options.gradient_mode("recompute"):
+        thread = threading.Thread(target=lambda: seen.update(mode=options.get_gradient_mode()))
+        thread.start()
+        thread.join(10)
+        assert options.get_gradient_mode() == "recompute"
+    assert seen["mode"] == "forward" and options.get_gradient_mode() == "forward"
+    with pytest.raises(ValueError):
+        options.set_gradient_mode("lazy")
+    old = options.set_gradient_mode("recompute")
+    assert old == "forward"
+    options.set_gradient_mode(old)
+
+    gen = torch.Generator().manual_seed(0)
+    hidden = torch.randn(6, 64, generator=gen).bfloat16()
+    weight = torch.randn(128, 64, generator=gen).bfloat16()
+    labels = torch.randint(0, 128, (6,), generator=gen)
+    assert not native.fused_gradients_supported(hidden, weight, None, False)   # host tensors
+    results = []
+    for mode in options.GRADIENT_MODES:
+        x = hidden.clone().requires_grad_(True)
+        with options.gradient_mode(mode):
+            loss = tiled_linear_cross_entropy(x, weight, labels, dtype=torch.float32,
+                                              weight_layout="vocab_first")
+            loss.backward()
+        results.append((loss.detach(), x.grad))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+
+
 def test_verify_dflash_symbols():
     """Start-up check of the DFlash executor (reference shim,
     chunked_linear_ce_native.py:353-363): unknown kinds raise ValueError, known

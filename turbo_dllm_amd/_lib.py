@@ -114,6 +114,7 @@ SIGNATURES = {
         c_int,
         [
             c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # hidden weight labels row_idx weights
+            c_void_p,                                           # row_count
             c_int64, c_int64, c_int64, c_int64, c_int,          # m n_out h v dtype
             c_int64, c_int64, c_float, c_float,                 # ignore exclude softcap multiplier
             c_void_p, c_void_p, c_void_p,                       # losses lse valid_count
@@ -124,7 +125,8 @@ SIGNATURES = {
     "tlce_apply_grad_output": (
         c_int,
         [
-            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # dh32 dw32 row_idx grad_output valid
+            c_void_p, c_void_p, c_void_p, c_void_p,             # dh32 dw32 row_idx row_count
+            c_void_p, c_void_p,                                 # grad_output valid_count
             c_int64, c_int64, c_int64, c_int64, c_int, c_int,   # m n_out h v dtype reduction
             c_void_p, c_void_p, c_void_p,                       # grad_hidden grad_weight stream
         ],

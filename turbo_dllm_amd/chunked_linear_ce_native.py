@@ -490,6 +490,7 @@ def forward_with_gradients(
     logit_multiplier: float = 1.0,
     row_idx: torch.Tensor | None = None,
     n_out: int | None = None,
+    row_count: torch.Tensor | None = None,
 ):
     """The forward and, in the same pass over the logits, the float32 gradients of
     ``sum_r token_weights[r] * loss[r]`` (three contractions instead of the four
@@ -498,9 +499,11 @@ def forward_with_gradients(
     Returns ``(losses [n_out] f32, lse [m] f32, valid_count [1] f32,
     grad_hidden_f32 [m, H], grad_weight_f32 [V, H] or None)``;
     ``apply_grad_output`` turns the last two into the gradients of the reduced
-    loss once the upstream gradient is known.
+    loss once the upstream gradient is known.  ``row_count`` (device int64, with
+    ``row_idx``): the real number of rows when the operands are sized for a
+    capacity, as the "device" compaction mode leaves them.
     """
-    device = _require_device(hidden, weight, labels, row_idx, token_weights)
+    device = _require_device(hidden, weight, labels, row_idx, token_weights, row_count)
     if not fused_gradients_supported(hidden, weight, None, False):
         raise RuntimeError(
             "forward_with_gradients needs bf16 operands, a [V, H] head and H, V multiples "
@@ -538,7 +541,7 @@ def forward_with_gradients(
         _lib.check(
             lib.tlce_forward_with_gradients(
                 _ptr(hidden), _ptr(weight), _ptr(labels), _ptr(row_idx), _ptr(token_weights),
-                m, n_out, h, v, code,
+                _ptr(row_count), m, n_out, h, v, code,
                 int(ignore_index), int(exclude_index), float(logit_softcap),
                 float(logit_multiplier),
                 _ptr(losses), _ptr(lse), valid_count.data_ptr(),
@@ -561,6 +564,7 @@ def apply_grad_output(
     row_idx: torch.Tensor | None = None,
     n_out: int | None = None,
     vocab: int | None = None,
+    row_count: torch.Tensor | None = None,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``(grad_hidden [n_out, H], grad_weight [V, H] or None)`` in ``dtype``: the
     float32 gradients ``forward_with_gradients`` left, times the upstream gradient
@@ -584,8 +588,8 @@ def apply_grad_output(
                        if grad_weight32 is not None else None)
         _lib.check(
             _lib.library().tlce_apply_grad_output(
-                _ptr(grad_hidden32), _ptr(grad_weight32), _ptr(row_idx), _ptr(grad_output),
-                _ptr(valid_count), m, n_out, h, v, code, reduction_code,
+                _ptr(grad_hidden32), _ptr(grad_weight32), _ptr(row_idx), _ptr(row_count),
+                _ptr(grad_output), _ptr(valid_count), m, n_out, h, v, code, reduction_code,
                 _ptr(grad_hidden), _ptr(grad_weight), _stream(device),
             ),
             "tlce_apply_grad_output",

@@ -103,6 +103,14 @@ __device__ __forceinline__ int effective_rows(int m, const int64_t* m_dev) {
   return c < 0 ? 0 : (c < (int64_t)m ? (int)c : m);
 }
 
+// Rows of a block of `cap` rows that starts at row `offset` of a matrix whose real
+// row count is on the device (null: all `cap`).
+__device__ __forceinline__ int effective_block_rows(int cap, const int64_t* m_dev, int64_t offset) {
+  if (m_dev == nullptr) return cap;
+  const int64_t c = *m_dev - offset;
+  return c < 0 ? 0 : (c < (int64_t)cap ? (int)c : cap);
+}
+
 // Logical block id when only the first `tiles` of the launched workgroups have
 // work (the launch was sized for more rows than there are): the same mapping a
 // launch of round_up(tiles, 8) workgroups would get; -1 for the others.

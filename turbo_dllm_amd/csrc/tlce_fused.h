@@ -64,6 +64,10 @@ struct ExpPanelArgs {
   float* part_max;      // [n_vtiles, part_ld] tile maximum of z in base-2 units
   int part_ld;
   const int* run_flag;  // non-null: the launch does nothing unless *run_flag != 0
+  // Row count known only to the device (null: m is exact): m is then the block's
+  // capacity, and the block holds rows [row0, row0 + m) of the counted rows.
+  const int64_t* m_dev = nullptr;
+  int64_t row0 = 0;
 };
 
 template <class E, bool kSoftcap>
@@ -73,6 +77,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPa
   static_assert(E::kHasKMajor && sizeof(T) == 2 && E::kCols == 4,
                 "written for the four-wave direct-to-LDS engine");
   if (p.run_flag != nullptr && *p.run_flag == 0) return;
+  if (p.m_dev != nullptr) {
+    p.m = effective_block_rows(p.m, p.m_dev, p.row0);
+    p.n_ttiles = (p.m + E::kTile - 1) / E::kTile;
+  }
   const int logical = xcd_logical_block_of(blockIdx.x, p.n_ttiles * p.n_vtiles);
   if (logical < 0) return;
   int tt, vt;
@@ -218,6 +226,7 @@ struct LabelLogitArgs {
   float* target;        // [m] cap(scale * h . w[label]); 0 when the label has no logit
   float* ref;           // [m] reference logit; +inf for rows without loss
   float* valid_count;   // [1] += rows with a label other than `ignore`
+  const int64_t* m_dev = nullptr;   // device row count (null: m is exact)
 };
 
 struct FusedRowsArgs {
@@ -244,6 +253,8 @@ struct FusedRowsArgs {
   float* ref_next;             // [m] reference of the second try
   int* redo;                   // [1] set when some row needs the second try
   const int* run_flag;         // non-null: run only when *run_flag != 0
+  const int64_t* m_dev = nullptr;   // device row count (null: m is exact); the block's
+  int64_t row0 = 0;                 // first row among the counted rows
 };
 
 // grad_hidden32[r, :] = row_scale[r] * sum over K splits of slab[s][r, :]
@@ -254,6 +265,12 @@ struct ReduceSlabsArgs {
   const float* row_scale;
   int m, h;
   float* out;   // [m, h]
+  const int64_t* m_dev = nullptr;   // device row count (null: m is exact); the block's
+  int64_t row0 = 0;                 // first row among the counted rows
+  // with a device row count the contraction derives its K splits and slab stride from
+  // the real rows of the block (dynamic_k_splits); the same inputs reproduce them here
+  int n_htiles = 0, tile = 0, launched_splits = 0, k_steps = 0;
+  int64_t slab_budget = 0;
 };
 
 // out[row_idx[r], :] = dtype(g * in[r, :]) with g = grad_output[0] (/ valid_count[0]
@@ -268,6 +285,7 @@ struct ScaleCastArgs {
   int64_t rows;
   int h;
   void* out;
+  const int64_t* m_dev = nullptr;   // device row count: rows past it are not written
 };
 
 int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream);
@@ -342,6 +360,7 @@ inline FusedLayout fused_layout(const FusedPlan& p, int64_t m, int64_t h, int dt
 struct FusedOptions {
   float logit_scale = 1.0f;
   const float* token_weights = nullptr;   // [m] per-row loss weights or null
+  const int64_t* row_count = nullptr;     // device int64: the real number of rows (m: capacity)
 };
 
 template <class E>
@@ -351,6 +370,9 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
                          float* losses, float* lse, float* valid_count, float* grad_hidden32,
                          float* grad_weight32, char* ws, hipStream_t stream,
                          const FusedOptions& opt) {
+  // opt.row_count != null: m is the capacity every launch is sized for; the kernels
+  // take the real count from the device and the workgroups past it exit at once
+  const int64_t* m_dev = opt.row_count;
   using T = typename E::T;
   const bool weight_grad = grad_weight32 != nullptr;
   const FusedLayout l = fused_layout(p, m, h, dtype, weight_grad);
@@ -371,7 +393,7 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
   la.hidden = hidden; la.weight = weight; la.labels = labels;
   la.m = (int)m; la.h = (int)h; la.v = (int)v;
   la.ignore = ignore; la.exclude = exclude; la.softcap = softcap; la.logit_scale = opt.logit_scale;
-  la.target = target; la.ref = ref; la.valid_count = valid_count;
+  la.target = target; la.ref = ref; la.valid_count = valid_count; la.m_dev = m_dev;
   if (int rc = launch_label_logit(la, stream)) return rc;
 
   for (int block = 0; block < p.n_blocks; ++block) {
@@ -389,6 +411,7 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
     ea.n_ttiles = n_ttiles; ea.n_vtiles = p.n_vtiles;
     ea.panel = panel; ea.ld = p.vp;
     ea.part_sum = part_sum; ea.part_max = part_max; ea.part_ld = (int)p.block_rows;
+    ea.m_dev = m_dev; ea.row0 = r0;
 
     FusedRowsArgs ra;
     ra.hidden = hidden_t + r0 * h; ra.labels = labels + r0;
@@ -405,6 +428,7 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
     ra.lse = lse + r0; ra.losses = losses;
     ra.row_scale = row_scale; ra.scaled_hidden = scaled_hidden;
     ra.ref_next = ref_next; ra.redo = redo + block;
+    ra.m_dev = m_dev; ra.row0 = r0;
 
     for (int attempt = 0; attempt < 2; ++attempt) {
       ea.ref = attempt ? ref_next : ref + r0;
@@ -430,16 +454,28 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
     dh.c = slabs; dh.ldc = h; dh.c_rows = (int)rows_p; dh.c_cols = (int)h;
     dh.c_split_stride = p.block_rows * h;
     dh.mode = kStoreF32;
-    const int ksplit = (rows_p == p.block_rows)
-                           ? p.dh_ksplit
-                           : std::min(p.dh_ksplit,
-                                      grad_hidden_k_splits((int64_t)n_ttiles * p.n_htiles,
-                                                           p.dh_ksplit, p.vp / 64, rows_p * h));
-    if (int rc = launch_gemm<E, true, false>(dh, ksplit, kClassGradHidden, stream)) return rc;
+    int ksplit = (rows_p == p.block_rows)
+                     ? p.dh_ksplit
+                     : std::min(p.dh_ksplit,
+                                grad_hidden_k_splits((int64_t)n_ttiles * p.n_htiles, p.dh_ksplit,
+                                                     p.vp / 64, rows_p * h));
     ReduceSlabsArgs rs;
+    if (m_dev != nullptr) {
+      // The block may hold far fewer rows than it was sized for (down to none): up to 16
+      // splits are launched and the kernel takes as many as the real rows call for,
+      // within the slab memory the plan allocated; the others exit at once.
+      dh.m_dev = m_dev; dh.m_role = kRowsFollow; dh.m_dev_offset = r0;
+      dh.slab_budget = (int64_t)p.dh_ksplit * p.block_rows * h;
+      dh.k_steps_plan = (int)(p.vp / 64);
+      ksplit = (int)std::max<int64_t>(p.dh_ksplit, std::min<int64_t>(16, p.vp / 64 / 8));
+      rs.n_htiles = p.n_htiles; rs.tile = E::kTile; rs.launched_splits = ksplit;
+      rs.k_steps = dh.k_steps_plan; rs.slab_budget = dh.slab_budget;
+    }
+    if (int rc = launch_gemm<E, true, false>(dh, ksplit, kClassGradHidden, stream)) return rc;
     rs.slabs = slabs; rs.n_splits = ksplit; rs.split_stride = p.block_rows * h;
     rs.row_scale = row_scale; rs.m = (int)rows; rs.h = (int)h;
     rs.out = grad_hidden32 + r0 * h;
+    rs.m_dev = m_dev; rs.row0 = r0;
     if (int rc = launch_reduce_slabs(rs, stream)) return rc;
 
     if (weight_grad) {
@@ -453,6 +489,7 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
       dw.c = grad_weight32; dw.ldc = h; dw.c_rows = (int)v; dw.c_cols = (int)h;
       dw.c_split_stride = 0;
       dw.mode = block == 0 ? kStoreF32 : kAddF32;
+      dw.m_dev = m_dev; dw.m_role = kKFollows; dw.m_round = 64; dw.m_dev_offset = r0;
       if (int rc = launch_gemm<E, true, true>(dw, 1, kClassGradWeight, stream)) return rc;
     }
   }

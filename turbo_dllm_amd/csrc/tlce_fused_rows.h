@@ -17,6 +17,7 @@ __global__ __launch_bounds__(256) void lce_label_logit_kernel(LabelLogitArgs p) 
   const int wave = threadIdx.x >> 6;
   if (threadIdx.x == 0) block_valid = 0;
   __syncthreads();
+  p.m = effective_rows(p.m, p.m_dev);
   int wave_valid = 0;
   for (int i = 0; i < 4; ++i) {
     const int r = blockIdx.x * 16 + wave * 4 + i;
@@ -55,6 +56,10 @@ constexpr int kFusedRowsPerBlock = 64;
 template <typename T>
 __global__ __launch_bounds__(256) void lce_fused_rows_kernel(FusedRowsArgs p) {
   if (p.run_flag != nullptr && *p.run_flag == 0) return;
+  if (p.m_dev != nullptr) {
+    p.m = effective_block_rows(p.m, p.m_dev, p.row0);
+    p.m_pad = min(p.m_pad, (p.m + 255) / 256 * 256);   // the token tiles the producer wrote
+  }
   __shared__ float sh_sum[4][kFusedRowsPerBlock];
   __shared__ float sh_max[4][kFusedRowsPerBlock];
   const int lane = threadIdx.x & 63;
@@ -136,6 +141,12 @@ __global__ __launch_bounds__(256) void lce_fused_rows_kernel(FusedRowsArgs p) {
 
 __global__ __launch_bounds__(256) void lce_reduce_scaled_slabs_kernel(ReduceSlabsArgs p) {
   const int r = blockIdx.x;
+  if (p.m_dev != nullptr) {
+    const int rows = effective_block_rows(p.m, p.m_dev, p.row0);
+    if (r >= rows) return;
+    p.n_splits = dynamic_k_splits((rows + p.tile - 1) / p.tile, p.n_htiles, p.tile, p.h,
+                                  p.launched_splits, p.slab_budget, p.k_steps, &p.split_stride);
+  }
   const float s = p.row_scale[r];
   const float* src = p.slabs + (int64_t)r * p.h;
   float* dst = p.out + (int64_t)r * p.h;
@@ -156,6 +167,7 @@ __global__ __launch_bounds__(256) void lce_scale_cast_rows_kernel(ScaleCastArgs 
     g = count > 0.0f ? g / count : 0.0f;
   }
   const int64_t r = blockIdx.x;
+  if (p.m_dev != nullptr && r >= *p.m_dev) return;
   const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : r;
   const float* src = p.in + r * p.h;
   T* dst = static_cast<T*>(p.out) + o * p.h;

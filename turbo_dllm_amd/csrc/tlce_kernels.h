@@ -1071,6 +1071,7 @@ struct GemmArgs {
   // (grad_weight): k shrinks to the real count rounded up to m_round.
   const int64_t* m_dev = nullptr;
   int m_role = 0, m_round = 1;
+  int64_t m_dev_offset = 0;  // the operand's first token row is row m_dev_offset of the counted rows
   int64_t slab_budget = 0;   // kRowsFollow: float32 elements all K-split slabs may take
   int k_steps_plan = 0;      // kRowsFollow: K steps of a full panel, what the split rule plans on
 };
@@ -1226,15 +1227,17 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
   using T = typename E::T;
   if (p.m_dev != nullptr) {
     if (p.m_role == kRowsFollow) {
-      p.c_rows = effective_rows(p.c_rows, p.m_dev);
+      p.c_rows = effective_block_rows(p.c_rows, p.m_dev, p.m_dev_offset);
       p.nj = (p.c_rows + E::kTile - 1) / E::kTile;
       const int ks = dynamic_k_splits(p.nj, p.ni, E::kTile, (int)p.ldc, (int)gridDim.y,
                                       p.slab_budget, p.k_steps_plan, &p.c_split_stride);
       if ((int)blockIdx.y >= ks) return;
       p.k_per_split = (p.k / E::kBK + ks - 1) / ks * E::kBK;
     } else if (p.m_role == kKFollows) {
-      const int rows = effective_rows(p.k, p.m_dev);
+      const int rows = effective_block_rows(p.k, p.m_dev, p.m_dev_offset);
       p.k = (rows + p.m_round - 1) / p.m_round * p.m_round;
+      // nothing to add to an accumulator that already holds earlier blocks of rows
+      if (p.k == 0 && p.mode == kAddF32) return;
     }
   }
   const int logical = xcd_logical_block_of(blockIdx.x, p.ni * p.nj);

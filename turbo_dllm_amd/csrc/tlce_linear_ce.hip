@@ -704,8 +704,9 @@ extern "C" int64_t tlce_forward_with_gradients_workspace_bytes(int64_t m, int64_
 
 extern "C" int tlce_forward_with_gradients(
     const void* hidden, const void* weight, const int64_t* labels, const int64_t* row_idx,
-    const float* token_weights, int64_t m, int64_t n_out, int64_t h, int64_t v, int dtype,
-    int64_t ignore_index, int64_t exclude_index, float logit_softcap, float logit_multiplier,
+    const float* token_weights, const int64_t* row_count, int64_t m, int64_t n_out, int64_t h,
+    int64_t v, int dtype, int64_t ignore_index, int64_t exclude_index, float logit_softcap,
+    float logit_multiplier,
     float* losses, float* lse, float* valid_count, float* grad_hidden_f32, float* grad_weight_f32,
     int64_t panel_bytes, void* workspace, int64_t workspace_bytes, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -720,6 +721,8 @@ extern "C" int tlce_forward_with_gradients(
                (long long)m);
   TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
                "forward_with_gradients: n_out != m without row_idx");
+  TLCE_REQUIRE(row_count == nullptr || row_idx != nullptr,
+               "forward_with_gradients: a device-side row count needs row_idx");
   TLCE_REQUIRE(((uintptr_t)grad_hidden_f32 & 15) == 0 && ((uintptr_t)grad_weight_f32 & 15) == 0,
                "forward_with_gradients: gradients must be 16-byte aligned");
   // everything that can be refused is refused before the first launch
@@ -745,6 +748,7 @@ extern "C" int tlce_forward_with_gradients(
   FusedOptions opt;
   opt.logit_scale = logit_multiplier;
   opt.token_weights = token_weights;
+  opt.row_count = row_count;
   return fused_gradients_impl<MfmaDirect4Engine<__bf16>>(
       p, hidden, weight, labels, row_idx, m, h, v, dtype, ignore_index, exclude_index,
       logit_softcap, losses, lse, valid_count, grad_hidden_f32, grad_weight_f32,
@@ -752,7 +756,8 @@ extern "C" int tlce_forward_with_gradients(
 }
 
 extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float* grad_weight_f32,
-                                      const int64_t* row_idx, const float* grad_output,
+                                      const int64_t* row_idx, const int64_t* row_count,
+                                      const float* grad_output,
                                       const float* valid_count, int64_t m, int64_t n_out,
                                       int64_t h, int64_t v, int dtype, int reduction_code,
                                       void* grad_hidden, void* grad_weight, void* stream_) {
@@ -766,6 +771,8 @@ extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float*
                (long long)m);
   TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
                "apply_grad_output: n_out != m without row_idx");
+  TLCE_REQUIRE(row_count == nullptr || row_idx != nullptr,
+               "apply_grad_output: a device-side row count needs row_idx");
   TLCE_REQUIRE(grad_hidden != nullptr || n_out == 0, "apply_grad_output: grad_hidden is null");
   TLCE_REQUIRE(grad_output != nullptr, "apply_grad_output: grad_output is null");
   TLCE_REQUIRE(valid_count != nullptr || reduction_code != TLCE_REDUCTION_MEAN,
@@ -785,7 +792,9 @@ extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float*
   if (m > 0) {
     TLCE_REQUIRE(grad_hidden_f32 != nullptr, "apply_grad_output: null pointer");
     a.in = grad_hidden_f32; a.row_idx = row_idx; a.rows = m; a.out = grad_hidden;
+    a.m_dev = row_count;
     if (int rc = launch_scale_cast(a, stream)) return rc;
+    a.m_dev = nullptr;
   }
   if (grad_weight != nullptr) {
     a.in = grad_weight_f32; a.row_idx = nullptr; a.rows = v; a.out = grad_weight;

@@ -67,7 +67,7 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
         # gradients while the logits exist (3 contractions instead of 4), where the
         # library takes the operands and the row count is known to the host
         ctx.fused = (
-            bool(ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) and mode != "device"
+            bool(ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
             and get_gradient_mode() == "forward"
             and native.fused_gradients_supported(rows, weight, bias, False)
         )
@@ -77,9 +77,10 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
                 logit_softcap=logit_softcap, compute_weight_grad=bool(ctx.needs_input_grad[1]),
                 token_weights=None if token_weights is None else token_weights[:m],
                 logit_multiplier=multiplier,
-                row_idx=row_idx, n_out=n,
+                row_idx=row_idx, n_out=n, row_count=row_count if mode == "device" else None,
             )
-            ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx)
+            ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx,
+                                  row_count if mode == "device" else None)
             ctx.hidden_shape = hidden.shape
             ctx.n_rows, ctx.m = n, m
             ctx.grad_dtype, ctx.vocab = hidden.dtype, weight.shape[0]
@@ -103,10 +104,11 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
         from . import chunked_linear_ce_native as native
 
         if ctx.fused:
-            grad_rows32, grad_weight32, valid_count, row_idx = ctx.saved_tensors
+            grad_rows32, grad_weight32, valid_count, row_idx, row_count = ctx.saved_tensors
             grad_hidden, grad_weight = native.apply_grad_output(
                 grad_rows32, grad_weight32, grad_output, valid_count, reduction="sum",
                 dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows, vocab=ctx.vocab,
+                row_count=row_count,
             )
             return (grad_hidden.reshape(ctx.hidden_shape), grad_weight, None) + (None,) * 6
         rows, weight, bias, targets, token_weights, lse, row_idx, row_count = ctx.saved_tensors

@@ -275,7 +275,7 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
     # operands (options.GRADIENT_MODES).
     wants_grad = bool(ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
     ctx.fused = (
-        wants_grad and mode != "device" and reduction in ("mean", "sum")
+        wants_grad and reduction in ("mean", "sum")
         and options.get_gradient_mode() == "forward"
         and native.fused_gradients_supported(rows, weight_vf, bias, in_place or weight_dim_first)
     )
@@ -285,8 +285,10 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
             rows[:m], weight_vf, targets[:m], ignore_index=ignore_index, exclude_index=exclude_index,
             logit_softcap=float(logit_softcap),
             compute_weight_grad=bool(ctx.needs_input_grad[1]), row_idx=row_idx, n_out=n,
+            row_count=row_count if mode == "device" else None,
         )
-        ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx)
+        ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx,
+                              row_count if mode == "device" else None)
         ctx.hidden_shape = hidden.shape
         ctx.n_rows, ctx.m = n, m
         ctx.reduction = reduction
@@ -332,10 +334,11 @@ def _device_backward(ctx, grad_output, frozen: bool):
     from . import chunked_linear_ce_native as native
 
     if ctx.fused:
-        grad_rows32, grad_weight32, valid_count, row_idx = ctx.saved_tensors
+        grad_rows32, grad_weight32, valid_count, row_idx, row_count = ctx.saved_tensors
         grad_hidden, grad_weight = native.apply_grad_output(
             grad_rows32, grad_weight32, grad_output, valid_count, reduction=ctx.reduction,
             dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows, vocab=ctx.vocab,
+            row_count=row_count,
         )
         return (grad_hidden.reshape(ctx.hidden_shape), None if frozen else grad_weight,
                 None) + (None,) * 9
