@@ -58,6 +58,9 @@ def within(name, err, bar):
 HARD_CASES = {
     7954: dict(widen=2.0, measured="3.7e-2 against 2e-2",
                why="bf16, 2 rows, V=3: one rounded gradient entry of magnitude 1e-5"),
+    15338: dict(widen=2.0, measured="2.8e-5 against 2e-5 (bias gradient)",
+                why="float32, 7 rows, V=3, bias, soft cap 30: exp(z - lse) - 1 cancels; found by a "
+                    "second 40 000-draw run, the only draw of it outside the bars"),
     17331: dict(widen=1.0, measured="1.8e-5 against 2e-5",
                 why="float32, 1 row, V=3, soft cap 30: was the tanh approximation"),
     17376: dict(widen=2.0, measured="2.4e-5 against 2e-5",

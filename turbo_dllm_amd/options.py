@@ -32,7 +32,9 @@ import contextvars
 COMPACTION_MODES = ("sync", "device", "none")
 
 _compaction = contextvars.ContextVar("tlce_compaction_mode", default="sync")
-# 0 selects the library default (1 GiB)
+# 0 selects the library default: 2.5 GiB for the panel of exponentiated logits of the
+# forward that leaves the gradients, 1 GiB for the recomputing backward's panel of logit
+# gradients
 _panel_bytes = contextvars.ContextVar("tlce_panel_bytes", default=0)
 
 
@@ -123,7 +125,7 @@ def set_panel_bytes(nbytes: int) -> int:
 
 @contextlib.contextmanager
 def panel_budget(nbytes: int):
-    """Bounds the backward's logit-gradient staging panel inside the block
+    """Bounds the staging panel between the contractions inside the block
     (0 = library default)."""
     if nbytes < 0:
         raise ValueError("panel budget must be >= 0 bytes")
