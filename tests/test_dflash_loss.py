@@ -90,6 +90,9 @@ GPU_CASES = [
     # 1/16 of the drafter shape: 64 sequences x <=1024 tokens, H=4096, V=151936
     ("bf16_sixteenth_shape", torch.bfloat16, 4, 560, 256, 320, 9496, 0.35, None),
     ("bf16_one_sample_unsupervised", torch.bfloat16, 5, 64, 128, 128, 2048, 0.5, 30.0),
+    # H and V multiples of 64: "paper_ce" forms its gradients in the forward (per-row
+    # factors w_r / ((count_b + 1e-5) * B) instead of per-sample numerators)
+    ("bf16_direct_engine", torch.bfloat16, 6, 200, 256, 128, 4160, 0.4, None),
 ]
 
 

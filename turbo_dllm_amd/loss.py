@@ -393,6 +393,20 @@ def dflash_token_loss(
                                           teacher_head.weight, logit_softcap=logit_softcap)
         else:
             targets = gather_rows(target_token_ids.reshape(-1).contiguous(), valid_indices)
+            if (device_path and get_gradient_mode() == "forward"
+                    and (hidden.requires_grad or lm_head.weight.requires_grad)
+                    and native.fused_gradients_supported(hidden, lm_head.weight, None, False)):
+                # The whole reduction is linear in the token losses,
+                #   loss = sum_r token_loss_r * w_r / ((count_{b(r)} + 1e-5) * B),
+                # and its per-row factors depend on the inputs only, so the gradients can
+                # be formed while the logits exist (three contractions instead of four; two
+                # instead of three with a frozen head) and the upstream gradient is a scalar.
+                sample = torch.div(valid_indices, tokens_per_sample, rounding_mode="floor")
+                row_factors = weights / ((denominators[sample] + 1.0e-5) * batch_size)
+                loss = _FusedMaskedTokenLoss.apply(
+                    hidden, lm_head.weight, None, targets, row_factors, 1.0, -1,
+                    0.0 if logit_softcap is None else float(logit_softcap), "none")
+                return loss * float(loss_scale)
             # the rows are compacted and every one of them bears loss
             token_loss = tiled_linear_cross_entropy(
                 hidden, lm_head.weight, targets, reduction="none", dtype=hidden.dtype,
