@@ -528,14 +528,22 @@ def main() -> int:
                  and native.fused_gradients_supported(rows, weight.detach(), None, False))
         on_device = count if args.compaction_mode == "device" else None
         if fused:
+            # as the autograd functions do: one block of rows -> the grad_weight contraction
+            # waits for the upstream gradient and is stored in bf16 at once
+            postpone = native.weight_grad_can_wait(m_rows, h, v, hidden.dtype)
             with _lib.kernel_profile() as prof:
                 out = native.forward_with_gradients(
                     rows[:m_rows], weight.detach(), targets[:m_rows], ignore_index=-100,
                     exclude_index=-1, logit_softcap=softcap, compute_weight_grad=True,
-                    row_idx=row_idx, n_out=n, row_count=on_device)
-                native.apply_grad_output(out[3], out[4], go, out[2], reduction="mean",
-                                         dtype=hidden.dtype, row_idx=row_idx, n_out=n,
-                                         row_count=on_device)
+                    row_idx=row_idx, n_out=n, row_count=on_device,
+                    postpone_weight_grad=postpone)
+                native.apply_grad_output(out[3], None if postpone else out[4], go, out[2],
+                                         reduction="mean", dtype=hidden.dtype, row_idx=row_idx,
+                                         n_out=n, row_count=on_device, vocab=v)
+                if postpone:
+                    native.grad_weight_from_panel(
+                        rows[:m_rows], out[4], go, out[2], reduction="mean", vocab=v,
+                        panel_bytes=options.get_panel_bytes(), row_count=on_device)
             del out
         elif count is not None:
             kw = dict(m=m_rows, row_idx=row_idx, row_count=count, n_out=n, ignore_index=-100,

@@ -488,6 +488,25 @@ int tlce_apply_grad_output(const float* grad_hidden_f32, const float* grad_weigh
                            int64_t h, int64_t v, int dtype, int reduction_code,
                            void* grad_hidden, void* grad_weight, void* stream);
 
+/* One block of rows only (tlce_query_fused_plan: n_blocks == 1): the grad_weight
+ * contraction of tlce_forward_with_gradients postponed until the upstream
+ * gradient is known.  Call the forward with grad_weight_f32 = NULL (as for a
+ * frozen head) on a workspace sized with compute_weight_grad = 1 and keep that
+ * workspace untouched; the panel in it still holds exp(logit - reference) of
+ * every row, so
+ *     grad_weight[v, :] = sum_r panel[r, v] * (g * s_r * hidden[r, :])
+ * (g = grad_output[0], over valid_count[0] for the mean; s_r the row factor the
+ * forward left in the workspace) is stored directly in the input dtype: no
+ * float32 [v, h] accumulator and no pass that scales and rounds it.  m, h, v,
+ * dtype, panel_bytes and row_count as given to the forward.  May be called
+ * again on the same workspace (it rewrites only its own operand area). */
+int tlce_grad_weight_from_panel(const void* hidden, const int64_t* row_count,
+                                const float* grad_output, const float* valid_count,
+                                int64_t m, int64_t h, int64_t v, int dtype,
+                                int reduction_code, void* grad_weight,
+                                int64_t panel_bytes, void* forward_workspace,
+                                int64_t workspace_bytes, void* stream);
+
 /* ---- introspection used by the benchmark and the tests -------------------
  * Tile plan the host scheduler would use for a problem; any pointer may be
  * NULL.  `engine` is 2 for the bf16/f16 MFMA kernels with direct-to-LDS loads

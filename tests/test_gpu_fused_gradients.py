@@ -41,17 +41,29 @@ def make_case(m, h, v, *, seed, dtype=torch.bfloat16, ignored=0.0, std=0.05):
 
 def run_fused(dev, hidden, weight, labels, *, reduction="mean", exclude=-1, softcap=0.0,
               grad_output=0.7, weight_grad=True, token_weights=None, multiplier=1.0,
-              row_idx=None, n_out=None):
+              row_idx=None, n_out=None, postpone=None):
+    """Through the ctypes binding.  postpone: leave the grad_weight contraction to the
+    backward where all rows fit one block (None: whenever that is possible, as the
+    autograd functions do; False: always accumulate it in float32 in the forward)."""
+    m, h = hidden.shape
+    v = weight.shape[0]
+    can_wait = weight_grad and native.weight_grad_can_wait(m, h, v, hidden.dtype)
+    postpone = can_wait if postpone is None else (postpone and can_wait)
+    x = hidden.to(dev)
     out = native.forward_with_gradients(
-        hidden.to(dev), weight.to(dev), labels.to(dev), ignore_index=-100, exclude_index=exclude,
+        x, weight.to(dev), labels.to(dev), ignore_index=-100, exclude_index=exclude,
         logit_softcap=softcap, compute_weight_grad=weight_grad,
         token_weights=None if token_weights is None else token_weights.to(dev),
-        logit_multiplier=multiplier, row_idx=row_idx, n_out=n_out)
+        logit_multiplier=multiplier, row_idx=row_idx, n_out=n_out,
+        postpone_weight_grad=postpone)
     losses, lse, valid, dh32, dw32 = out
     go = torch.tensor([grad_output], device=dev)
-    dh, dw = native.apply_grad_output(dh32, dw32, go, valid, reduction=reduction,
-                                      dtype=hidden.dtype, row_idx=row_idx, n_out=n_out,
-                                      vocab=weight.shape[0])
+    dh, dw = native.apply_grad_output(dh32, None if postpone else dw32, go, valid,
+                                      reduction=reduction, dtype=hidden.dtype, row_idx=row_idx,
+                                      n_out=n_out, vocab=v)
+    if postpone:
+        dw = native.grad_weight_from_panel(x, dw32, go, valid, reduction=reduction, vocab=v,
+                                           panel_bytes=options.get_panel_bytes())
     torch.cuda.synchronize()
     return losses.cpu(), lse.cpu(), float(valid), dh.cpu(), None if dw is None else dw.cpu()
 
@@ -66,8 +78,9 @@ def run_fused(dev, hidden, weight, labels, *, reduction="mean", exclude=-1, soft
     (2048, 1024, 32000, dict(panel=40 << 20)),          # 2 blocks of rows
     (1500, 256, 5120, dict(panel=1, ignored=0.2)),        # one token tile per block, 6 blocks
 ])
-def test_fused_gradients_match_the_oracle(gpu_device, m, h, v, kw):
-    say("fused gradients", m, h, v, kw)
+@pytest.mark.parametrize("postpone", [True, False])
+def test_fused_gradients_match_the_oracle(gpu_device, m, h, v, kw, postpone):
+    say("fused gradients", m, h, v, kw, "postpone", postpone)
     kw = dict(kw)
     dtype = kw.pop("dtype", torch.bfloat16)
     reduction = kw.pop("reduction", "mean")
@@ -80,7 +93,8 @@ def test_fused_gradients_match_the_oracle(gpu_device, m, h, v, kw):
     with options.panel_budget(panel):
         losses, lse, valid, dh, dw = run_fused(
             gpu_device, hidden, weight, labels, reduction=reduction,
-            exclude=-1 if exclude is None else exclude, softcap=softcap or 0.0)
+            exclude=-1 if exclude is None else exclude, softcap=softcap or 0.0,
+            postpone=postpone)
     okw = dict(exclude_index=exclude, logit_softcap=softcap, dtype=torch.float32)
     ref_losses, ref_lse = oracle.dense_linear_ce(hidden, weight, labels, reduction="none",
                                                  return_lse=True, **okw)
@@ -252,6 +266,41 @@ def test_loss_api_takes_the_fused_path_and_agrees_with_recompute(gpu_device, red
     assert abs(a[0] - float(ref)) <= LOSS_RTOL * abs(float(ref))
 
 
+def test_postponed_weight_gradient_twice_and_refusals(gpu_device):
+    """The postponed contraction may run twice on one workspace (retain_graph) with
+    different upstream gradients; it is refused when the forward took several blocks."""
+    say("postponed grad_weight")
+    dev = gpu_device
+    m, h, v = 500, 128, 2048
+    hidden, weight, labels = make_case(m, h, v, seed=71, ignored=0.2)
+    x, w, y = hidden.to(dev), weight.to(dev), labels.to(dev)
+    assert native.weight_grad_can_wait(m, h, v, torch.bfloat16)
+    out = native.forward_with_gradients(x, w, y, ignore_index=-100, exclude_index=-1,
+                                        logit_softcap=0.0, compute_weight_grad=True,
+                                        postpone_weight_grad=True)
+    ws, valid = out[4], out[2]
+    assert ws.dtype == torch.uint8            # the workspace, not a float32 gradient
+    grads = []
+    for g in (1.0, 0.25, 1.0):
+        go = torch.tensor([g], device=dev)
+        grads.append(native.grad_weight_from_panel(x, ws, go, valid, reduction="mean", vocab=v,
+                                                   panel_bytes=0).cpu())
+    assert torch.equal(grads[0], grads[2])
+    assert torch.equal(grads[1].float() * 4, grads[0].float())
+    _, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, torch.tensor(1.0),
+                                             dtype=torch.float32)
+    assert oracle.relative_max_error(grads[0], rdw) <= GRAD_REL_MAX
+    with options.panel_budget(256 * v * 2):          # one token tile per block: two blocks
+        assert not native.weight_grad_can_wait(m, h, v, torch.bfloat16)
+        with pytest.raises(RuntimeError, match="one block"):
+            native.forward_with_gradients(x, w, y, ignore_index=-100, exclude_index=-1,
+                                          logit_softcap=0.0, compute_weight_grad=True,
+                                          postpone_weight_grad=True)
+        with pytest.raises(RuntimeError, match="blocks of rows"):
+            native.grad_weight_from_panel(x, ws, torch.ones(1, device=dev), valid,
+                                          reduction="mean", vocab=v, panel_bytes=256 * v * 2)
+
+
 def test_no_gradient_needed_means_plain_forward(gpu_device):
     say("no grad")
     hidden, weight, labels = make_case(300, 128, 1024, seed=41)
@@ -268,11 +317,13 @@ def test_linear_in_the_upstream_gradient_and_repeatable(gpu_device):
     whole path gives the same bits on every run (no float atomics on the gradients)."""
     say("linearity / determinism")
     hidden, weight, labels = make_case(777, 256, 3072, seed=51, ignored=0.1)
-    a = run_fused(gpu_device, hidden, weight, labels, grad_output=0.5)
-    b = run_fused(gpu_device, hidden, weight, labels, grad_output=1.0)
-    c = run_fused(gpu_device, hidden, weight, labels, grad_output=1.0)
-    assert torch.equal(b[3], c[3]) and torch.equal(b[4], c[4]) and torch.equal(b[0], c[0])
-    assert torch.equal(a[3].float() * 2, b[3].float()) and torch.equal(a[4].float() * 2, b[4].float())
+    for postpone in (True, False):
+        a = run_fused(gpu_device, hidden, weight, labels, grad_output=0.5, postpone=postpone)
+        b = run_fused(gpu_device, hidden, weight, labels, grad_output=1.0, postpone=postpone)
+        c = run_fused(gpu_device, hidden, weight, labels, grad_output=1.0, postpone=postpone)
+        assert torch.equal(b[3], c[3]) and torch.equal(b[4], c[4]) and torch.equal(b[0], c[0])
+        assert torch.equal(a[3].float() * 2, b[3].float())
+        assert torch.equal(a[4].float() * 2, b[4].float())
 
 
 def test_unsupported_operands_are_rejected_before_any_launch(gpu_device):

@@ -122,6 +122,14 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_grad_weight_from_panel": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p,             # hidden row_count grad_output valid
+            c_int64, c_int64, c_int64, c_int, c_int,            # m h v dtype reduction
+            c_void_p, c_int64, c_void_p, c_int64, c_void_p,     # grad_weight panel_bytes ws bytes stream
+        ],
+    ),
     "tlce_apply_grad_output": (
         c_int,
         [

@@ -491,6 +491,7 @@ def forward_with_gradients(
     row_idx: torch.Tensor | None = None,
     n_out: int | None = None,
     row_count: torch.Tensor | None = None,
+    postpone_weight_grad: bool = False,
 ):
     """The forward and, in the same pass over the logits, the float32 gradients of
     ``sum_r token_weights[r] * loss[r]`` (three contractions instead of the four
@@ -502,6 +503,12 @@ def forward_with_gradients(
     loss once the upstream gradient is known.  ``row_count`` (device int64, with
     ``row_idx``): the real number of rows when the operands are sized for a
     capacity, as the "device" compaction mode leaves them.
+
+    ``postpone_weight_grad`` (with ``compute_weight_grad``, when all rows fit one
+    block: ``weight_grad_can_wait``): the grad_weight contraction is left to
+    ``grad_weight_from_panel``, which runs it once the upstream gradient is
+    known and stores it directly in the input dtype.  The last element returned
+    is then the workspace to hand to that call instead of a float32 gradient.
     """
     device = _require_device(hidden, weight, labels, row_idx, token_weights, row_count)
     if not fused_gradients_supported(hidden, weight, None, False):
@@ -531,8 +538,12 @@ def forward_with_gradients(
         lse = torch.empty(m, dtype=torch.float32, device=device)
         valid_count = torch.empty(1, dtype=torch.float32, device=device)
         grad_hidden32 = torch.empty((m, h), dtype=torch.float32, device=device)
+        postpone = bool(postpone_weight_grad and compute_weight_grad)
+        if postpone and not weight_grad_can_wait(m, h, v, hidden.dtype):
+            raise RuntimeError("the weight gradient can be postponed only when all rows fit "
+                               "one block of the forward (weight_grad_can_wait)")
         grad_weight32 = (torch.empty((v, h), dtype=torch.float32, device=device)
-                         if compute_weight_grad else None)
+                         if compute_weight_grad and not postpone else None)
         ws = _workspace(
             lib.tlce_forward_with_gradients_workspace_bytes(
                 m, h, v, code, int(compute_weight_grad), panel),
@@ -550,7 +561,53 @@ def forward_with_gradients(
             ),
             "tlce_forward_with_gradients",
         )
-    return losses, lse, valid_count, grad_hidden32, grad_weight32
+    return losses, lse, valid_count, grad_hidden32, (ws if postpone else grad_weight32)
+
+
+def weight_grad_can_wait(m: int, h: int, v: int, dtype: torch.dtype) -> bool:
+    """Whether ``forward_with_gradients`` takes ``m`` rows as one block under the
+    panel budget in force, so that its grad_weight contraction can be postponed to
+    the backward (``grad_weight_from_panel``)."""
+    if dtype != torch.bfloat16 or not _lib.library().tlce_fused_gradients_supported(
+            h, v, _lib.DTYPE_BF16):
+        return False
+    return _lib.query_fused_plan(m, h, v, _lib.DTYPE_BF16, get_panel_bytes())["n_blocks"] == 1
+
+
+def grad_weight_from_panel(
+    hidden: torch.Tensor,
+    workspace: torch.Tensor,
+    grad_output: torch.Tensor,
+    valid_count: torch.Tensor,
+    *,
+    reduction: str,
+    vocab: int,
+    panel_bytes: int,
+    row_count: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """``grad_weight [V, H]`` in the input dtype from the workspace a
+    ``forward_with_gradients(..., postpone_weight_grad=True)`` call left, times the
+    upstream gradient (over ``valid_count`` for the mean).  ``panel_bytes`` is the
+    panel budget that forward ran under (``get_panel_bytes()`` at that time)."""
+    device = _require_device(hidden, workspace, grad_output, valid_count, row_count)
+    reduction_code = _reduction_code(reduction)
+    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
+    if grad_output.numel() != 1:
+        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected 1")
+    hidden = _dense(hidden)
+    m, h = hidden.shape
+    with torch.cuda.device(device):
+        grad_weight = torch.empty((int(vocab), h), dtype=hidden.dtype, device=device)
+        _lib.check(
+            _lib.library().tlce_grad_weight_from_panel(
+                _ptr(hidden), _ptr(row_count), _ptr(grad_output), _ptr(valid_count),
+                m, h, int(vocab), _dtype_code(hidden), reduction_code,
+                _ptr(grad_weight), int(panel_bytes), workspace.data_ptr(), workspace.numel(),
+                _stream(device),
+            ),
+            "tlce_grad_weight_from_panel",
+        )
+    return grad_weight
 
 
 def apply_grad_output(

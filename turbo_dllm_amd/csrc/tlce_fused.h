@@ -288,7 +288,22 @@ struct ScaleCastArgs {
   const int64_t* m_dev = nullptr;   // device row count: rows past it are not written
 };
 
+// scaled[r, :] = dtype(g * row_scale[r] * hidden[r, :]) with g as in ScaleCastArgs, zero
+// rows from the row count up to m_pad: the K-major operand of a grad_weight
+// contraction that was postponed until the upstream gradient is known.
+struct ScaleRowsArgs {
+  const void* hidden;       // [m, h]
+  const float* row_scale;   // [m]
+  const float* grad_output; // [1]
+  const float* valid_count; // [1], read for the mean reduction only
+  int reduction;
+  int m, m_pad, h;
+  void* out;                // [m_pad, h]
+  const int64_t* m_dev = nullptr;   // device row count (null: m is exact)
+};
+
 int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream);
+int launch_scale_rows(const ScaleRowsArgs& a, hipStream_t stream);
 int launch_fused_rows(const FusedRowsArgs& a, hipStream_t stream);
 int launch_reduce_slabs(const ReduceSlabsArgs& a, hipStream_t stream);
 int launch_scale_cast(const ScaleCastArgs& a, hipStream_t stream);
@@ -496,6 +511,40 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
   return 0;
 }
 
+// The grad_weight contraction of a single-block forward, postponed to the backward:
+// when all rows fit one block the panel still holds every exp(z - c) after the forward,
+// so grad_weight = panel^T . (g * s * hidden) can be formed once the upstream gradient
+// g is known and stored directly in the input dtype: no float32 [v, h] accumulator
+// and no pass that scales and rounds it.  `ws` is the forward's workspace, untouched
+// since (the forward was called without a grad_weight buffer, as for a frozen head,
+// on a workspace sized for one).
+template <class E>
+int deferred_grad_weight_impl(const FusedPlan& p, const void* hidden, int64_t m, int64_t h,
+                              int64_t v, int dtype, const float* grad_output,
+                              const float* valid_count, int reduction, const int64_t* m_dev,
+                              void* grad_weight, char* ws, hipStream_t stream) {
+  using T = typename E::T;
+  const FusedLayout l = fused_layout(p, m, h, dtype, true);
+  const int64_t rows_p = round_up(m, E::kTile);
+  ScaleRowsArgs sa;
+  sa.hidden = hidden; sa.row_scale = reinterpret_cast<const float*>(ws + l.row_scale);
+  sa.grad_output = grad_output; sa.valid_count = valid_count; sa.reduction = reduction;
+  sa.m = (int)m; sa.m_pad = (int)rows_p; sa.h = (int)h;
+  sa.out = ws + l.scaled_hidden; sa.m_dev = m_dev;
+  if (int rc = launch_scale_rows(sa, stream)) return rc;
+  GemmArgs dw;
+  dw.a = ws + l.scaled_hidden; dw.lda = h; dw.a_rows = (int)h;
+  dw.b = ws + l.panel; dw.ldb = p.vp; dw.b_rows = (int)p.vp;
+  dw.k = (int)round_up(m, 64);
+  dw.k_per_split = 0;
+  dw.ni = p.n_htiles; dw.nj = p.n_vtiles;
+  dw.c = static_cast<T*>(grad_weight); dw.ldc = h; dw.c_rows = (int)v; dw.c_cols = (int)h;
+  dw.c_split_stride = 0;
+  dw.mode = kStoreT;
+  dw.m_dev = m_dev; dw.m_role = kKFollows; dw.m_round = 64;
+  return launch_gemm<E, true, true>(dw, 1, kClassGradWeight, stream);
+}
+
 #define TLCE_LAUNCHERS_EXP_PANEL(X, E)                                            \
   X int launch_exp_panel_variant<E, false>(const ExpPanelArgs&, hipStream_t);     \
   X int launch_exp_panel_variant<E, true>(const ExpPanelArgs&, hipStream_t);
@@ -503,6 +552,9 @@ int fused_gradients_impl(const FusedPlan& p, const void* hidden, const void* wei
   X int fused_gradients_impl<E>(const FusedPlan&, const void*, const void*, const int64_t*,      \
                                 const int64_t*, int64_t, int64_t, int64_t, int, int64_t,         \
                                 int64_t, float, float*, float*, float*, float*, float*, char*,   \
-                                hipStream_t, const FusedOptions&);
+                                hipStream_t, const FusedOptions&);                               \
+  X int deferred_grad_weight_impl<E>(const FusedPlan&, const void*, int64_t, int64_t, int64_t,   \
+                                     int, const float*, const float*, int, const int64_t*,       \
+                                     void*, char*, hipStream_t);
 
 }  // namespace tlce

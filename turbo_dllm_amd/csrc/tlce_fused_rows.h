@@ -139,6 +139,39 @@ __global__ __launch_bounds__(256) void lce_fused_rows_kernel(FusedRowsArgs p) {
   }
 }
 
+// One wave per row, 16 rows per workgroup.
+template <typename T>
+__global__ __launch_bounds__(256) void lce_scale_rows_kernel(ScaleRowsArgs p) {
+  float g = p.grad_output[0];
+  if (p.reduction == TLCE_REDUCTION_MEAN) {
+    const float count = p.valid_count[0];
+    g = count > 0.0f ? g / count : 0.0f;
+  }
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int m = effective_rows(p.m, p.m_dev);
+  for (int i = 0; i < 4; ++i) {
+    const int r = blockIdx.x * 16 + wave * 4 + i;
+    if (r >= p.m_pad) return;
+    const float factor = (r < m) ? g * p.row_scale[r] : 0.0f;
+    const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)min(r, max(m - 1, 0)) * p.h;
+    T* out = static_cast<T*>(p.out) + (int64_t)r * p.h;
+    typedef T v8_t __attribute__((ext_vector_type(8)));
+    for (int k = lane * 8; k < p.h; k += 64 * 8) {
+      v8_t y;
+      if (r < m) {
+        const v8_t x = *reinterpret_cast<const v8_t*>(hrow + k);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = from_float<T>(to_float<T>(x[e]) * factor);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) y[e] = from_float<T>(0.0f);
+      }
+      *reinterpret_cast<v8_t*>(out + k) = y;
+    }
+  }
+}
+
 __global__ __launch_bounds__(256) void lce_reduce_scaled_slabs_kernel(ReduceSlabsArgs p) {
   const int r = blockIdx.x;
   if (p.m_dev != nullptr) {

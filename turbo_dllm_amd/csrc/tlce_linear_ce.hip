@@ -82,6 +82,13 @@ int launch_fused_rows(const FusedRowsArgs& a, hipStream_t stream) {
   return 0;
 }
 
+int launch_scale_rows(const ScaleRowsArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_scale_rows_kernel<__bf16><<<(int)ceil_div(a.m_pad, 16), 256, 0, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
 int launch_reduce_slabs(const ReduceSlabsArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassOther, stream);
   lce_reduce_scaled_slabs_kernel<<<a.m, 256, 0, stream>>>(a);
@@ -801,6 +808,42 @@ extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float*
     if (int rc = launch_scale_cast(a, stream)) return rc;
   }
   return 0;
+}
+
+extern "C" int tlce_grad_weight_from_panel(const void* hidden, const int64_t* row_count,
+                                           const float* grad_output, const float* valid_count,
+                                           int64_t m, int64_t h, int64_t v, int dtype,
+                                           int reduction_code, void* grad_weight,
+                                           int64_t panel_bytes, void* forward_workspace,
+                                           int64_t workspace_bytes, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  TLCE_REQUIRE(m >= 0 && h > 0 && v > 0, "grad_weight_from_panel: bad shape");
+  TLCE_REQUIRE(fused_gradients_supported(h, v, dtype),
+               "grad_weight_from_panel: needs bf16 inputs with h and v multiples of 64");
+  TLCE_REQUIRE(reduction_code == TLCE_REDUCTION_SUM || reduction_code == TLCE_REDUCTION_MEAN,
+               "grad_weight_from_panel: the upstream gradient must be a scalar (sum or mean)");
+  TLCE_REQUIRE(grad_weight != nullptr && grad_output != nullptr,
+               "grad_weight_from_panel: null pointer");
+  TLCE_REQUIRE(valid_count != nullptr || reduction_code != TLCE_REDUCTION_MEAN,
+               "grad_weight_from_panel: the mean reduction needs valid_count");
+  TLCE_REQUIRE(((uintptr_t)grad_weight & 15) == 0 && ((uintptr_t)hidden & 15) == 0,
+               "grad_weight_from_panel: operands must be 16-byte aligned");
+  const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
+  TLCE_REQUIRE(p.n_blocks == 1,
+               "grad_weight_from_panel: the forward took %d blocks of rows; the panel holds all "
+               "rows only when there is one", p.n_blocks);
+  if (m == 0) return fill_zero(grad_weight, v * h * dtype_bytes(dtype), stream);
+  TLCE_REQUIRE(hidden != nullptr && forward_workspace != nullptr,
+               "grad_weight_from_panel: null pointer");
+  const int64_t need = fused_layout(p, m, h, dtype, true).total;
+  TLCE_REQUIRE(workspace_bytes >= need,
+               "grad_weight_from_panel: workspace too small (%lld < %lld): size it with "
+               "compute_weight_grad = 1", (long long)workspace_bytes, (long long)need);
+  TLCE_REQUIRE(((uintptr_t)forward_workspace & 255) == 0,
+               "grad_weight_from_panel: workspace must be 256-byte aligned");
+  return deferred_grad_weight_impl<MfmaDirect4Engine<__bf16>>(
+      p, hidden, m, h, v, dtype, grad_output, valid_count, reduction_code, row_count, grad_weight,
+      static_cast<char*>(forward_workspace), stream);
 }
 
 extern "C" int tlce_profile_begin(void) {

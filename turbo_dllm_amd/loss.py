@@ -72,15 +72,21 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
             and native.fused_gradients_supported(rows, weight, bias, False)
         )
         if ctx.fused:
+            rows = rows[:m]
+            ctx.postponed = bool(ctx.needs_input_grad[1]) and native.weight_grad_can_wait(
+                m, rows.shape[1], weight.shape[0], rows.dtype)
             losses, _, valid_count, grad_rows32, grad_weight32 = native.forward_with_gradients(
-                rows[:m], weight, targets[:m], ignore_index=-100, exclude_index=exclude_index,
+                rows, weight, targets[:m], ignore_index=-100, exclude_index=exclude_index,
                 logit_softcap=logit_softcap, compute_weight_grad=bool(ctx.needs_input_grad[1]),
                 token_weights=None if token_weights is None else token_weights[:m],
                 logit_multiplier=multiplier,
                 row_idx=row_idx, n_out=n, row_count=row_count if mode == "device" else None,
+                postpone_weight_grad=ctx.postponed,
             )
             ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx,
-                                  row_count if mode == "device" else None)
+                                  row_count if mode == "device" else None,
+                                  rows if ctx.postponed else None)
+            ctx.panel_bytes = native.get_panel_bytes()
             ctx.hidden_shape = hidden.shape
             ctx.n_rows, ctx.m = n, m
             ctx.grad_dtype, ctx.vocab = hidden.dtype, weight.shape[0]
@@ -104,12 +110,17 @@ class _FusedMaskedTokenLoss(torch.autograd.Function):
         from . import chunked_linear_ce_native as native
 
         if ctx.fused:
-            grad_rows32, grad_weight32, valid_count, row_idx, row_count = ctx.saved_tensors
+            grad_rows32, grad_weight32, valid_count, row_idx, row_count, rows = ctx.saved_tensors
             grad_hidden, grad_weight = native.apply_grad_output(
-                grad_rows32, grad_weight32, grad_output, valid_count, reduction="sum",
-                dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows, vocab=ctx.vocab,
-                row_count=row_count,
+                grad_rows32, None if ctx.postponed else grad_weight32, grad_output, valid_count,
+                reduction="sum", dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows,
+                vocab=ctx.vocab, row_count=row_count,
             )
+            if ctx.postponed:
+                grad_weight = native.grad_weight_from_panel(
+                    rows, grad_weight32, grad_output, valid_count, reduction="sum",
+                    vocab=ctx.vocab, panel_bytes=ctx.panel_bytes, row_count=row_count,
+                )
             return (grad_hidden.reshape(ctx.hidden_shape), grad_weight, None) + (None,) * 6
         rows, weight, bias, targets, token_weights, lse, row_idx, row_count = ctx.saved_tensors
         with native.panel_budget(ctx.panel_bytes):

@@ -281,14 +281,22 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
     )
     if ctx.fused:
         # (rows compacted with the count read back carry up to 63 zero rows of padding)
+        rows, targets = rows[:m], targets[:m]
+        # all rows in one block: the grad_weight contraction waits for the upstream
+        # gradient and is stored in the input dtype at once (no float32 [V, H] buffer)
+        ctx.postponed = bool(ctx.needs_input_grad[1]) and native.weight_grad_can_wait(
+            m, rows.shape[1], weight_vf.shape[0], rows.dtype)
         losses, lse, valid_count, grad_rows32, grad_weight32 = native.forward_with_gradients(
-            rows[:m], weight_vf, targets[:m], ignore_index=ignore_index, exclude_index=exclude_index,
+            rows, weight_vf, targets, ignore_index=ignore_index, exclude_index=exclude_index,
             logit_softcap=float(logit_softcap),
             compute_weight_grad=bool(ctx.needs_input_grad[1]), row_idx=row_idx, n_out=n,
             row_count=row_count if mode == "device" else None,
+            postpone_weight_grad=ctx.postponed,
         )
         ctx.save_for_backward(grad_rows32, grad_weight32, valid_count, row_idx,
-                              row_count if mode == "device" else None)
+                              row_count if mode == "device" else None,
+                              rows if ctx.postponed else None)
+        ctx.panel_bytes = native.get_panel_bytes()
         ctx.hidden_shape = hidden.shape
         ctx.n_rows, ctx.m = n, m
         ctx.reduction = reduction
@@ -334,12 +342,18 @@ def _device_backward(ctx, grad_output, frozen: bool):
     from . import chunked_linear_ce_native as native
 
     if ctx.fused:
-        grad_rows32, grad_weight32, valid_count, row_idx, row_count = ctx.saved_tensors
+        grad_rows32, grad_weight32, valid_count, row_idx, row_count, rows = ctx.saved_tensors
         grad_hidden, grad_weight = native.apply_grad_output(
-            grad_rows32, grad_weight32, grad_output, valid_count, reduction=ctx.reduction,
-            dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows, vocab=ctx.vocab,
-            row_count=row_count,
+            grad_rows32, None if ctx.postponed else grad_weight32, grad_output, valid_count,
+            reduction=ctx.reduction, dtype=ctx.grad_dtype, row_idx=row_idx, n_out=ctx.n_rows,
+            vocab=ctx.vocab, row_count=row_count,
         )
+        if ctx.postponed and not frozen:
+            # grad_weight32 is the forward's workspace: its panel still holds every row
+            grad_weight = native.grad_weight_from_panel(
+                rows, grad_weight32, grad_output, valid_count, reduction=ctx.reduction,
+                vocab=ctx.vocab, panel_bytes=ctx.panel_bytes, row_count=row_count,
+            )
         return (grad_hidden.reshape(ctx.hidden_shape), None if frozen else grad_weight,
                 None) + (None,) * 9
     rows, weight_vf, bias, targets, lse, valid_count, row_idx, row_count = ctx.saved_tensors
