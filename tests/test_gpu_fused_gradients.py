@@ -353,8 +353,10 @@ def test_seeded_sweep_against_the_masked_token_oracle(gpu_device, case):
     """Seeded draws over what the path branches on: rows around tile and block edges,
     blocks of one to three token tiles (or everything in one), soft cap, an excluded
     column that some labels sit on, most rows ignored, per-row weights, a logit
-    multiplier, a frozen head, rows that need the second try.  (4000 draws of this
-    generator were run once on this build: none outside the bars.)"""
+    multiplier, a frozen head, rows that need the second try.  (20 000 draws of this
+    generator, with the row count kept on the device and the postponed grad_weight
+    contraction drawn at random as well, were run once on this build: none outside
+    the bars.)"""
     rnd = random.Random(5000 + case)
     n, h, v = rnd.choice(SWEEP_ROWS), rnd.choice(SWEEP_WIDTHS), rnd.choice(SWEEP_VOCABS)
     softcap = rnd.choice([None, None, 2.0, 30.0])
