@@ -516,6 +516,26 @@ def main() -> int:
     ms_median = per_step[len(per_step) // 2] if per_step else float("nan")
     loss_value = float(loss.detach())
 
+    # the two halves of a step, a few more steps with an event between them (outside the
+    # timed region): with the gradients formed in the forward the backward only scales and
+    # rounds them (and runs the grad_weight contraction when that one was postponed)
+    halves = []
+    for _ in range(min(args.steps, 5)):
+        hidden.grad = None
+        weight.grad = None
+        e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+        e0.record()
+        loss = tiled_linear_cross_entropy(hidden, weight, labels, reduction="mean",
+                                          logit_softcap=wl.logit_softcap, dtype=hidden.dtype,
+                                          weight_layout="vocab_first")
+        e1.record()
+        loss.backward()
+        e2.record()
+        torch.cuda.synchronize()
+        halves.append((e0.elapsed_time(e1), e1.elapsed_time(e2)))
+    forward_ms = _median([a for a, _ in halves])
+    backward_ms = _median([b for _, b in halves])
+
     # per-kernel-class durations of one forward + backward (HIP events on the launch stream;
     # the library calls are made directly so that all of them run on this thread)
     softcap = float(wl.logit_softcap or 0.0)
@@ -636,6 +656,8 @@ def main() -> int:
         "frac_of_bf16_peak_useful": useful_tflops / PEAK_BF16_TFLOPS,
         "mfma_util_executed": executed_tflops / PEAK_BF16_TFLOPS,
         "ms_per_step_median": ms_median,
+        "forward_only_ms": round(forward_ms, 3),
+        "backward_only_ms": round(backward_ms, 3),
         "kernel_ms": {k: round(x, 3) for k, x in prof.ms.items()},
         "kernel_launches": prof.launches,
         "roofline": {

@@ -438,7 +438,8 @@ int tlce_segment_weighted_sum(const float* values, const float* weights,
  * while the logits of a block of rows exist:
  *     grad_hidden_f32[r, :]  = dS / d hidden[r, :]      [m, h] float32, compact rows
  *     grad_weight_f32[v, :]  = dS / d weight[v, :]      [v, h] float32 (NULL: frozen head)
- * and writes losses / lse / valid_count as tlce_forward does (losses unweighted).
+ * and writes losses / lse / valid_count as tlce_forward does (losses unweighted;
+ * lse is 0, not computed, for rows whose label is ignore_index).
  * tlce_apply_grad_output then multiplies both by the upstream gradient
  * (grad_output[0], divided by valid_count[0] for TLCE_REDUCTION_MEAN), rounds
  * them once to the input dtype, and un-compacts grad_hidden through row_idx
