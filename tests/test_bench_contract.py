@@ -23,9 +23,10 @@ def test_more_than_one_gpu_is_refused_with_a_message():
 
 
 @pytest.mark.gpu
-def test_json_line_on_a_small_workload(gpu_device):
+@pytest.mark.parametrize("gradients,contractions", [("forward", 3), ("recompute", 4)])
+def test_json_line_on_a_small_workload(gpu_device, gradients, contractions):
     result = run_bench("--workload", "small_head", "--steps", "3", "--warmup", "1",
-                       "--cpu-rows", "64", "--no-library-gemm")
+                       "--cpu-rows", "64", "--no-library-gemm", "--gradients", gradients)
     assert result.returncode == 0, result.stderr[-2000:]
     lines = [line for line in result.stdout.splitlines() if line.startswith("{")]
     assert len(lines) == 1
@@ -37,6 +38,9 @@ def test_json_line_on_a_small_workload(gpu_device):
     assert record["n_gpus"] == 1 and record["steps"] == 3 and record["warmup"] == 1
     assert record["vs_baseline"] is None and record["higher_is_better"] is True
     assert "workload" in record["config"] and "model" not in record["config"]
+    assert record["config"]["gradients"] == gradients
+    assert record["contractions_executed"] == contractions
+    assert record["forward_only_ms"] > 0 and record["backward_only_ms"] > 0
     roofline = record["roofline"]
     assert roofline["bound"] == "mfma" and roofline["unit"] == "TFLOP/s"
     assert abs(roofline["frac"] - roofline["achieved"] / roofline["peak"]) < 1e-9
