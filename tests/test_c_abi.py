@@ -173,6 +173,34 @@ def test_fused_gradient_entry_points_validate_before_touching_a_gpu():
     assert rc != 0 and "valid_count" in _lib.last_error()
 
 
+def test_postponed_weight_gradient_entry_validates_before_touching_a_gpu():
+    import torch
+
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    from turbo_dllm_amd import options
+
+    lib = _lib.library()
+    fake = 4096
+
+    def call(m=8, h=64, v=128, dtype=_lib.DTYPE_BF16, reduction=_lib.REDUCTION_SUM,
+             panel=0, ws_bytes=1 << 30, valid=fake):
+        return lib.tlce_grad_weight_from_panel(fake, None, fake, valid, m, h, v, dtype, reduction,
+                                               fake, panel, fake, ws_bytes, None)
+
+    assert call(h=72) != 0 and "multiples of 64" in _lib.last_error()
+    assert call(reduction=_lib.REDUCTION_NONE) != 0 and "scalar" in _lib.last_error()
+    assert call(reduction=_lib.REDUCTION_MEAN, valid=None) != 0 and "valid_count" in _lib.last_error()
+    assert call(ws_bytes=16) != 0 and "workspace too small" in _lib.last_error()
+    # 600 rows over a 128-word vocabulary with a one-tile panel: three blocks of rows
+    assert call(m=600, panel=1) != 0 and "blocks of rows" in _lib.last_error()
+    # whether the contraction can wait follows the plan under the budget in force
+    assert native.weight_grad_can_wait(8298, 4096, 151936, torch.bfloat16)
+    assert not native.weight_grad_can_wait(32768, 4096, 151936, torch.bfloat16)
+    assert not native.weight_grad_can_wait(8298, 4096, 151936, torch.float16)
+    with options.panel_budget(1 << 30):
+        assert not native.weight_grad_can_wait(8298, 4096, 151936, torch.bfloat16)
+
+
 def test_fused_plan_blocks():
     # the benchmark's shape: 2.5 GiB hold 34 token tiles over 594 vocabulary tiles; four
     # balanced blocks of 32 tiles (whole rounds of 256 workgroups for grad_hidden)
