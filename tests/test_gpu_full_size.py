@@ -206,6 +206,34 @@ def test_headline_shape_gradients_formed_in_the_forward(gpu_device):
     assert torch.equal(dw2.float(), dw.float() * 2.0)
 
 
+def test_headline_shape_in_one_block_with_a_panel_beyond_2_31_entries(gpu_device):
+    """A panel budget that lets all 32768 rows form one block: the panel then has
+    4.98e9 entries (9.96 GB), so every row offset into it must be formed in 64 bits,
+    and the grad_weight contraction is the one postponed to the backward.  Compared on
+    every entry with the default plan (four blocks), which the test above holds to the
+    oracle: the two differ only by where sums are rounded."""
+    from turbo_dllm_amd import _lib, options
+    wl = workloads.block_diffusion_shard(seed=0, all_rows_loss_bearing=True)
+    n, v = wl.n_rows, wl.weight.shape[0]
+    budget = 10 << 30
+    plan = _lib.query_fused_plan(n, 4096, v, _lib.DTYPE_BF16, budget)
+    say("plan", plan)
+    assert plan["n_blocks"] == 1 and plan["block_rows"] * v > 2 ** 31
+    with options.panel_budget(budget):
+        loss1, dh1, dw1 = run(gpu_device, wl, reduction="mean")
+    loss4, dh4, dw4 = run(gpu_device, wl, reduction="mean")
+    say("mean loss", float(loss1), float(loss4))
+    assert abs(float(loss1) - float(loss4)) <= 1e-5 * abs(float(loss4))
+    assert bool(torch.isfinite(dh1.float()).all()) and bool(torch.isfinite(dw1.float()).all())
+    err_h = oracle.relative_max_error(dh1, dh4.float())
+    err_w = oracle.relative_max_error(dw1, dw4.float())
+    say("one block against four: grad_hidden", f"{err_h:.2e}", "grad_weight", f"{err_w:.2e}")
+    assert err_h <= 1e-2 and err_w <= 1e-2
+    # the last rows and the last vocabulary rows sit at the largest offsets
+    assert oracle.relative_max_error(dh1[-256:], dh4[-256:].float()) <= 1e-2
+    assert oracle.relative_max_error(dw1[-256:], dw4[-256:].float()) <= 1e-2
+
+
 def test_block_diffusion_shard_full_size_gradients_formed_in_the_forward(gpu_device):
     check_configuration_full_size(gpu_device, workloads.block_diffusion_shard(seed=6),
                                   reduction="mean")
