@@ -1089,6 +1089,10 @@ __device__ __forceinline__ int dynamic_k_splits(int n_ttiles, int n_htiles, int 
   return ks;
 }
 enum { kRowsFollow = 1, kKFollows = 2 };
+// Output tiles per K split below which lce_gemm_nt_kernel orders its workgroups
+// split-major over the XCDs (measured: 20 tiles x 12 splits 150 -> 85 us; 112 tiles x
+// 2 splits 1.78 -> 1.84 ms, hence not there).
+constexpr int kSplitMajorBelowTiles = 64;
 
 // Output stage of the contraction kernels for the direct engine: the accumulator
 // tile leaves through LDS (free after the main loop) in whole output rows, so that
@@ -1225,14 +1229,14 @@ template <class E, bool kAKMajor, bool kBKMajor>
 __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
+  int n_splits = gridDim.y;
   if (p.m_dev != nullptr) {
     if (p.m_role == kRowsFollow) {
       p.c_rows = effective_block_rows(p.c_rows, p.m_dev, p.m_dev_offset);
       p.nj = (p.c_rows + E::kTile - 1) / E::kTile;
-      const int ks = dynamic_k_splits(p.nj, p.ni, E::kTile, (int)p.ldc, (int)gridDim.y,
-                                      p.slab_budget, p.k_steps_plan, &p.c_split_stride);
-      if ((int)blockIdx.y >= ks) return;
-      p.k_per_split = (p.k / E::kBK + ks - 1) / ks * E::kBK;
+      n_splits = dynamic_k_splits(p.nj, p.ni, E::kTile, (int)p.ldc, (int)gridDim.y,
+                                  p.slab_budget, p.k_steps_plan, &p.c_split_stride);
+      p.k_per_split = (p.k / E::kBK + n_splits - 1) / n_splits * E::kBK;
     } else if (p.m_role == kKFollows) {
       const int rows = effective_block_rows(p.k, p.m_dev, p.m_dev_offset);
       p.k = (rows + p.m_round - 1) / p.m_round * p.m_round;
@@ -1240,16 +1244,38 @@ __global__ __launch_bounds__(E::kThreads) void lce_gemm_nt_kernel(GemmArgs p) {
       if (p.k == 0 && p.mode == kAddF32) return;
     }
   }
-  const int logical = xcd_logical_block_of(blockIdx.x, p.ni * p.nj);
-  if (logical < 0) return;
+  int logical, split;
+  const int tiles = p.ni * p.nj;
+  if (gridDim.y == 1 || tiles >= kSplitMajorBelowTiles) {
+    // every split deals its tiles to the 8 XCDs in contiguous runs of tiles / 8
+    split = blockIdx.y;
+    if (split >= n_splits) return;
+    logical = xcd_logical_block_of(blockIdx.x, tiles);
+    if (logical < 0) return;
+  } else {
+    // Few output tiles under many K splits (a small head, the last rows of a call
+    // whose row count is on the device): a run of tiles / 8 would be 2 or 3 tiles, and
+    // all 8 XCDs would fetch every K range of both operands.  The (split, tile) pairs
+    // in split-major order are dealt to the XCDs in 8 contiguous, equally long runs
+    // instead, so the tiles that stream one K range sit on one XCD (or two) and share
+    // it through that L2.
+    const int total = n_splits * tiles;
+    const int flat = blockIdx.y * gridDim.x + blockIdx.x;   // gridDim.x is a multiple of 8
+    const int xcd = flat % kXcds, slot = flat / kXcds;
+    const int first = (int)((int64_t)xcd * total / kXcds);
+    const int last = (int)((int64_t)(xcd + 1) * total / kXcds);
+    if (slot >= last - first) return;
+    split = (first + slot) / tiles;
+    logical = (first + slot) - split * tiles;
+  }
   int ti, tj;
   grouped_tile(logical, p.ni, p.nj, 4, &ti, &tj);
   // each K split owns its own output slab: no atomics, reproducible sums; a
   // split whose K range is empty still writes its (zero) tile
-  const int k_begin = blockIdx.y * p.k_per_split;
+  const int k_begin = split * p.k_per_split;
   const int k_end = min(p.k, k_begin + p.k_per_split);
   p.c = static_cast<char*>(p.c) +
-        (int64_t)blockIdx.y * p.c_split_stride * (p.mode == kStoreT ? sizeof(T) : sizeof(float));
+        (int64_t)split * p.c_split_stride * (p.mode == kStoreT ? sizeof(T) : sizeof(float));
 
   E eng;
   typename E::Acc acc;
