@@ -443,7 +443,13 @@ int tlce_segment_weighted_sum(const float* values, const float* weights,
  * tlce_apply_grad_output then multiplies both by the upstream gradient
  * (grad_output[0], divided by valid_count[0] for TLCE_REDUCTION_MEAN), rounds
  * them once to the input dtype, and un-compacts grad_hidden through row_idx
- * into [n_out, h] (other rows zero).  No bias, head stored [v, h], bf16 inputs
+ * into [n_out, h] (other rows zero).  With TLCE_REDUCTION_NONE the upstream
+ * gradient is one float per output row, grad_output[n_out] (row r of the compact
+ * rows reads grad_output[row_idx[r]]): call the forward without token_weights;
+ * grad_hidden rows are scaled one by one, and grad_weight, which needs the
+ * upstream gradient inside its contraction, is only available through
+ * tlce_grad_weight_from_panel, i.e. when all rows form one block
+ * (grad_weight_f32 must be NULL here).  No bias, head stored [v, h], bf16 inputs
  * with h and v multiples of 64 (tlce_fused_gradients_supported); everything else
  * goes through tlce_forward / tlce_backward (f16 included: its exponent range
  * cannot hold exp(logit - reference) and the row sums of it).
@@ -496,13 +502,14 @@ int tlce_apply_grad_output(const float* grad_hidden_f32, const float* grad_weigh
  * workspace untouched; the panel in it still holds exp(logit - reference) of
  * every row, so
  *     grad_weight[v, :] = sum_r panel[r, v] * (g * s_r * hidden[r, :])
- * (g = grad_output[0], over valid_count[0] for the mean; s_r the row factor the
- * forward left in the workspace) is stored directly in the input dtype: no
+ * (g = grad_output[0], over valid_count[0] for the mean; grad_output[row_idx[r]],
+ * or grad_output[r] without row_idx, for TLCE_REDUCTION_NONE; s_r the row factor
+ * the forward left in the workspace) is stored directly in the input dtype: no
  * float32 [v, h] accumulator and no pass that scales and rounds it.  m, h, v,
- * dtype, panel_bytes and row_count as given to the forward.  May be called
+ * dtype, panel_bytes, row_idx and row_count as given to the forward.  May be called
  * again on the same workspace (it rewrites only its own operand area). */
-int tlce_grad_weight_from_panel(const void* hidden, const int64_t* row_count,
-                                const float* grad_output, const float* valid_count,
+int tlce_grad_weight_from_panel(const void* hidden, const int64_t* row_idx,
+                                const int64_t* row_count, const float* grad_output, const float* valid_count,
                                 int64_t m, int64_t h, int64_t v, int dtype,
                                 int reduction_code, void* grad_weight,
                                 int64_t panel_bytes, void* forward_workspace,

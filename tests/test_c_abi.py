@@ -161,10 +161,13 @@ def test_fused_gradient_entry_points_validate_before_touching_a_gpu():
     assert forward(n_out=4) != 0 and "n_out" in _lib.last_error()
     assert forward(n_out=16) != 0 and "without row_idx" in _lib.last_error()
     assert forward(row_count=fake) != 0 and "needs row_idx" in _lib.last_error()
-    # the upstream gradient must be one number
+    # one upstream gradient per row: grad_weight cannot be finished from a float32 sum
     rc = lib.tlce_apply_grad_output(fake, fake, None, None, fake, fake, 8, 8, 64, 128,
                                     _lib.DTYPE_BF16, _lib.REDUCTION_NONE, fake, fake, None)
-    assert rc != 0 and "scalar" in _lib.last_error()
+    assert rc != 0 and "has to wait" in _lib.last_error()
+    rc = lib.tlce_apply_grad_output(fake, None, None, None, fake, fake, 8, 8, 64, 128,
+                                    _lib.DTYPE_BF16, 7, fake, None, None)
+    assert rc != 0 and "unknown reduction" in _lib.last_error()
     rc = lib.tlce_apply_grad_output(fake, None, None, None, fake, fake, 8, 8, 64, 128,
                                     _lib.DTYPE_BF16, _lib.REDUCTION_SUM, fake, fake, None)
     assert rc != 0 and "go together" in _lib.last_error()
@@ -184,11 +187,11 @@ def test_postponed_weight_gradient_entry_validates_before_touching_a_gpu():
 
     def call(m=8, h=64, v=128, dtype=_lib.DTYPE_BF16, reduction=_lib.REDUCTION_SUM,
              panel=0, ws_bytes=1 << 30, valid=fake):
-        return lib.tlce_grad_weight_from_panel(fake, None, fake, valid, m, h, v, dtype, reduction,
-                                               fake, panel, fake, ws_bytes, None)
+        return lib.tlce_grad_weight_from_panel(fake, None, None, fake, valid, m, h, v, dtype,
+                                               reduction, fake, panel, fake, ws_bytes, None)
 
     assert call(h=72) != 0 and "multiples of 64" in _lib.last_error()
-    assert call(reduction=_lib.REDUCTION_NONE) != 0 and "scalar" in _lib.last_error()
+    assert call(reduction=7) != 0 and "unknown reduction" in _lib.last_error()
     assert call(reduction=_lib.REDUCTION_MEAN, valid=None) != 0 and "valid_count" in _lib.last_error()
     assert call(ws_bytes=16) != 0 and "workspace too small" in _lib.last_error()
     # 600 rows over a 128-word vocabulary with a one-tile panel: three blocks of rows

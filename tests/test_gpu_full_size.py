@@ -28,15 +28,20 @@ def say(*parts):
     print("[case]", *parts, flush=True)
 
 
-def run(dev, wl, grad_scale=1.0, reduction="none"):
-    """Forward + backward through the public operator.  reduction "none" with a
-    per-row upstream gradient goes through the backward that recomputes the logits;
-    "mean" through the forward that forms the gradients while the logits exist."""
+def run(dev, wl, grad_scale=1.0, reduction="none", gradients=None):
+    """Forward + backward through the public operator.  gradients: the gradient mode
+    (options.GRADIENT_MODES); by default reduction "none" is run through the backward
+    that recomputes the logits and "mean" through the forward that forms the gradients
+    while the logits exist, so that the tests below cover both at full size."""
+    from turbo_dllm_amd import options
+    if gradients is None:
+        gradients = "recompute" if reduction == "none" else "forward"
     hidden = wl.hidden.to(dev).requires_grad_(True)
     weight = wl.weight.to(dev).requires_grad_(True)
-    losses = tiled_linear_cross_entropy(hidden, weight, wl.labels.to(dev), reduction=reduction,
-                                        logit_softcap=wl.logit_softcap, dtype=hidden.dtype,
-                                        weight_layout="vocab_first")
+    with options.gradient_mode(gradients):
+        losses = tiled_linear_cross_entropy(hidden, weight, wl.labels.to(dev),
+                                            reduction=reduction, logit_softcap=wl.logit_softcap,
+                                            dtype=hidden.dtype, weight_layout="vocab_first")
     m = max(wl.n_loss_rows, 1)
     if reduction == "none":
         losses.backward(torch.full_like(losses, grad_scale / m))
@@ -106,7 +111,7 @@ def test_block_diffusion_labels_compaction_full_size(gpu_device):
 
 # ------------------------------------------------- remaining configurations ----
 def check_configuration_full_size(dev, wl, *, check_column_sums=True, token_rows=None,
-                                  vocab_rows=None, reduction="none"):
+                                  vocab_rows=None, reduction="none", gradients=None):
     """One benchmark configuration at full size against the float32 oracle.
 
     The oracle's per-row loss and lse are computed for every loss-bearing row (in
@@ -120,7 +125,7 @@ def check_configuration_full_size(dev, wl, *, check_column_sums=True, token_rows
     h, v = wl.hidden.shape[1], wl.weight.shape[0]
     cap = wl.logit_softcap
     say(wl.name, "N", n, "M", m, "H", h, "V", v, "softcap", cap)
-    losses, dh, dw = run(dev, wl, reduction=reduction)
+    losses, dh, dw = run(dev, wl, reduction=reduction, gradients=gradients)
     say("device done")
     keep = wl.labels != -100
     rows = torch.nonzero(keep).flatten()
@@ -237,6 +242,15 @@ def test_headline_shape_in_one_block_with_a_panel_beyond_2_31_entries(gpu_device
 def test_block_diffusion_shard_full_size_gradients_formed_in_the_forward(gpu_device):
     check_configuration_full_size(gpu_device, workloads.block_diffusion_shard(seed=6),
                                   reduction="mean")
+
+
+def test_block_diffusion_shard_full_size_per_token_losses_gradients_formed_in_the_forward(
+        gpu_device):
+    """Per-token losses (reduction "none") as the reference's call sites ask for them:
+    one block of rows, grad_hidden rows scaled in the backward, grad_weight contracted
+    there from the panel the forward left."""
+    check_configuration_full_size(gpu_device, workloads.block_diffusion_shard(seed=6),
+                                  reduction="none", gradients="forward")
 
 
 def test_gemma_softcap_head_full_size_gradients_formed_in_the_forward(gpu_device):

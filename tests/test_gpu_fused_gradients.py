@@ -266,6 +266,75 @@ def test_loss_api_takes_the_fused_path_and_agrees_with_recompute(gpu_device, red
     assert abs(a[0] - float(ref)) <= LOSS_RTOL * abs(float(ref))
 
 
+@pytest.mark.parametrize("compaction", ["sync", "device", "none"])
+@pytest.mark.parametrize("frozen,tiles_per_block,softcap", [
+    (False, 0, None),      # trainable head, all rows in one block: grad_weight in the backward
+    (False, 0, 20.0),
+    (True, 0, None),
+    (True, 1, None),       # frozen head: any number of blocks
+    (False, 1, None),      # trainable head over several blocks: recomputing backward
+])
+def test_per_token_losses_with_one_upstream_gradient_per_row(gpu_device, compaction, frozen,
+                                                             tiles_per_block, softcap):
+    """reduction "none" with a different upstream gradient on every row (the reference's
+    call sites: per-token losses times loss weights, summed by the caller).  grad_hidden
+    rows are scaled one by one in the backward; grad_weight is the contraction postponed
+    to the backward, which takes the per-row gradients into its operand.  Against the
+    float32 oracle; which path ran is read from the library's per-class launch counts."""
+    say("per-token losses", compaction, frozen, tiles_per_block, softcap)
+    dev = gpu_device
+    m, h, v = 700, 128, 2048
+    hidden, weight, labels = make_case(m, h, v, seed=83, ignored=0.35)
+    gen = torch.Generator().manual_seed(84)
+    go = torch.randn(m, generator=gen)
+    go[5] = 0.0
+    x = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(not frozen)
+    budget = tiles_per_block * 256 * v * 2
+    with options.panel_budget(budget), _lib.kernel_profile() as prof:
+        losses = tiled_linear_cross_entropy(x, w, labels.to(dev), reduction="none",
+                                            logit_softcap=softcap, dtype=torch.bfloat16,
+                                            weight_layout="vocab_first", compaction=compaction)
+        losses.backward(go.to(dev))
+        torch.cuda.synchronize()
+    fused = frozen or tiles_per_block == 0
+    assert (prof.launches["exp_logits_panel"] > 0) == fused
+    assert (prof.launches["forward_stats"] == 0) == fused
+    ref = oracle.dense_linear_ce(hidden, weight, labels, reduction="none", logit_softcap=softcap,
+                                 dtype=torch.float32)
+    torch.testing.assert_close(losses.detach().cpu(), ref, rtol=LOSS_RTOL, atol=1e-4)
+    rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, go, reduction="none",
+                                               logit_softcap=softcap, dtype=torch.float32)
+    keep = labels != -100
+    assert torch.count_nonzero(x.grad.cpu()[~keep]) == 0
+    assert torch.count_nonzero(x.grad.cpu()[5]) == 0
+    assert oracle.relative_max_error(x.grad, rdh) <= GRAD_REL_MAX
+    if not frozen:
+        assert oracle.relative_max_error(w.grad, rdw) <= GRAD_REL_MAX
+
+
+def test_per_token_losses_backward_twice(gpu_device):
+    """retain_graph: the second backward brings other per-row gradients and gets the
+    gradients that belong to them."""
+    say("per-token losses, two backwards")
+    dev = gpu_device
+    m, h, v = 300, 64, 1024
+    hidden, weight, labels = make_case(m, h, v, seed=85, ignored=0.2)
+    x = hidden.to(dev).requires_grad_(True)
+    w = weight.to(dev).requires_grad_(True)
+    losses = tiled_linear_cross_entropy(x, w, labels.to(dev), reduction="none",
+                                        dtype=torch.bfloat16, weight_layout="vocab_first")
+    gen = torch.Generator().manual_seed(86)
+    for _ in range(2):
+        go = torch.rand(m, generator=gen)
+        x.grad = w.grad = None
+        losses.backward(go.to(dev), retain_graph=True)
+        rdh, rdw, _ = oracle.dense_linear_ce_grads(hidden, weight, labels, go, reduction="none",
+                                                   dtype=torch.float32)
+        assert oracle.relative_max_error(x.grad, rdh) <= GRAD_REL_MAX
+        assert oracle.relative_max_error(w.grad, rdw) <= GRAD_REL_MAX
+
+
 def test_postponed_weight_gradient_twice_and_refusals(gpu_device):
     """The postponed contraction may run twice on one workspace (retain_graph) with
     different upstream gradients; it is refused when the forward took several blocks."""

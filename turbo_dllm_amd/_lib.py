@@ -125,7 +125,8 @@ SIGNATURES = {
     "tlce_grad_weight_from_panel": (
         c_int,
         [
-            c_void_p, c_void_p, c_void_p, c_void_p,             # hidden row_count grad_output valid
+            c_void_p, c_void_p, c_void_p,                       # hidden row_idx row_count
+            c_void_p, c_void_p,                                 # grad_output valid_count
             c_int64, c_int64, c_int64, c_int, c_int,            # m h v dtype reduction
             c_void_p, c_int64, c_void_p, c_int64, c_void_p,     # grad_weight panel_bytes ws bytes stream
         ],

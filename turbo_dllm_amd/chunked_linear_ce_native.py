@@ -574,6 +574,16 @@ def weight_grad_can_wait(m: int, h: int, v: int, dtype: torch.dtype) -> bool:
     return _lib.query_fused_plan(m, h, v, _lib.DTYPE_BF16, get_panel_bytes())["n_blocks"] == 1
 
 
+def _upstream_gradient(grad_output: torch.Tensor, reduction_code: int, n_out: int) -> torch.Tensor:
+    """The upstream gradient as the library reads it: float32, one element for a
+    scalar reduction, one per output row for reduction "none"."""
+    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
+    expected = n_out if reduction_code == _lib.REDUCTION_NONE else 1
+    if grad_output.numel() != expected:
+        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected {expected}")
+    return grad_output
+
+
 def grad_weight_from_panel(
     hidden: torch.Tensor,
     workspace: torch.Tensor,
@@ -584,24 +594,27 @@ def grad_weight_from_panel(
     vocab: int,
     panel_bytes: int,
     row_count: torch.Tensor | None = None,
+    row_idx: torch.Tensor | None = None,
+    n_out: int | None = None,
 ) -> torch.Tensor:
     """``grad_weight [V, H]`` in the input dtype from the workspace a
     ``forward_with_gradients(..., postpone_weight_grad=True)`` call left, times the
-    upstream gradient (over ``valid_count`` for the mean).  ``panel_bytes`` is the
-    panel budget that forward ran under (``get_panel_bytes()`` at that time)."""
-    device = _require_device(hidden, workspace, grad_output, valid_count, row_count)
+    upstream gradient (over ``valid_count`` for the mean; for reduction "none" one
+    value per output row, ``n_out`` of them, row ``r`` of ``hidden`` taking the one at
+    ``row_idx[r]``).  ``panel_bytes`` is the panel budget that forward ran under
+    (``get_panel_bytes()`` at that time)."""
+    device = _require_device(hidden, workspace, grad_output, valid_count, row_count, row_idx)
     reduction_code = _reduction_code(reduction)
-    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
-    if grad_output.numel() != 1:
-        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected 1")
     hidden = _dense(hidden)
     m, h = hidden.shape
+    grad_output = _upstream_gradient(grad_output, reduction_code,
+                                     m if n_out is None else int(n_out))
     with torch.cuda.device(device):
         grad_weight = torch.empty((int(vocab), h), dtype=hidden.dtype, device=device)
         _lib.check(
             _lib.library().tlce_grad_weight_from_panel(
-                _ptr(hidden), _ptr(row_count), _ptr(grad_output), _ptr(valid_count),
-                m, h, int(vocab), _dtype_code(hidden), reduction_code,
+                _ptr(hidden), _ptr(row_idx), _ptr(row_count), _ptr(grad_output),
+                _ptr(valid_count), m, h, int(vocab), _dtype_code(hidden), reduction_code,
                 _ptr(grad_weight), int(panel_bytes), workspace.data_ptr(), workspace.numel(),
                 _stream(device),
             ),
@@ -625,17 +638,15 @@ def apply_grad_output(
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """``(grad_hidden [n_out, H], grad_weight [V, H] or None)`` in ``dtype``: the
     float32 gradients ``forward_with_gradients`` left, times the upstream gradient
-    (over ``valid_count`` for the mean), each entry rounded once."""
+    (over ``valid_count`` for the mean), each entry rounded once.  For reduction
+    "none" the upstream gradient has one value per output row and only grad_hidden
+    can be finished here (``grad_weight32`` must be None: ``grad_weight_from_panel``)."""
     device = _require_device(grad_hidden32, grad_weight32, grad_output, valid_count, row_idx)
     reduction_code = _reduction_code(reduction)
-    if reduction_code == _lib.REDUCTION_NONE:
-        raise RuntimeError("apply_grad_output needs a scalar upstream gradient (sum or mean)")
-    grad_output = grad_output.reshape(-1).to(torch.float32).contiguous()
-    if grad_output.numel() != 1:
-        raise RuntimeError(f"grad_output has {grad_output.numel()} elements, expected 1")
     m, h = grad_hidden32.shape
     v = grad_weight32.shape[0] if grad_weight32 is not None else int(vocab or 1)
     n_out = m if n_out is None else int(n_out)
+    grad_output = _upstream_gradient(grad_output, reduction_code, n_out)
     if dtype != torch.bfloat16:
         raise RuntimeError("apply_grad_output writes bf16 gradients only")
     code = _lib.DTYPE_BF16

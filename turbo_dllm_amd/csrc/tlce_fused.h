@@ -279,7 +279,7 @@ struct ReduceSlabsArgs {
 struct ScaleCastArgs {
   const float* in;          // [rows, h]
   const int64_t* row_idx;   // or null
-  const float* grad_output; // [1]
+  const float* grad_output; // [1]; reduction none: one per output row, read at row_idx[r]
   const float* valid_count; // [1], read for the mean reduction only
   int reduction;
   int64_t rows;
@@ -294,12 +294,13 @@ struct ScaleCastArgs {
 struct ScaleRowsArgs {
   const void* hidden;       // [m, h]
   const float* row_scale;   // [m]
-  const float* grad_output; // [1]
+  const float* grad_output; // [1]; reduction none: one per output row, read at row_idx[r]
   const float* valid_count; // [1], read for the mean reduction only
   int reduction;
   int m, m_pad, h;
   void* out;                // [m_pad, h]
   const int64_t* m_dev = nullptr;   // device row count (null: m is exact)
+  const int64_t* row_idx = nullptr; // output row of row r (null: r)
 };
 
 int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream);
@@ -522,7 +523,8 @@ template <class E>
 int deferred_grad_weight_impl(const FusedPlan& p, const void* hidden, int64_t m, int64_t h,
                               int64_t v, int dtype, const float* grad_output,
                               const float* valid_count, int reduction, const int64_t* m_dev,
-                              void* grad_weight, char* ws, hipStream_t stream) {
+                              const int64_t* row_idx, void* grad_weight, char* ws,
+                              hipStream_t stream) {
   using T = typename E::T;
   const FusedLayout l = fused_layout(p, m, h, dtype, true);
   const int64_t rows_p = round_up(m, E::kTile);
@@ -530,7 +532,7 @@ int deferred_grad_weight_impl(const FusedPlan& p, const void* hidden, int64_t m,
   sa.hidden = hidden; sa.row_scale = reinterpret_cast<const float*>(ws + l.row_scale);
   sa.grad_output = grad_output; sa.valid_count = valid_count; sa.reduction = reduction;
   sa.m = (int)m; sa.m_pad = (int)rows_p; sa.h = (int)h;
-  sa.out = ws + l.scaled_hidden; sa.m_dev = m_dev;
+  sa.out = ws + l.scaled_hidden; sa.m_dev = m_dev; sa.row_idx = row_idx;
   if (int rc = launch_scale_rows(sa, stream)) return rc;
   GemmArgs dw;
   dw.a = ws + l.scaled_hidden; dw.lda = h; dw.a_rows = (int)h;
@@ -555,6 +557,6 @@ int deferred_grad_weight_impl(const FusedPlan& p, const void* hidden, int64_t m,
                                 hipStream_t, const FusedOptions&);                               \
   X int deferred_grad_weight_impl<E>(const FusedPlan&, const void*, int64_t, int64_t, int64_t,   \
                                      int, const float*, const float*, int, const int64_t*,       \
-                                     void*, char*, hipStream_t);
+                                     const int64_t*, void*, char*, hipStream_t);
 
 }  // namespace tlce

@@ -142,7 +142,8 @@ __global__ __launch_bounds__(256) void lce_fused_rows_kernel(FusedRowsArgs p) {
 // One wave per row, 16 rows per workgroup.
 template <typename T>
 __global__ __launch_bounds__(256) void lce_scale_rows_kernel(ScaleRowsArgs p) {
-  float g = p.grad_output[0];
+  float g = 0.0f;
+  if (p.reduction != TLCE_REDUCTION_NONE) g = p.grad_output[0];
   if (p.reduction == TLCE_REDUCTION_MEAN) {
     const float count = p.valid_count[0];
     g = count > 0.0f ? g / count : 0.0f;
@@ -153,6 +154,8 @@ __global__ __launch_bounds__(256) void lce_scale_rows_kernel(ScaleRowsArgs p) {
   for (int i = 0; i < 4; ++i) {
     const int r = blockIdx.x * 16 + wave * 4 + i;
     if (r >= p.m_pad) return;
+    if (p.reduction == TLCE_REDUCTION_NONE && r < m)
+      g = p.grad_output[p.row_idx != nullptr ? p.row_idx[r] : (int64_t)r];
     const float factor = (r < m) ? g * p.row_scale[r] : 0.0f;
     const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)min(r, max(m - 1, 0)) * p.h;
     T* out = static_cast<T*>(p.out) + (int64_t)r * p.h;
@@ -193,15 +196,15 @@ __global__ __launch_bounds__(256) void lce_reduce_scaled_slabs_kernel(ReduceSlab
 
 template <typename T>
 __global__ __launch_bounds__(256) void lce_scale_cast_rows_kernel(ScaleCastArgs p) {
-  float g = p.grad_output[0];
+  const int64_t r = blockIdx.x;
+  if (p.m_dev != nullptr && r >= *p.m_dev) return;
+  const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : r;
+  float g = p.grad_output[p.reduction == TLCE_REDUCTION_NONE ? o : 0];
   if (p.reduction == TLCE_REDUCTION_MEAN) {
     // no row with a loss: every gradient entry is zero and stays zero
     const float count = p.valid_count[0];
     g = count > 0.0f ? g / count : 0.0f;
   }
-  const int64_t r = blockIdx.x;
-  if (p.m_dev != nullptr && r >= *p.m_dev) return;
-  const int64_t o = (p.row_idx != nullptr) ? p.row_idx[r] : r;
   const float* src = p.in + r * p.h;
   T* dst = static_cast<T*>(p.out) + o * p.h;
   for (int k = threadIdx.x * 4; k < p.h; k += 256 * 4) {

@@ -772,8 +772,12 @@ extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float*
   TLCE_REQUIRE(dtype == TLCE_DTYPE_BF16, "apply_grad_output: unsupported dtype code %d (bf16 only)",
                dtype);
   TLCE_REQUIRE(m >= 0 && h > 0 && v > 0 && (h % 4) == 0, "apply_grad_output: bad shape");
-  TLCE_REQUIRE(reduction_code == TLCE_REDUCTION_SUM || reduction_code == TLCE_REDUCTION_MEAN,
-               "apply_grad_output: the upstream gradient must be a scalar (sum or mean)");
+  TLCE_REQUIRE(reduction_code == TLCE_REDUCTION_SUM || reduction_code == TLCE_REDUCTION_MEAN ||
+                   reduction_code == TLCE_REDUCTION_NONE,
+               "apply_grad_output: unknown reduction code %d", reduction_code);
+  TLCE_REQUIRE(reduction_code != TLCE_REDUCTION_NONE || grad_weight_f32 == nullptr,
+               "apply_grad_output: with one upstream gradient per row (reduction none) the "
+               "grad_weight contraction has to wait for it (grad_weight_from_panel)");
   TLCE_REQUIRE(n_out >= m, "apply_grad_output: n_out=%lld < m=%lld", (long long)n_out,
                (long long)m);
   TLCE_REQUIRE(row_idx != nullptr || n_out == m || m == 0,
@@ -810,7 +814,8 @@ extern "C" int tlce_apply_grad_output(const float* grad_hidden_f32, const float*
   return 0;
 }
 
-extern "C" int tlce_grad_weight_from_panel(const void* hidden, const int64_t* row_count,
+extern "C" int tlce_grad_weight_from_panel(const void* hidden, const int64_t* row_idx,
+                                           const int64_t* row_count,
                                            const float* grad_output, const float* valid_count,
                                            int64_t m, int64_t h, int64_t v, int dtype,
                                            int reduction_code, void* grad_weight,
@@ -820,8 +825,9 @@ extern "C" int tlce_grad_weight_from_panel(const void* hidden, const int64_t* ro
   TLCE_REQUIRE(m >= 0 && h > 0 && v > 0, "grad_weight_from_panel: bad shape");
   TLCE_REQUIRE(fused_gradients_supported(h, v, dtype),
                "grad_weight_from_panel: needs bf16 inputs with h and v multiples of 64");
-  TLCE_REQUIRE(reduction_code == TLCE_REDUCTION_SUM || reduction_code == TLCE_REDUCTION_MEAN,
-               "grad_weight_from_panel: the upstream gradient must be a scalar (sum or mean)");
+  TLCE_REQUIRE(reduction_code == TLCE_REDUCTION_SUM || reduction_code == TLCE_REDUCTION_MEAN ||
+                   reduction_code == TLCE_REDUCTION_NONE,
+               "grad_weight_from_panel: unknown reduction code %d", reduction_code);
   TLCE_REQUIRE(grad_weight != nullptr && grad_output != nullptr,
                "grad_weight_from_panel: null pointer");
   TLCE_REQUIRE(valid_count != nullptr || reduction_code != TLCE_REDUCTION_MEAN,
@@ -842,8 +848,8 @@ extern "C" int tlce_grad_weight_from_panel(const void* hidden, const int64_t* ro
   TLCE_REQUIRE(((uintptr_t)forward_workspace & 255) == 0,
                "grad_weight_from_panel: workspace must be 256-byte aligned");
   return deferred_grad_weight_impl<MfmaDirect4Engine<__bf16>>(
-      p, hidden, m, h, v, dtype, grad_output, valid_count, reduction_code, row_count, grad_weight,
-      static_cast<char*>(forward_workspace), stream);
+      p, hidden, m, h, v, dtype, grad_output, valid_count, reduction_code, row_count, row_idx,
+      grad_weight, static_cast<char*>(forward_workspace), stream);
 }
 
 extern "C" int tlce_profile_begin(void) {

@@ -38,14 +38,19 @@ _compaction = contextvars.ContextVar("tlce_compaction_mode", default="sync")
 _panel_bytes = contextvars.ContextVar("tlce_panel_bytes", default=0)
 
 
-# When the gradients of a scalar-reduced loss ("mean" / "sum") are formed:
+# When the gradients are formed:
 #   "forward"   (default) during the forward, while the logits of a block of rows
 #               exist: 3 contractions per step instead of 4.  Taken where the
-#               library supports it (16-bit inputs, no bias, H and V multiples of
-#               64, the row count known to the host) and a gradient is required;
-#               other calls fall back to "recompute".  The forward then holds the
-#               float32 gradients ([M, H] and [V, H]) until the backward scales
-#               and rounds them;
+#               library supports it (bf16 inputs, no bias, head stored [V, H], H
+#               and V multiples of 64) and a gradient is required; other calls
+#               fall back to "recompute".  The forward then holds the float32
+#               grad_hidden [M, H] and either the float32 grad_weight [V, H] or,
+#               when all rows fit one block, its workspace, until the backward
+#               scales and rounds them.  Per-token losses (reduction "none")
+#               take this path with a frozen head, and with a trainable head
+#               when all rows fit one block: grad_weight needs the per-row
+#               upstream gradients inside its contraction, which then runs in
+#               the backward;
 #   "recompute" by a backward that recomputes the logits in vocabulary panels, as
 #               the reference's backward does block by block
 #               (fused_linear_ce_cuda.cu:618-791).

@@ -270,22 +270,27 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
         rows, targets, _, row_idx, row_count, m = native.compact_loss_rows(
             hidden_flat, labels_flat, None, ignore_index, mode)
 
-    # Gradients while the logits exist (3 contractions instead of 4): when the loss
-    # is reduced to a scalar, some input needs a gradient, and the library takes the
-    # operands (options.GRADIENT_MODES).
+    # Gradients while the logits exist (3 contractions instead of 4): when some input
+    # needs a gradient and the library takes the operands (options.GRADIENT_MODES).
+    # grad_hidden is linear in each row's upstream gradient, so it can be formed for
+    # any reduction; grad_weight needs the upstream gradient inside its contraction,
+    # so with per-token losses (reduction "none") it must be the postponed contraction,
+    # which exists when all rows form one block.
     wants_grad = bool(ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
     ctx.fused = (
-        wants_grad and reduction in ("mean", "sum")
-        and options.get_gradient_mode() == "forward"
+        wants_grad and options.get_gradient_mode() == "forward"
         and native.fused_gradients_supported(rows, weight_vf, bias, in_place or weight_dim_first)
     )
+    can_wait = ctx.fused and bool(ctx.needs_input_grad[1]) and native.weight_grad_can_wait(
+        m, rows.shape[1], weight_vf.shape[0], rows.dtype)
+    if reduction == "none" and bool(ctx.needs_input_grad[1]) and not can_wait:
+        ctx.fused = False
     if ctx.fused:
         # (rows compacted with the count read back carry up to 63 zero rows of padding)
         rows, targets = rows[:m], targets[:m]
         # all rows in one block: the grad_weight contraction waits for the upstream
         # gradient and is stored in the input dtype at once (no float32 [V, H] buffer)
-        ctx.postponed = bool(ctx.needs_input_grad[1]) and native.weight_grad_can_wait(
-            m, rows.shape[1], weight_vf.shape[0], rows.dtype)
+        ctx.postponed = can_wait
         losses, lse, valid_count, grad_rows32, grad_weight32 = native.forward_with_gradients(
             rows, weight_vf, targets, ignore_index=ignore_index, exclude_index=exclude_index,
             logit_softcap=float(logit_softcap),
@@ -302,6 +307,8 @@ def _device_forward(ctx, hidden, weight, bias, labels, reduction, ignore_index, 
         ctx.reduction = reduction
         ctx.grad_dtype = hidden.dtype
         ctx.vocab = weight_vf.shape[0]
+        if reduction == "none":
+            return losses.reshape(labels.shape)
         if reduction == "sum":
             return losses.sum()
         return losses.sum() / valid_count.squeeze(0)
@@ -353,6 +360,7 @@ def _device_backward(ctx, grad_output, frozen: bool):
             grad_weight = native.grad_weight_from_panel(
                 rows, grad_weight32, grad_output, valid_count, reduction=ctx.reduction,
                 vocab=ctx.vocab, panel_bytes=ctx.panel_bytes, row_count=row_count,
+                row_idx=row_idx, n_out=ctx.n_rows,
             )
         return (grad_hidden.reshape(ctx.hidden_shape), None if frozen else grad_weight,
                 None) + (None,) * 9
