@@ -404,7 +404,7 @@ def bench_next_objective(args) -> int:
             streaming_soft_embedding(hidden, weight, row_chunk_size=1024, vocab_chunk_size=8192,
                                      logit_softcap=30.0)
 
-        contractions, name = 3, "streaming soft embedding fwd"
+        contractions, name = 2, "streaming soft embedding fwd"
         shape = f"M={m}, H={h}, V={v}, softcap=30"
     for _ in range(args.warmup):
         step()

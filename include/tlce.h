@@ -324,7 +324,12 @@ int tlce_backward_local(const void* hidden, const void* weight, const float* bia
  *   out[r] = embedding_scale * softmax(cap(hidden[r] . weight^T)) . weight
  * forward-only, without a logits buffer: the forward tile loop yields lse, the
  * probability panels (rounded to `dtype`, as the reference rounds them before
- * its second matmul) are contracted with the weight rows in float32.
+ * its second matmul) are contracted with the weight rows in float32: three
+ * contractions.  Under a soft cap of at most 40 (bf16, h and v multiples of 64)
+ * two suffice: capped logits lie in [-cap, cap], so exp(logit - cap) needs no
+ * row maximum; it is written for a block of rows over the whole vocabulary
+ * into a panel of panel_bytes (0: 2.5 GiB), contracted with the weight rows, and
+ * the result divided by the row's sum.  The workspace query covers both.
  *   hidden [m,h], weight [v,h], out [m,h], all `dtype`. */
 int64_t tlce_soft_embedding_workspace_bytes(int64_t m, int64_t h, int64_t v,
                                             int dtype, int64_t panel_bytes);

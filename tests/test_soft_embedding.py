@@ -86,3 +86,38 @@ def test_device_path_matches_dense(gpu_device, case):
         h.to(gpu_device), (w[: v // 2].to(gpu_device), w[v // 2:].to(gpu_device)),
         row_chunk_size=64, vocab_chunk_size=256, logit_softcap=softcap, embedding_scale=scale)
     assert torch.equal(two, got)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("softcap,tiles_per_block,std", [
+    (30.0, 0, 3.0),      # the production cap, one block of rows
+    (30.0, 1, 3.0),      # three blocks of rows
+    (30.0, 0, 60.0),     # logits far into the cap on both sides: exp(z - cap) spans exp(-60)..1
+    (40.0, 2, 8.0),      # the largest cap the two-contraction sequence takes
+    (50.0, 0, 8.0),      # beyond it: statistics pass first, three contractions
+])
+def test_capped_soft_embedding_takes_two_contractions(gpu_device, softcap, tiles_per_block, std):
+    """Capped logits lie in [-cap, cap]: exp(z - cap) needs no row maximum, so the
+    device path writes it to the panel in one contraction and normalises after the
+    second (which sequence ran is read from the library's per-class launch counts)."""
+    from turbo_dllm_amd import _lib, options
+    print("[case] capped soft embedding", softcap, tiles_per_block, std, flush=True)
+    m, hdim, v = 700, 128, 2048
+    gen = torch.Generator().manual_seed(int(softcap) + tiles_per_block)
+    h = torch.randn(m, hdim, generator=gen).to(torch.bfloat16)
+    w = (torch.randn(v, hdim, generator=gen) * (std / hdim ** 0.5)).to(torch.bfloat16)
+    with options.panel_budget(tiles_per_block * 256 * v * 2), _lib.kernel_profile() as prof:
+        got = streaming_soft_embedding(h.to(gpu_device), w.to(gpu_device), row_chunk_size=64,
+                                       vocab_chunk_size=256, logit_softcap=softcap,
+                                       embedding_scale=2.0)
+        torch.cuda.synchronize()
+    two_contractions = softcap <= 40.0
+    assert (prof.launches["exp_logits_panel"] > 0) == two_contractions
+    assert (prof.launches["forward_stats"] == 0) == two_contractions
+    if two_contractions:
+        assert prof.launches["exp_logits_panel"] == (1 if tiles_per_block == 0 else
+                                                     -(-m // (256 * tiles_per_block)))
+    assert bool(torch.isfinite(got.float()).all())
+    err = rel_max(got.cpu(), dense(h, w, softcap, 2.0))
+    print("[case] rel max err", f"{err:.2e}", flush=True)
+    assert err <= 2e-2

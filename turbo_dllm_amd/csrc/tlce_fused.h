@@ -53,6 +53,7 @@ struct ExpPanelArgs {
   const void* hidden;   // [m, h] the rows of this block
   const void* weight;   // [v, h]
   const float* ref;     // [m] reference logit per row (natural units); +inf: row without loss
+  float ref_const = 0.0f;   // ref == null: the reference of every row
   int m, h, v;
   int64_t exclude;
   float softcap;
@@ -70,7 +71,9 @@ struct ExpPanelArgs {
   int64_t row0 = 0;
 };
 
-template <class E, bool kSoftcap>
+// kPlain: the panel receives exp(z - c) itself, without the soft cap's derivative
+// (a forward value, the unnormalised softmax, not a logit gradient).
+template <class E, bool kSoftcap, bool kPlain = false>
 __global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPanelArgs p) {
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
@@ -97,7 +100,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPa
   float* ref_stash = reinterpret_cast<float*>(smem + E::kSmemBytes);
   for (int c = threadIdx.x; c < E::kTile; c += E::kThreads) {
     const int r = tt * E::kTile + c;
-    ref_stash[c] = (r < p.m) ? p.ref[r] * TLCE_LOG2E : INFINITY;
+    ref_stash[c] = (r < p.m) ? (p.ref != nullptr ? p.ref[r] : p.ref_const) * TLCE_LOG2E
+                             : INFINITY;
   }
   eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
                    static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
@@ -147,7 +151,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPa
           }
           mx = fmaxf(mx, z2);
           s += e;
-          e4[q] = kSoftcap ? e * dcap : e;
+          e4[q] = (kSoftcap && !kPlain) ? e * dcap : e;
         }
         const int vq = eng.row(i) >> 2;
         T* dst = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
@@ -198,15 +202,15 @@ __global__ __launch_bounds__(E::kThreads) void lce_exp_logits_panel_kernel(ExpPa
   }
 }
 
-template <class E, bool kSoftcap>
+template <class E, bool kSoftcap, bool kPlain = false>
 int launch_exp_panel_variant(const ExpPanelArgs& a, hipStream_t stream) {
   static LdsOptIn lds;
   constexpr int kLdsBytes = E::kSmemBytes + E::kTile * (int)sizeof(float);   // stages + stash
-  if (int rc = enable_large_lds(lce_exp_logits_panel_kernel<E, kSoftcap>, kLdsBytes, lds))
+  if (int rc = enable_large_lds(lce_exp_logits_panel_kernel<E, kSoftcap, kPlain>, kLdsBytes, lds))
     return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_vtiles);
   ScopedTimer timer(kClassExpPanel, stream);
-  lce_exp_logits_panel_kernel<E, kSoftcap><<<grid, E::kThreads, kLdsBytes, stream>>>(a);
+  lce_exp_logits_panel_kernel<E, kSoftcap, kPlain><<<grid, E::kThreads, kLdsBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
@@ -265,6 +269,7 @@ struct ReduceSlabsArgs {
   const float* row_scale;
   int m, h;
   float* out;   // [m, h]
+  void* out_t = nullptr;            // non-null: the result goes here in bf16 instead
   const int64_t* m_dev = nullptr;   // device row count (null: m is exact); the block's
   int64_t row0 = 0;                 // first row among the counted rows
   // with a device row count the contraction derives its K splits and slab stride from
@@ -303,6 +308,17 @@ struct ScaleRowsArgs {
   const int64_t* row_idx = nullptr; // output row of row r (null: r)
 };
 
+// row_scale[r] = scale / sum over the vocabulary tiles of part_sum[tile][r] (0 for rows
+// from m up to m_pad): the normaliser of rows whose panel holds exp(z - c).
+struct SoftRowsArgs {
+  const float* part_sum;
+  int part_ld, n_vtiles;
+  int m, m_pad;
+  float scale;
+  float* row_scale;
+};
+
+int launch_soft_rows(const SoftRowsArgs& a, hipStream_t stream);
 int launch_label_logit(const LabelLogitArgs& a, hipStream_t stream);
 int launch_scale_rows(const ScaleRowsArgs& a, hipStream_t stream);
 int launch_fused_rows(const FusedRowsArgs& a, hipStream_t stream);
@@ -547,14 +563,87 @@ int deferred_grad_weight_impl(const FusedPlan& p, const void* hidden, int64_t m,
   return launch_gemm<E, true, true>(dw, 1, kClassGradWeight, stream);
 }
 
-#define TLCE_LAUNCHERS_EXP_PANEL(X, E)                                            \
-  X int launch_exp_panel_variant<E, false>(const ExpPanelArgs&, hipStream_t);     \
-  X int launch_exp_panel_variant<E, true>(const ExpPanelArgs&, hipStream_t);
+// Soft embedding under a soft cap in two contractions instead of three
+// (streaming_soft_embedding.py:60-148 computes softmax(cap(h W^T)) W with running
+// maxima over vocabulary chunks): capped logits lie in [-cap, cap], so exp(z - cap)
+// lies in [exp(-2 cap), 1] and needs no row maximum.  Per block of rows over the whole
+// vocabulary: the panel receives exp(z - cap) in bf16 and the per-tile sums go out as
+// partials, then out[r, :] = (scale / sum_r) * (panel . weight)[r, :] in float32,
+// rounded once.  cap <= kSoftEmbeddingMaxCap keeps exp(-2 cap) a normal bf16 number.
+constexpr float kSoftEmbeddingMaxCap = 40.0f;
+
+template <class E>
+int soft_embedding_fused_impl(const FusedPlan& p, const void* hidden, const void* weight,
+                              int64_t m, int64_t h, int64_t v, int dtype, float softcap,
+                              float scale, void* out, char* ws, hipStream_t stream) {
+  using T = typename E::T;
+  const FusedLayout l = fused_layout(p, m, h, dtype, false);
+  T* panel = reinterpret_cast<T*>(ws + l.panel);
+  float* part_sum = reinterpret_cast<float*>(ws + l.part_sum);
+  float* part_max = reinterpret_cast<float*>(ws + l.part_max);
+  float* row_scale = reinterpret_cast<float*>(ws + l.row_scale);
+  float* slabs = reinterpret_cast<float*>(ws + l.slabs);
+  const T* hidden_t = static_cast<const T*>(hidden);
+  for (int block = 0; block < p.n_blocks; ++block) {
+    const int64_t r0 = (int64_t)block * p.block_rows;
+    const int64_t rows = std::min<int64_t>(p.block_rows, m - r0);
+    if (rows <= 0) break;
+    const int n_ttiles = (int)ceil_div(rows, E::kTile);
+    const int64_t rows_p = (int64_t)n_ttiles * E::kTile;
+
+    ExpPanelArgs ea;
+    ea.hidden = hidden_t + r0 * h; ea.weight = weight;
+    ea.ref = nullptr; ea.ref_const = softcap;
+    ea.m = (int)rows; ea.h = (int)h; ea.v = (int)v;
+    ea.exclude = -1; ea.softcap = softcap; ea.logit_scale = 1.0f;
+    ea.n_ttiles = n_ttiles; ea.n_vtiles = p.n_vtiles;
+    ea.panel = panel; ea.ld = p.vp;
+    ea.part_sum = part_sum; ea.part_max = part_max; ea.part_ld = (int)p.block_rows;
+    ea.run_flag = nullptr;
+    if (int rc = launch_exp_panel_variant<E, true, true>(ea, stream)) return rc;
+
+    SoftRowsArgs sr;
+    sr.part_sum = part_sum; sr.part_ld = (int)p.block_rows; sr.n_vtiles = p.n_vtiles;
+    sr.m = (int)rows; sr.m_pad = (int)rows_p; sr.scale = scale; sr.row_scale = row_scale;
+    if (int rc = launch_soft_rows(sr, stream)) return rc;
+
+    // the contraction of grad_hidden in the forward that leaves the gradients: K = the
+    // vocabulary, K splits into slabs for few rows
+    GemmArgs g;
+    g.a = weight; g.lda = h; g.a_rows = (int)h;
+    g.b = panel; g.ldb = p.vp; g.b_rows = (int)rows_p;
+    g.k = (int)round_up(v, 64); g.k_per_split = 0;
+    g.ni = p.n_htiles; g.nj = n_ttiles;
+    g.c = slabs; g.ldc = h; g.c_rows = (int)rows_p; g.c_cols = (int)h;
+    g.c_split_stride = p.block_rows * h;
+    g.mode = kStoreF32;
+    const int ksplit = (rows_p == p.block_rows)
+                           ? p.dh_ksplit
+                           : std::min(p.dh_ksplit,
+                                      grad_hidden_k_splits((int64_t)n_ttiles * p.n_htiles,
+                                                           p.dh_ksplit, p.vp / 64, rows_p * h));
+    if (int rc = launch_gemm<E, true, false>(g, ksplit, kClassGradHidden, stream)) return rc;
+    ReduceSlabsArgs rs;
+    rs.slabs = slabs; rs.n_splits = ksplit; rs.split_stride = p.block_rows * h;
+    rs.row_scale = row_scale; rs.m = (int)rows; rs.h = (int)h;
+    rs.out = nullptr; rs.out_t = static_cast<T*>(out) + r0 * h;
+    if (int rc = launch_reduce_slabs(rs, stream)) return rc;
+  }
+  return 0;
+}
+
+#define TLCE_LAUNCHERS_EXP_PANEL(X, E)                                                  \
+  X int launch_exp_panel_variant<E, false, false>(const ExpPanelArgs&, hipStream_t);    \
+  X int launch_exp_panel_variant<E, true, false>(const ExpPanelArgs&, hipStream_t);     \
+  X int launch_exp_panel_variant<E, true, true>(const ExpPanelArgs&, hipStream_t);
 #define TLCE_FUSED_ENTRY_POINTS(X, E)                                                            \
   X int fused_gradients_impl<E>(const FusedPlan&, const void*, const void*, const int64_t*,      \
                                 const int64_t*, int64_t, int64_t, int64_t, int, int64_t,         \
                                 int64_t, float, float*, float*, float*, float*, float*, char*,   \
                                 hipStream_t, const FusedOptions&);                               \
+  X int soft_embedding_fused_impl<E>(const FusedPlan&, const void*, const void*, int64_t,        \
+                                     int64_t, int64_t, int, float, float, void*, char*,          \
+                                     hipStream_t);                                               \
   X int deferred_grad_weight_impl<E>(const FusedPlan&, const void*, int64_t, int64_t, int64_t,   \
                                      int, const float*, const float*, int, const int64_t*,       \
                                      const int64_t*, void*, char*, hipStream_t);

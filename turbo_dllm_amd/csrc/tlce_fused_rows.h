@@ -185,13 +185,42 @@ __global__ __launch_bounds__(256) void lce_reduce_scaled_slabs_kernel(ReduceSlab
   }
   const float s = p.row_scale[r];
   const float* src = p.slabs + (int64_t)r * p.h;
-  float* dst = p.out + (int64_t)r * p.h;
   for (int k = threadIdx.x * 4; k < p.h; k += 256 * 4) {
     f32x4_t sum = *reinterpret_cast<const f32x4_t*>(src + k);
     for (int q = 1; q < p.n_splits; ++q)
       sum += *reinterpret_cast<const f32x4_t*>(src + (int64_t)q * p.split_stride + k);
-    *reinterpret_cast<f32x4_t*>(dst + k) = sum * s;
+    sum = sum * s;
+    if (p.out_t != nullptr) {
+      store4<__bf16>(static_cast<__bf16*>(p.out_t) + (int64_t)r * p.h + k, sum[0], sum[1], sum[2],
+                     sum[3]);
+    } else {
+      *reinterpret_cast<f32x4_t*>(p.out + (int64_t)r * p.h + k) = sum;
+    }
   }
+}
+
+// 64 rows per workgroup of 16 waves, the rows across the lanes (the partials are
+// stored [tile][row]: a wave reads 256 consecutive bytes per tile); wave w adds the
+// tiles w, w + 16, ... in order and the 16 sums are merged in a fixed order.
+constexpr int kSoftRowsWaves = 16;
+
+__global__ __launch_bounds__(64 * kSoftRowsWaves) void lce_soft_rows_kernel(SoftRowsArgs p) {
+  __shared__ float sh[kSoftRowsWaves][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = blockIdx.x * 64 + lane;
+  float sum = 0.0f;
+  if (r < p.m) {
+    for (int t = wave; t < p.n_vtiles; t += kSoftRowsWaves)
+      sum += p.part_sum[(int64_t)t * p.part_ld + r];
+  }
+  sh[wave][lane] = sum;
+  __syncthreads();
+  if (wave != 0 || r >= p.m_pad) return;
+  sum = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kSoftRowsWaves; ++w) sum += sh[w][lane];
+  p.row_scale[r] = (r < p.m && sum > 0.0f) ? p.scale / sum : 0.0f;
 }
 
 template <typename T>

@@ -89,6 +89,13 @@ int launch_scale_rows(const ScaleRowsArgs& a, hipStream_t stream) {
   return 0;
 }
 
+int launch_soft_rows(const SoftRowsArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassCombine, stream);
+  lce_soft_rows_kernel<<<(int)ceil_div(a.m_pad, 64), 64 * kSoftRowsWaves, 0, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
 int launch_reduce_slabs(const ReduceSlabsArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassOther, stream);
   lce_reduce_scaled_slabs_kernel<<<a.m, 256, 0, stream>>>(a);
@@ -481,7 +488,13 @@ extern "C" int64_t tlce_soft_embedding_workspace_bytes(int64_t m, int64_t h, int
   if (m < 0 || h <= 0 || v <= 0) return -1;
   const Plan fp = make_plan(m, h, v, dtype, false, 0);
   const Plan bp = make_plan(m, h, v, dtype, false, panel_bytes);
-  return soft_embedding_layout(fp, bp, m, h, dtype).total;
+  int64_t need = soft_embedding_layout(fp, bp, m, h, dtype).total;
+  // the soft cap is not known here: enough for either sequence
+  if (fused_gradients_supported(h, v, dtype)) {
+    const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
+    need = std::max(need, fused_layout(p, m, h, dtype, false).total);
+  }
+  return need;
 }
 
 extern "C" int tlce_soft_embedding(const void* hidden, const void* weight, int64_t m, int64_t h,
@@ -493,6 +506,19 @@ extern "C" int tlce_soft_embedding(const void* hidden, const void* weight, int64
   if (m == 0) return 0;
   TLCE_REQUIRE(out != nullptr && workspace != nullptr, "soft_embedding: null pointer");
   TLCE_REQUIRE(((uintptr_t)out & 15) == 0, "soft_embedding: out must be 16-byte aligned");
+  if (logit_softcap > 0.0f && logit_softcap <= kSoftEmbeddingMaxCap &&
+      fused_gradients_supported(h, v, dtype)) {
+    // under a soft cap no row maximum is needed: two contractions instead of three
+    const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
+    const int64_t need = fused_layout(p, m, h, dtype, false).total;
+    TLCE_REQUIRE(workspace_bytes >= need, "soft_embedding: workspace too small (%lld < %lld)",
+                 (long long)workspace_bytes, (long long)need);
+    TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+                 "soft_embedding: workspace must be 256-byte aligned");
+    return soft_embedding_fused_impl<MfmaDirect4Engine<__bf16>>(
+        p, hidden, weight, m, h, v, dtype, logit_softcap, embedding_scale, out,
+        static_cast<char*>(workspace), stream);
+  }
   const Plan fp = make_plan(m, h, v, dtype, false, 0);
   const Plan bp = make_plan(m, h, v, dtype, false, panel_bytes);
   const SoftEmbeddingLayout l = soft_embedding_layout(fp, bp, m, h, dtype);
