@@ -609,6 +609,11 @@ def grad_weight_from_panel(
     m, h = hidden.shape
     grad_output = _upstream_gradient(grad_output, reduction_code,
                                      m if n_out is None else int(n_out))
+    # the C ABI cannot see tensor lengths: what the kernels read must exist
+    if row_idx is not None and (row_idx.dtype != torch.long or row_idx.numel() < m):
+        raise RuntimeError("row_idx must be int64 with one entry per row of hidden")
+    if workspace.dtype != torch.uint8 or not workspace.is_contiguous():
+        raise RuntimeError("workspace must be the uint8 buffer forward_with_gradients returned")
     with torch.cuda.device(device):
         grad_weight = torch.empty((int(vocab), h), dtype=hidden.dtype, device=device)
         _lib.check(
@@ -647,6 +652,15 @@ def apply_grad_output(
     v = grad_weight32.shape[0] if grad_weight32 is not None else int(vocab or 1)
     n_out = m if n_out is None else int(n_out)
     grad_output = _upstream_gradient(grad_output, reduction_code, n_out)
+    # the C ABI cannot see tensor lengths: what the kernels read must exist
+    if grad_hidden32.dtype != torch.float32 or not grad_hidden32.is_contiguous():
+        raise RuntimeError("grad_hidden32 must be a contiguous float32 [m, h] tensor")
+    if grad_weight32 is not None and (grad_weight32.dtype != torch.float32
+                                      or not grad_weight32.is_contiguous()
+                                      or grad_weight32.shape[1] != h):
+        raise RuntimeError("grad_weight32 must be a contiguous float32 [v, h] tensor")
+    if row_idx is not None and (row_idx.dtype != torch.long or row_idx.numel() < m):
+        raise RuntimeError("row_idx must be int64 with one entry per row of grad_hidden32")
     if dtype != torch.bfloat16:
         raise RuntimeError("apply_grad_output writes bf16 gradients only")
     code = _lib.DTYPE_BF16
