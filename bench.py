@@ -394,7 +394,10 @@ def bench_next_objective(args) -> int:
             loss, prob, values, _ = frozen_linear_ce_topk(hidden, weight, labels, top_k=k)
             (loss.sum() + prob.sum() + values.sum()).backward()
 
-        contractions, name = 3, "frozen-head CE + top-16 fwd+bwd"   # 1 forward + 2 backward
+        # the logits and, in the same forward, d lse / d hidden; the backward is a row pass
+        # (--gradients recompute: 1 forward + 2 backward)
+        contractions = 2 if args.gradients == "forward" else 3
+        name = "frozen-head CE + top-16 fwd+bwd"
         shape = f"M={m}, H={h}, V={v}, top_k={k}"
     else:
         h, v = 3840, 262144

@@ -416,6 +416,45 @@ int tlce_ce_topk_backward(const void* hidden, const void* weight,
                           int64_t panel_bytes, void* workspace,
                           int64_t workspace_bytes, void* stream);
 
+/* The same pair with the softmax part of the gradient formed in the forward
+ * (dflash_ce_topk_forward + dflash_ce_topk_backward, fused_linear_ce.cpp:306-354,
+ * whose backward recomputes the logits): while a float32 logits panel exists,
+ * exp(z - the row's largest logit so far) * dz/draw is written in bf16 into a
+ * panel over the whole vocabulary (2 bytes per row and vocabulary entry inside
+ * the workspace; panels written before a row's maximum grew are rescaled
+ * afterwards), and one contraction with the weight rows leaves
+ *   unit_grad_hidden_f32[r, :] = d lse[r] / d hidden[r, :]      float32 [m, h].
+ * tlce_ce_topk_apply_gradient then forms, in one pass over rows,
+ *   grad_hidden[r, :] = ce_scale[r] * unit[r, :]
+ *                       - ce_scale[r] * dz/draw[label] * weight[label]
+ *                       + sum_j grad_top_values[r,j] * dz/draw[id_j] * weight[id_j]
+ * rounded once: 2 contractions per step instead of 3.  bf16, h and v multiples
+ * of 64, and all rows in one block of the 2.5 GiB panel budget (8192 rows at
+ * v = 151936): tlce_ce_topk_gradient_in_forward_supported; panel_bytes bounds
+ * the float32 logits panels as in tlce_ce_topk_forward. */
+int tlce_ce_topk_gradient_in_forward_supported(int64_t m, int64_t h, int64_t v,
+                                               int dtype);
+
+int64_t tlce_ce_topk_forward_with_gradient_workspace_bytes(int64_t m, int64_t h,
+                                                           int64_t v, int dtype,
+                                                           int64_t panel_bytes);
+
+int tlce_ce_topk_forward_with_gradient(
+    const void* hidden, const void* weight, const int64_t* labels, int64_t m,
+    int64_t h, int64_t v, int dtype, int top_k, float output_multiplier,
+    float logit_softcap, float* losses, float* probabilities, float* top_values,
+    int64_t* top_ids, float* lse, float* unit_grad_hidden_f32,
+    int64_t panel_bytes, void* workspace, int64_t workspace_bytes, void* stream);
+
+int tlce_ce_topk_apply_gradient(const float* unit_grad_hidden_f32,
+                                const void* hidden, const void* weight,
+                                const int64_t* labels, const int64_t* top_ids,
+                                const float* ce_scale, const float* grad_top_values,
+                                int64_t m, int64_t h, int64_t v, int dtype,
+                                int top_k, float output_multiplier,
+                                float logit_softcap, void* grad_hidden,
+                                void* stream);
+
 /* ---- per-sample loss numerators of the DFlash loss method -----------------
  * Replaces `numerators.scatter_add_(0, sample_indices, token_loss * position_weights)`
  * with sample_indices = valid_indices // tokens_per_sample

@@ -187,3 +187,75 @@ def test_selection_is_exact_on_exactly_representable_logits(gpu_device, case, se
     assert torch.equal(ids.cpu(), r_ids)
     assert torch.equal(vals.cpu().double(), r_vals)
     torch.testing.assert_close(loss.cpu().double(), r_loss, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("softcap,std", [(None, 0.2), (None, 2.5), (4.0, 0.5)])
+def test_gradient_formed_in_the_forward_over_several_logits_panels(gpu_device, softcap, std,
+                                                                   set_panel_budget):
+    """bf16 operands the library takes: the forward also leaves d lse / d hidden (its
+    grad_hidden contraction shows up in the forward's launch counts) and the backward is
+    one pass over rows.  Four float32 logits panels, so most rows' maxima grow after their
+    first panels were written and those are rescaled (std 2.5: by tens of nats).  Against
+    the oracle and against the recomputing backward."""
+    from turbo_dllm_amd import _lib, options
+    print("[case] top-k gradient in the forward", softcap, std, flush=True)
+    n, h, v, k = 520, 128, 4096, 8
+    set_panel_budget(768 * 1024 * 4)
+    gen = torch.Generator().manual_seed(17)
+    hidden = torch.randn(n, h, generator=gen).to(torch.bfloat16)
+    weight = (torch.randn(v, h, generator=gen) * std).to(torch.bfloat16)
+    labels = torch.randint(0, v, (n,), generator=gen)
+    gl, gp, gv = (torch.randn(n, generator=gen), torch.randn(n, generator=gen),
+                  torch.randn(n, k, generator=gen))
+    grads = {}
+    for mode in options.GRADIENT_MODES:
+        x = hidden.to(gpu_device).requires_grad_(True)
+        with options.gradient_mode(mode), _lib.kernel_profile() as prof:
+            loss, prob, vals, ids = frozen_linear_ce_topk(
+                x, weight.to(gpu_device), labels.to(gpu_device), top_k=k,
+                output_multiplier=0.75, logit_softcap=softcap)
+            torch.cuda.synchronize()
+        assert prof.launches["grad_logits_panel"] == 4          # the float32 logits panels
+        assert (prof.launches["grad_hidden_gemm"] > 0) == (mode == "forward")
+        ((gl.to(gpu_device) * loss).sum() + (gp.to(gpu_device) * prob).sum()
+         + (gv.to(gpu_device) * vals).sum()).backward()
+        torch.cuda.synchronize()
+        grads[mode] = (x.grad.cpu(), ids.cpu(), loss.detach().cpu())
+    assert torch.equal(grads["forward"][1], grads["recompute"][1])
+    assert torch.equal(grads["forward"][2], grads["recompute"][2])
+    r_grad = oracle.dense_ce_topk_grad(hidden, weight, labels, grads["forward"][1], gl, gp, gv,
+                                       output_multiplier=0.75, logit_softcap=softcap)
+    for mode in options.GRADIENT_MODES:
+        err = oracle.relative_max_error(grads[mode][0], r_grad)
+        print("[case]", mode, "grad rel max err", f"{err:.2e}", flush=True)
+        assert bool(torch.isfinite(grads[mode][0].float()).all())
+        assert err <= 2e-2
+
+
+@pytest.mark.gpu
+def test_gradient_in_the_forward_backward_twice_and_no_gradient(gpu_device):
+    """retain_graph: a second backward with other upstream gradients; and a forward whose
+    hidden states need no gradient runs no gradient contraction."""
+    from turbo_dllm_amd import _lib
+    n, h, v, k = 300, 64, 2048, 4
+    gen = torch.Generator().manual_seed(23)
+    hidden = torch.randn(n, h, generator=gen).to(torch.bfloat16)
+    weight = (torch.randn(v, h, generator=gen) * 0.3).to(torch.bfloat16)
+    labels = torch.randint(0, v, (n,), generator=gen)
+    x = hidden.to(gpu_device).requires_grad_(True)
+    loss, prob, vals, ids = frozen_linear_ce_topk(x, weight.to(gpu_device), labels.to(gpu_device),
+                                                  top_k=k)
+    for seed in (1, 2):
+        g = torch.Generator().manual_seed(seed)
+        gl, gp, gv = torch.randn(n, generator=g), torch.randn(n, generator=g), torch.randn(n, k, generator=g)
+        x.grad = None
+        ((gl.to(gpu_device) * loss).sum() + (gp.to(gpu_device) * prob).sum()
+         + (gv.to(gpu_device) * vals).sum()).backward(retain_graph=True)
+        r_grad = oracle.dense_ce_topk_grad(hidden, weight, labels, ids.cpu(), gl, gp, gv)
+        assert oracle.relative_max_error(x.grad.cpu(), r_grad) <= 2e-2
+    with _lib.kernel_profile() as prof:
+        frozen_linear_ce_topk(hidden.to(gpu_device), weight.to(gpu_device),
+                              labels.to(gpu_device), top_k=k)
+        torch.cuda.synchronize()
+    assert prof.launches["grad_hidden_gemm"] == 0

@@ -122,6 +122,27 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_ce_topk_gradient_in_forward_supported": (c_int, [c_int64, c_int64, c_int64, c_int]),
+    "tlce_ce_topk_forward_with_gradient_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int, c_int64]),
+    "tlce_ce_topk_forward_with_gradient": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int,  # h w labels m h v dtype k
+            c_float, c_float,                                   # multiplier softcap
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # losses probs top_values top_ids lse
+            c_void_p, c_int64, c_void_p, c_int64, c_void_p,     # unit panel_bytes ws bytes stream
+        ],
+    ),
+    "tlce_ce_topk_apply_gradient": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,   # unit hidden weight labels top_ids
+            c_void_p, c_void_p,                                 # ce_scale grad_top_values
+            c_int64, c_int64, c_int64, c_int, c_int,            # m h v dtype k
+            c_float, c_float, c_void_p, c_void_p,               # multiplier softcap grad_hidden stream
+        ],
+    ),
     "tlce_grad_weight_from_panel": (
         c_int,
         [

@@ -1263,6 +1263,113 @@ def dflash_ce_topk_forward(
     return loss, probability, top_values, top_ids, lse
 
 
+def ce_topk_gradient_in_forward_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether ``dflash_ce_topk_forward_with_gradient`` takes these operands: bf16,
+    H and V multiples of 64, and all rows in one block of the panel of exponentiated
+    logits (2.5 GiB over the whole vocabulary: 8192 rows at V = 151936)."""
+    if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or hidden.shape[0] == 0:
+        return False
+    return bool(_lib.library().tlce_ce_topk_gradient_in_forward_supported(
+        hidden.shape[0], hidden.shape[1], weight.shape[0], _lib.DTYPE_BF16))
+
+
+def dflash_ce_topk_forward_with_gradient(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    *,
+    top_k: int,
+    output_multiplier: float,
+    logit_softcap: float,
+) -> tuple[torch.Tensor, ...]:
+    """``dflash_ce_topk_forward`` plus ``d lse / d hidden`` as a float32 ``[N, D]``
+    tensor, formed while the forward's logits panels exist (one more contraction
+    instead of the backward's two).  ``dflash_ce_topk_apply_gradient`` turns it into
+    grad_hidden once the upstream gradients are known."""
+    device = _require_device(hidden, weight, labels)
+    if hidden.dim() != 2 or weight.dim() != 2 or weight.shape[1] != hidden.shape[1]:
+        raise RuntimeError("CE top-k expects hidden [N, D] and weight [V, D]")
+    hidden = _dense(hidden)
+    weight = _dense(weight)
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v = weight.shape[0]
+    if labels.numel() != m:
+        raise RuntimeError("CE top-k expects one label per row")
+    k = int(top_k)
+    code = _dtype_code(hidden)
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        loss = torch.empty(m, dtype=torch.float32, device=device)
+        probability = torch.empty(m, dtype=torch.float32, device=device)
+        lse = torch.empty(m, dtype=torch.float32, device=device)
+        top_values = torch.empty((m, k), dtype=torch.float32, device=device)
+        top_ids = torch.empty((m, k), dtype=torch.long, device=device)
+        unit = torch.empty((m, h), dtype=torch.float32, device=device)
+        nbytes = lib.tlce_ce_topk_forward_with_gradient_workspace_bytes(m, h, v, code,
+                                                                         get_panel_bytes())
+        if nbytes < 0:
+            raise RuntimeError("CE top-k with the gradient formed in the forward does not take "
+                               "these operands (ce_topk_gradient_in_forward_supported)")
+        ws = _workspace(nbytes, device)
+        _lib.check(
+            lib.tlce_ce_topk_forward_with_gradient(
+                _ptr(hidden), _ptr(weight), _ptr(labels), m, h, v, code, k,
+                float(output_multiplier), float(logit_softcap),
+                _ptr(loss), _ptr(probability), _ptr(top_values), _ptr(top_ids), _ptr(lse),
+                _ptr(unit), get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_ce_topk_forward_with_gradient",
+        )
+    return loss, probability, top_values, top_ids, lse, unit
+
+
+def dflash_ce_topk_apply_gradient(
+    unit: torch.Tensor,
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    labels: torch.Tensor,
+    probabilities: torch.Tensor,
+    top_ids: torch.Tensor,
+    grad_loss: torch.Tensor,
+    grad_probability: torch.Tensor,
+    grad_top_values: torch.Tensor | None,
+    *,
+    output_multiplier: float,
+    logit_softcap: float,
+) -> torch.Tensor:
+    """grad_hidden from the ``d lse / d hidden`` the forward left: one pass over rows
+    that scales it and adds the label's and the top-k ids' single-row terms."""
+    device = _require_device(unit, hidden, weight, labels, probabilities, top_ids, grad_loss,
+                             grad_probability, grad_top_values)
+    hidden = _dense(hidden)
+    weight = _dense(weight)
+    labels = labels.reshape(-1).to(torch.long).contiguous()
+    m, h = hidden.shape
+    v = weight.shape[0]
+    k = int(top_ids.shape[1])
+    if unit.dtype != torch.float32 or tuple(unit.shape) != (m, h) or not unit.is_contiguous():
+        raise RuntimeError("the forward's gradient must be a contiguous float32 [N, D] tensor")
+    if labels.numel() != m or top_ids.shape[0] != m:
+        raise RuntimeError("CE top-k expects one label and one row of ids per row")
+    ce_scale = (grad_loss.float() - grad_probability.float() * probabilities.float()).contiguous()
+    gtv = None if grad_top_values is None else grad_top_values.to(torch.float32).contiguous()
+    top_ids = top_ids.to(torch.long).contiguous()
+    with torch.cuda.device(device):
+        grad_hidden = torch.empty((m, h), dtype=hidden.dtype, device=device)
+        if m:
+            _lib.check(
+                _lib.library().tlce_ce_topk_apply_gradient(
+                    _ptr(unit), _ptr(hidden), _ptr(weight), _ptr(labels), _ptr(top_ids),
+                    _ptr(ce_scale), _ptr(gtv), m, h, v, _dtype_code(hidden), k,
+                    float(output_multiplier), float(logit_softcap), _ptr(grad_hidden),
+                    _stream(device),
+                ),
+                "tlce_ce_topk_apply_gradient",
+            )
+    return grad_hidden
+
+
 def dflash_ce_topk_backward(
     hidden: torch.Tensor,
     weight: torch.Tensor,

@@ -632,6 +632,125 @@ int soft_embedding_fused_impl(const FusedPlan& p, const void* hidden, const void
   return 0;
 }
 
+// ---- frozen-head cross entropy with top-k: the gradient formed in the forward ----
+// The backward of tlce_ce_topk_* recomputes the logits to form the softmax panel
+// (3 contractions per step).  Here the forward, which stages float32 logits panels
+// anyway, also writes e = exp(z - reference) * cap' of every panel in bf16 into a
+// panel over the whole vocabulary and contracts it with the weight rows once:
+//   unit[r, :] = (multiplier / sum_r) * (e . weight)[r, :] = d lse_r / d hidden[r, :]
+// (2 contractions).  The reference of a panel is the row's largest logit so far (known
+// after the panel's scan), so e <= 1; panels written before a row's maximum grew are
+// multiplied by exp(old - final) afterwards (lce_rescale_exp_rows_kernel).  The
+// backward is then one pass over rows: ce_scale[r] * unit[r, :] plus the single-row
+// terms of the label and the top-k ids, rounded once.
+struct RescaleExpArgs {
+  void* panel;             // bf16 [m_pad, ld]
+  int64_t ld;
+  int m, m_pad;
+  const float* ref_used;   // [n_panels, m_pad]
+  const float* run_max;    // [m] the final row maxima
+  int64_t panel_width;     // columns per logits panel
+  int64_t total_width;     // columns of the whole panel
+};
+
+struct TopkRowScaleArgs {
+  const float* run_sum;    // [m] sum of exp(z - max)
+  float multiplier;
+  int m, m_pad;
+  float* row_scale;        // [m_pad] multiplier / sum; 0 from m on
+};
+
+struct TopkApplyArgs {
+  const float* unit;       // [m, h] d lse / d hidden
+  const void* hidden;
+  const void* weight;
+  const int64_t* labels;
+  const int64_t* top_ids;          // [m, k]
+  const float* ce_scale;           // [m]
+  const float* grad_top_values;    // [m, k] or null
+  int m, h, k;
+  float softcap, logit_scale;
+  void* grad_hidden;               // bf16 [m, h]
+};
+
+int launch_rescale_exp_rows(const RescaleExpArgs& a, int n_panels, hipStream_t stream);
+int launch_topk_row_scale(const TopkRowScaleArgs& a, hipStream_t stream);
+int launch_topk_apply(const TopkApplyArgs& a, hipStream_t stream);
+
+struct TopkFusedLayout {
+  int64_t forward, panel, ref_used, row_scale, slabs, total;
+};
+
+// All rows must form one block of the panel budget of the forward that leaves the
+// gradients (its default: panel_bytes bounds the float32 logits panels here).
+inline bool topk_gradient_in_forward_supported(int64_t m, int64_t h, int64_t v, int dtype) {
+  return fused_gradients_supported(h, v, dtype) &&
+         make_fused_plan(m, h, v, dtype, 0).n_blocks == 1;
+}
+
+inline TopkFusedLayout topk_fused_layout(const TopkPlan& t, const FusedPlan& p, int64_t h) {
+  TopkFusedLayout l;
+  int64_t off = 0;
+  l.forward = off;    off += align256(t.forward_total);
+  l.panel = off;      off += align256(p.block_rows * p.vp * 2);
+  l.ref_used = off;   off += align256((int64_t)t.n_fpanels * p.block_rows * 4);
+  l.row_scale = off;  off += align256(p.block_rows * 4);
+  l.slabs = off;      off += align256((int64_t)p.dh_ksplit * p.block_rows * h * 4);
+  l.total = off;
+  return l;
+}
+
+template <class E>
+int topk_forward_with_gradient_impl(const TopkPlan& t, const FusedPlan& p, const void* hidden,
+                                    const void* weight, const int64_t* labels, int64_t m,
+                                    int64_t h, int64_t v, int top_k, float multiplier,
+                                    float softcap, float* losses, float* probabilities,
+                                    float* top_values, int64_t* top_ids, float* lse,
+                                    float* unit_grad, char* ws, hipStream_t stream) {
+  using T = typename E::T;
+  const TopkFusedLayout l = topk_fused_layout(t, p, h);
+  char* fws = ws + l.forward;
+  T* panel = reinterpret_cast<T*>(ws + l.panel);
+  float* ref_used = reinterpret_cast<float*>(ws + l.ref_used);
+  float* row_scale = reinterpret_cast<float*>(ws + l.row_scale);
+  float* slabs = reinterpret_cast<float*>(ws + l.slabs);
+  const int m_pad = (int)p.block_rows;
+  TopkExpHook hook;
+  hook.panel = panel; hook.ld = p.vp; hook.m_pad = m_pad; hook.ref_used = ref_used;
+  if (int rc = topk_forward_impl<E>(t, hidden, weight, labels, m, h, v, top_k, multiplier,
+                                    softcap, losses, probabilities, top_values, top_ids, lse,
+                                    fws, stream, &hook))
+    return rc;
+  const float* run_max = reinterpret_cast<const float*>(fws + t.run_max);
+  const float* run_sum = reinterpret_cast<const float*>(fws + t.run_sum);
+  if (t.n_fpanels > 1) {
+    RescaleExpArgs ra;
+    ra.panel = panel; ra.ld = p.vp; ra.m = (int)m; ra.m_pad = m_pad;
+    ra.ref_used = ref_used; ra.run_max = run_max;
+    ra.panel_width = t.vcf; ra.total_width = p.vp;
+    if (int rc = launch_rescale_exp_rows(ra, t.n_fpanels - 1, stream)) return rc;
+  }
+  TopkRowScaleArgs sa;
+  sa.run_sum = run_sum; sa.multiplier = multiplier; sa.m = (int)m; sa.m_pad = m_pad;
+  sa.row_scale = row_scale;
+  if (int rc = launch_topk_row_scale(sa, stream)) return rc;
+
+  GemmArgs g;
+  g.a = weight; g.lda = h; g.a_rows = (int)h;
+  g.b = panel; g.ldb = p.vp; g.b_rows = m_pad;
+  g.k = (int)round_up(v, 64); g.k_per_split = 0;
+  g.ni = p.n_htiles; g.nj = m_pad / E::kTile;
+  g.c = slabs; g.ldc = h; g.c_rows = m_pad; g.c_cols = (int)h;
+  g.c_split_stride = p.block_rows * h;
+  g.mode = kStoreF32;
+  if (int rc = launch_gemm<E, true, false>(g, p.dh_ksplit, kClassGradHidden, stream)) return rc;
+  ReduceSlabsArgs rs;
+  rs.slabs = slabs; rs.n_splits = p.dh_ksplit; rs.split_stride = p.block_rows * h;
+  rs.row_scale = row_scale; rs.m = (int)m; rs.h = (int)h;
+  rs.out = unit_grad;
+  return launch_reduce_slabs(rs, stream);
+}
+
 #define TLCE_LAUNCHERS_EXP_PANEL(X, E)                                                  \
   X int launch_exp_panel_variant<E, false, false>(const ExpPanelArgs&, hipStream_t);    \
   X int launch_exp_panel_variant<E, true, false>(const ExpPanelArgs&, hipStream_t);     \
@@ -644,6 +763,10 @@ int soft_embedding_fused_impl(const FusedPlan& p, const void* hidden, const void
   X int soft_embedding_fused_impl<E>(const FusedPlan&, const void*, const void*, int64_t,        \
                                      int64_t, int64_t, int, float, float, void*, char*,          \
                                      hipStream_t);                                               \
+  X int topk_forward_with_gradient_impl<E>(const TopkPlan&, const FusedPlan&, const void*,       \
+                                           const void*, const int64_t*, int64_t, int64_t,        \
+                                           int64_t, int, float, float, float*, float*, float*,   \
+                                           int64_t*, float*, float*, char*, hipStream_t);        \
   X int deferred_grad_weight_impl<E>(const FusedPlan&, const void*, int64_t, int64_t, int64_t,   \
                                      int, const float*, const float*, int, const int64_t*,       \
                                      const int64_t*, void*, char*, hipStream_t);

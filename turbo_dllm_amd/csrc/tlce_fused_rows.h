@@ -199,6 +199,125 @@ __global__ __launch_bounds__(256) void lce_reduce_scaled_slabs_kernel(ReduceSlab
   }
 }
 
+// One row and 2048 columns per workgroup, 8 columns per thread.
+__global__ __launch_bounds__(256) void lce_exp_from_logits_kernel(ExpFromLogitsArgs p) {
+  const int r = blockIdx.x;
+  const int c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (c >= p.width) return;
+  __bf16* dst = static_cast<__bf16*>(p.out) + (int64_t)r * p.ld_out + p.col0 + c;
+  if (r >= p.m) {
+    store4<__bf16>(dst, 0.0f, 0.0f, 0.0f, 0.0f);
+    store4<__bf16>(dst + 4, 0.0f, 0.0f, 0.0f, 0.0f);
+    return;
+  }
+  const float ref = p.run_max[r];
+  if (c == 0) p.ref_used[r] = ref;
+  const float* src = p.logits + (int64_t)r * p.ld + c;
+  const f32x4_t z0 = *reinterpret_cast<const f32x4_t*>(src);
+  const f32x4_t z1 = *reinterpret_cast<const f32x4_t*>(src + 4);
+  float e[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float z = i < 4 ? z0[i] : z1[i - 4];
+    float x = __expf(z - ref);            // -inf (past the vocabulary) gives 0
+    if (p.softcap > 0.0f) {
+      const float t = z / p.softcap;
+      x = (z > -INFINITY) ? x * (1.0f - t * t) : 0.0f;
+    }
+    e[i] = x;
+  }
+  store4<__bf16>(dst, e[0], e[1], e[2], e[3]);
+  store4<__bf16>(dst + 4, e[4], e[5], e[6], e[7]);
+}
+
+// blockIdx.y = logits panel (all but the last, which was written with the final
+// maxima): rows whose maximum grew after the panel was written are brought to the
+// final reference.
+__global__ __launch_bounds__(256) void lce_rescale_exp_rows_kernel(RescaleExpArgs p) {
+  const int r = blockIdx.x;
+  const int j = blockIdx.y;
+  const float used = p.ref_used[(int64_t)j * p.m_pad + r];
+  const float fin = p.run_max[r];
+  if (used == fin) return;
+  const float f = __expf(used - fin);
+  const int64_t c0 = (int64_t)j * p.panel_width;
+  const int64_t c1 = min(c0 + p.panel_width, p.total_width);
+  __bf16* row = static_cast<__bf16*>(p.panel) + (int64_t)r * p.ld;
+  typedef __bf16 v8_t __attribute__((ext_vector_type(8)));
+  for (int64_t c = c0 + threadIdx.x * 8; c < c1; c += 256 * 8) {
+    v8_t x = *reinterpret_cast<v8_t*>(row + c);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = from_float<__bf16>(to_float<__bf16>(x[i]) * f);
+    *reinterpret_cast<v8_t*>(row + c) = x;
+  }
+}
+
+__global__ __launch_bounds__(256) void lce_topk_row_scale_kernel(TopkRowScaleArgs p) {
+  const int r = blockIdx.x * 256 + threadIdx.x;
+  if (r >= p.m_pad) return;
+  p.row_scale[r] = (r < p.m) ? p.multiplier / p.run_sum[r] : 0.0f;
+}
+
+// One workgroup per row: grad_hidden[r, :] = ce_scale[r] * unit[r, :]
+//   - ce_scale[r] * d'(label) * W[label] + sum_j grad_top_values[r, j] * d'(id_j) * W[id_j]
+// (dflash_linear_topk.py:196-225) with d'(v) = multiplier * (1 - tanh^2(multiplier *
+// h.W[v] / cap)) (multiplier alone without a cap), rounded once.  The coefficients
+// of the single-row terms are formed first (one dot product each), then every
+// column is summed in float32.
+constexpr int kTopkApplyMaxEntries = 257;   // top_k <= 256, plus the label
+
+template <typename T>
+__global__ __launch_bounds__(256) void lce_topk_apply_kernel(TopkApplyArgs p) {
+  __shared__ float red[4];
+  __shared__ float coef[kTopkApplyMaxEntries];
+  __shared__ int64_t ids[kTopkApplyMaxEntries];
+  const int t = threadIdx.x;
+  const int lane = t & 63, wave = t >> 6;
+  const int r = blockIdx.x;
+  const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
+  const float scale = p.ce_scale[r];
+  const int n_entries = (p.grad_top_values != nullptr ? p.k : 0) + 1;
+  for (int e = 0; e < n_entries; ++e) {
+    const bool is_label = e == n_entries - 1;
+    const int64_t id = is_label ? p.labels[r] : p.top_ids[(int64_t)r * p.k + e];
+    const float weight_in = is_label ? -scale : p.grad_top_values[(int64_t)r * p.k + e];
+    float c = 0.0f;
+    if (weight_in != 0.0f) {   // workgroup-uniform
+      const T* wrow = static_cast<const T*>(p.weight) + id * (int64_t)p.h;
+      float dot = 0.0f;
+      for (int k = t; k < p.h; k += 256)
+        dot = fmaf(to_float<T>(hrow[k]), to_float<T>(wrow[k]), dot);
+      dot = wave_sum(dot);
+      if (lane == 0) red[wave] = dot;
+      __syncthreads();
+      const float raw = (red[0] + red[1] + red[2] + red[3]) * p.logit_scale;
+      __syncthreads();
+      float deriv = p.logit_scale;
+      if (p.softcap > 0.0f) {
+        const float th = tanhf(raw / p.softcap);
+        deriv *= 1.0f - th * th;
+      }
+      c = weight_in * deriv;
+    }
+    if (t == 0) {
+      coef[e] = c;
+      ids[e] = id;
+    }
+  }
+  __syncthreads();
+  const float* unit = p.unit + (int64_t)r * p.h;
+  T* out = static_cast<T*>(p.grad_hidden) + (int64_t)r * p.h;
+  for (int k = t; k < p.h; k += 256) {
+    float acc = scale * unit[k];
+    for (int e = 0; e < n_entries; ++e) {
+      if (coef[e] != 0.0f)
+        acc = fmaf(coef[e], to_float<T>(static_cast<const T*>(p.weight)[ids[e] * (int64_t)p.h + k]),
+                   acc);
+    }
+    out[k] = from_float<T>(acc);
+  }
+}
+
 // 64 rows per workgroup of 16 waves, the rows across the lanes (the partials are
 // stored [tile][row]: a wave reads 256 consecutive bytes per tile); wave w adds the
 // tiles w, w + 16, ... in order and the 16 sums are merged in a fixed order.

@@ -802,12 +802,35 @@ int launch_logits_panel_variant(const LogitsPanelArgs& a, hipStream_t stream) {
   return 0;
 }
 
+// After the scan of a float32 logits panel: exp(logit - the row's largest logit so
+// far) * cap' of that panel, rounded to bf16, into a panel over the whole vocabulary
+// (the operand of the gradient contraction formed in the forward).
+struct ExpFromLogitsArgs {
+  const float* logits;   // [m, ld] float32 (columns past the vocabulary hold -inf)
+  int64_t ld;
+  int m, m_pad;          // rows with logits; rows of `out` to define (zeros from m on)
+  int width;             // columns of this logits panel, a multiple of 8
+  float softcap;
+  const float* run_max;  // [m] the reference: the row's largest logit so far
+  float* ref_used;       // [m] out: the reference this panel was written with
+  void* out;             // bf16 [m_pad, ld_out]; this panel goes to columns col0 ...
+  int64_t ld_out, col0;
+};
+int launch_exp_from_logits(const ExpFromLogitsArgs& a, hipStream_t stream);
+
+struct TopkExpHook {
+  void* panel;           // bf16 [m_pad, ld]
+  int64_t ld;
+  int m_pad;
+  float* ref_used;       // [n_fpanels, m_pad]
+};
+
 template <class E>
 int topk_forward_impl(const TopkPlan& t, const void* hidden, const void* weight,
                       const int64_t* labels, int64_t m, int64_t h, int64_t v, int top_k,
                       float multiplier, float softcap, float* losses, float* probabilities,
                       float* top_values, int64_t* top_ids, float* lse, char* ws,
-                      hipStream_t stream) {
+                      hipStream_t stream, const TopkExpHook* hook = nullptr) {
   using T = typename E::T;
   const Plan& p = t.plan;
   float* run_max = reinterpret_cast<float*>(ws + t.run_max);
@@ -833,6 +856,14 @@ int topk_forward_impl(const TopkPlan& t, const void* hidden, const void* weight,
     sa.k = top_k; sa.first = pi == 0;
     sa.run_max = run_max; sa.run_sum = run_sum; sa.top_values = top_values; sa.top_ids = top_ids;
     if (int rc = launch_topk_scan(sa, stream)) return rc;
+    if (hook != nullptr) {
+      ExpFromLogitsArgs xa;
+      xa.logits = panel; xa.ld = t.vcf; xa.m = (int)m; xa.m_pad = hook->m_pad;
+      xa.width = (int)width; xa.softcap = softcap;
+      xa.run_max = run_max; xa.ref_used = hook->ref_used + (int64_t)pi * hook->m_pad;
+      xa.out = hook->panel; xa.ld_out = hook->ld; xa.col0 = v0;
+      if (int rc = launch_exp_from_logits(xa, stream)) return rc;
+    }
   }
   TopkFinishArgs fa;
   fa.hidden = hidden; fa.weight = weight; fa.labels = labels; fa.m = (int)m; fa.h = (int)h;
@@ -971,7 +1002,8 @@ int soft_embedding_impl(const Plan& fp, const Plan& bp, const SoftEmbeddingLayou
                             hipStream_t);                                                       \
   X int topk_forward_impl<E>(const TopkPlan&, const void*, const void*, const int64_t*,         \
                              int64_t, int64_t, int64_t, int, float, float, float*, float*,      \
-                             float*, int64_t*, float*, char*, hipStream_t);                     \
+                             float*, int64_t*, float*, char*, hipStream_t,                      \
+                             const TopkExpHook*);                                               \
   X int topk_backward_impl<E>(const TopkPlan&, const void*, const void*, const int64_t*,        \
                               const float*, const int64_t*, const float*, const float*,         \
                               int64_t, int64_t, int64_t, int, int, float, float, void*, char*,  \

@@ -89,6 +89,36 @@ int launch_scale_rows(const ScaleRowsArgs& a, hipStream_t stream) {
   return 0;
 }
 
+int launch_exp_from_logits(const ExpFromLogitsArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_exp_from_logits_kernel<<<dim3((unsigned)a.m_pad, (unsigned)ceil_div(a.width, 2048)), 256, 0,
+                               stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_rescale_exp_rows(const RescaleExpArgs& a, int n_panels, hipStream_t stream) {
+  if (n_panels <= 0 || a.m <= 0) return 0;
+  ScopedTimer timer(kClassOther, stream);
+  lce_rescale_exp_rows_kernel<<<dim3((unsigned)a.m, (unsigned)n_panels), 256, 0, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_topk_row_scale(const TopkRowScaleArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_topk_row_scale_kernel<<<(int)ceil_div(a.m_pad, 256), 256, 0, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+int launch_topk_apply(const TopkApplyArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_topk_apply_kernel<__bf16><<<a.m, 256, 0, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
 int launch_soft_rows(const SoftRowsArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassCombine, stream);
   lce_soft_rows_kernel<<<(int)ceil_div(a.m_pad, 64), 64 * kSoftRowsWaves, 0, stream>>>(a);
@@ -660,6 +690,73 @@ extern "C" int tlce_ce_topk_forward(const void* hidden, const void* weight, cons
                 topk_forward_impl<E>(t, hidden, weight, labels, m, h, v, top_k, output_multiplier,
                                      logit_softcap, losses, probabilities, top_values, top_ids,
                                      lse, static_cast<char*>(workspace), stream));
+}
+
+extern "C" int tlce_ce_topk_gradient_in_forward_supported(int64_t m, int64_t h, int64_t v,
+                                                          int dtype) {
+  if (m <= 0 || h <= 0 || v <= 0) return 0;
+  return topk_gradient_in_forward_supported(m, h, v, dtype) ? 1 : 0;
+}
+
+extern "C" int64_t tlce_ce_topk_forward_with_gradient_workspace_bytes(int64_t m, int64_t h,
+                                                                      int64_t v, int dtype,
+                                                                      int64_t panel_bytes) {
+  if (m <= 0 || h <= 0 || v <= 0 || !topk_gradient_in_forward_supported(m, h, v, dtype)) return -1;
+  return topk_fused_layout(topk_plan(m, h, v, dtype, panel_bytes),
+                           make_fused_plan(m, h, v, dtype, 0), h).total;
+}
+
+extern "C" int tlce_ce_topk_forward_with_gradient(
+    const void* hidden, const void* weight, const int64_t* labels, int64_t m, int64_t h,
+    int64_t v, int dtype, int top_k, float output_multiplier, float logit_softcap, float* losses,
+    float* probabilities, float* top_values, int64_t* top_ids, float* lse,
+    float* unit_grad_hidden_f32, int64_t panel_bytes, void* workspace, int64_t workspace_bytes,
+    void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = topk_validate(hidden, weight, labels, m, h, v, dtype, top_k)) return rc;
+  if (m == 0) return 0;
+  TLCE_REQUIRE(topk_gradient_in_forward_supported(m, h, v, dtype),
+               "ce_topk_forward_with_gradient: needs bf16 inputs, h and v multiples of 64 and all "
+               "rows in one block of the exponentiated-logits panel (m=%lld, v=%lld)",
+               (long long)m, (long long)v);
+  TLCE_REQUIRE(losses && probabilities && top_values && top_ids && lse && unit_grad_hidden_f32 &&
+                   workspace,
+               "ce_topk_forward_with_gradient: null pointer");
+  TLCE_REQUIRE(((uintptr_t)unit_grad_hidden_f32 & 15) == 0,
+               "ce_topk_forward_with_gradient: the gradient buffer must be 16-byte aligned");
+  const TopkPlan t = topk_plan(m, h, v, dtype, panel_bytes);
+  const FusedPlan p = make_fused_plan(m, h, v, dtype, 0);
+  const int64_t need = topk_fused_layout(t, p, h).total;
+  TLCE_REQUIRE(workspace_bytes >= need,
+               "ce_topk_forward_with_gradient: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+               "ce_topk_forward_with_gradient: workspace must be 256-byte aligned");
+  return topk_forward_with_gradient_impl<MfmaDirect4Engine<__bf16>>(
+      t, p, hidden, weight, labels, m, h, v, top_k, output_multiplier, logit_softcap, losses,
+      probabilities, top_values, top_ids, lse, unit_grad_hidden_f32,
+      static_cast<char*>(workspace), stream);
+}
+
+extern "C" int tlce_ce_topk_apply_gradient(const float* unit_grad_hidden_f32, const void* hidden,
+                                           const void* weight, const int64_t* labels,
+                                           const int64_t* top_ids, const float* ce_scale,
+                                           const float* grad_top_values, int64_t m, int64_t h,
+                                           int64_t v, int dtype, int top_k,
+                                           float output_multiplier, float logit_softcap,
+                                           void* grad_hidden, void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = topk_validate(hidden, weight, labels, m, h, v, dtype, top_k)) return rc;
+  TLCE_REQUIRE(dtype == TLCE_DTYPE_BF16, "ce_topk_apply_gradient: bf16 only");
+  if (m == 0) return 0;
+  TLCE_REQUIRE(unit_grad_hidden_f32 && top_ids && ce_scale && grad_hidden,
+               "ce_topk_apply_gradient: null pointer");
+  TopkApplyArgs a;
+  a.unit = unit_grad_hidden_f32; a.hidden = hidden; a.weight = weight; a.labels = labels;
+  a.top_ids = top_ids; a.ce_scale = ce_scale; a.grad_top_values = grad_top_values;
+  a.m = (int)m; a.h = (int)h; a.k = top_k;
+  a.softcap = logit_softcap; a.logit_scale = output_multiplier; a.grad_hidden = grad_hidden;
+  return launch_topk_apply(a, stream);
 }
 
 extern "C" int tlce_ce_topk_backward(const void* hidden, const void* weight,

@@ -24,6 +24,22 @@ class _NativeFrozenLinearCETopK(torch.autograd.Function):
         hidden = hidden.contiguous()
         weight = weight.contiguous()
         labels = labels.to(device=hidden.device, dtype=torch.long).contiguous()
+        # d lse / d hidden while the forward's logits panels exist (one contraction more
+        # in the forward, none in the backward), where the library takes the operands
+        from . import options
+        ctx.fused = (bool(ctx.needs_input_grad[0]) and options.get_gradient_mode() == "forward"
+                     and native.ce_topk_gradient_in_forward_supported(hidden, weight))
+        if ctx.fused:
+            loss, probability, top_values, top_ids, lse, unit = (
+                native.dflash_ce_topk_forward_with_gradient(
+                    hidden, weight, labels, top_k=int(top_k),
+                    output_multiplier=float(output_multiplier),
+                    logit_softcap=float(logit_softcap)))
+            ctx.save_for_backward(hidden, weight, labels, unit, probability, top_ids)
+            ctx.output_multiplier = float(output_multiplier)
+            ctx.logit_softcap = float(logit_softcap)
+            ctx.mark_non_differentiable(top_ids)
+            return loss, probability, top_values, top_ids
         loss, probability, top_values, top_ids, lse = native.dflash_ce_topk_forward(
             hidden, weight, labels, top_k=int(top_k), row_block_size=0,
             output_multiplier=float(output_multiplier), logit_softcap=float(logit_softcap),
@@ -41,6 +57,15 @@ class _NativeFrozenLinearCETopK(torch.autograd.Function):
 
         hidden, weight, labels, lse, probability, top_ids = ctx.saved_tensors
         zeros = torch.zeros_like(probability)
+        if ctx.fused:
+            grad_hidden = native.dflash_ce_topk_apply_gradient(
+                lse, hidden, weight, labels, probability, top_ids,   # lse slot: d lse / d hidden
+                zeros if grad_loss is None else grad_loss,
+                zeros if grad_probability is None else grad_probability,
+                grad_top_values,
+                output_multiplier=ctx.output_multiplier, logit_softcap=ctx.logit_softcap,
+            )
+            return grad_hidden, None, None, None, None, None
         with native.panel_budget(ctx.panel_bytes):
             grad_hidden = native.dflash_ce_topk_backward(
                 hidden, weight, labels, lse, probability, top_ids,
