@@ -354,6 +354,12 @@ int tlce_soft_embedding(const void* hidden, const void* weight, int64_t m,
  * statistics pass over the teacher head, then per panel the teacher
  * probabilities and one pass over the draft head that yields both the loss
  * terms and the draft's softmax statistics.
+ * teacher_probabilities (optional, both calls): a caller-owned buffer of
+ * tlce_kl_teacher_probabilities_bytes (2 bytes per padded row and vocabulary
+ * entry: 2.5 GB at m = 8192, v = 151936) that the forward fills with the teacher
+ * probabilities of every panel and the backward reads instead of producing them
+ * again: 5 contractions per forward + backward instead of 6 (the reference runs
+ * 5 GEMMs, fused_linear_ce_cuda.cu:1270-1509).  NULL: nothing is kept.
  *   draft_hidden [m,h_draft], draft_weight [v,h_draft], teacher_hidden
  *   [m,h_teacher], teacher_weight [v,h_teacher], all `dtype`; losses,
  *   draft_lse, teacher_lse, grad_output: float32 [m]; grad_hidden [m,h_draft]. */
@@ -364,13 +370,18 @@ int tlce_kl_forward(const void* draft_hidden, const void* draft_weight,
                     const void* teacher_hidden, const void* teacher_weight,
                     int64_t m, int64_t h_draft, int64_t h_teacher, int64_t v,
                     int dtype, float logit_softcap, float* losses,
-                    float* draft_lse, float* teacher_lse, int64_t panel_bytes,
+                    float* draft_lse, float* teacher_lse,
+                    void* teacher_probabilities, int64_t panel_bytes,
                     void* workspace, int64_t workspace_bytes, void* stream);
+
+int64_t tlce_kl_teacher_probabilities_bytes(int64_t m, int64_t h_draft,
+                                            int64_t h_teacher, int64_t v, int dtype);
 
 int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
                      const void* teacher_hidden, const void* teacher_weight,
                      const float* draft_lse, const float* teacher_lse,
-                     const float* grad_output, int64_t m, int64_t h_draft,
+                     const float* grad_output, const void* teacher_probabilities,
+                     int64_t m, int64_t h_draft,
                      int64_t h_teacher, int64_t v, int dtype, float logit_softcap,
                      void* grad_hidden, int64_t panel_bytes, void* workspace,
                      int64_t workspace_bytes, void* stream);

@@ -97,3 +97,57 @@ def test_same_head_gives_zero(gpu_device):
     torch.cuda.synchronize()
     assert float(got.abs().max()) < 2e-3
     assert float(x.grad.float().abs().max()) < 2e-2 * float(w.float().abs().max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,hd,ht,v,softcap", [
+    (torch.bfloat16, 128, 192, 4096, None),     # direct engine, panels staged through LDS
+    (torch.bfloat16, 128, 128, 2048, 6.0),
+    (torch.float16, 72, 72, 1000, None),        # staged engine, plain loads of the panel
+    (torch.float32, 33, 40, 301, None),
+])
+def test_kept_teacher_probabilities_give_the_same_gradient(gpu_device, dtype, hd, ht, v, softcap,
+                                                           set_panel_budget):
+    """The default keeps the teacher probabilities of the whole vocabulary from the
+    forward to the backward (5 contractions per step); gradient mode "recompute" produces
+    them a second time (6).  Same producer, same values: the gradients agree bit for bit,
+    over several vocabulary panels.  Which one ran is read from the launch counts of the
+    backward, run on this thread through the shim."""
+    from turbo_dllm_amd import _lib, options
+    from turbo_dllm_amd import chunked_linear_ce_native as native
+    print("[case] kept teacher probabilities", dtype, hd, ht, v, softcap, flush=True)
+    m = 300
+    set_panel_budget(512 * 512 * 2)          # panels of 512 columns
+    gen = torch.Generator().manual_seed(v)
+    ops = [torch.randn(m, hd, generator=gen), torch.randn(v, hd, generator=gen) * 0.2,
+           torch.randn(m, ht, generator=gen), torch.randn(v, ht, generator=gen) * 0.2]
+    ops = [t.to(dtype).to(gpu_device) for t in ops]
+    go = torch.rand(m, generator=gen).to(gpu_device)
+    grads = {}
+    for mode in options.GRADIENT_MODES:
+        x = ops[0].clone().requires_grad_(True)
+        with options.gradient_mode(mode):
+            losses = frozen_linear_kl(x, ops[1], ops[2], ops[3], logit_softcap=softcap)
+        losses.backward(go)
+        torch.cuda.synchronize()
+        grads[mode] = (losses.detach().cpu(), x.grad.cpu())
+    assert torch.equal(grads["forward"][0], grads["recompute"][0])
+    assert torch.equal(grads["forward"][1], grads["recompute"][1])
+    # through the shim on this thread: the backward that reads the kept panel launches the
+    # panel kernels once per panel (the draft pass), the other twice (teacher, then draft)
+    cap = float(softcap or 0.0)
+    losses, dlse, tlse, kept = native.dflash_kl_forward(*ops, cap, keep_teacher_probabilities=True)
+    assert kept.dtype == torch.uint8 and kept.numel() == native.kl_teacher_probabilities_bytes(
+        ops[0], ops[1], ops[2])
+    counts = {}
+    for name, panel in (("kept", kept), ("again", None)):
+        with _lib.kernel_profile() as prof:
+            g = native.dflash_kl_backward(*ops, dlse, tlse, go, cap, teacher_probabilities=panel)
+            torch.cuda.synchronize()
+        counts[name] = prof.launches["grad_logits_panel"]
+        assert torch.equal(g.cpu(), grads["forward"][1])
+    assert counts["again"] == 2 * counts["kept"] and counts["kept"] >= 1
+    if dtype == torch.bfloat16:
+        assert counts["kept"] == v // 512          # several vocabulary panels
+    with pytest.raises(RuntimeError, match="teacher_probabilities"):
+        native.dflash_kl_backward(*ops, dlse, tlse, go, cap, teacher_probabilities=kept[:16])

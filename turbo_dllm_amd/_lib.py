@@ -228,14 +228,18 @@ SIGNATURES = {
             c_void_p, c_void_p, c_void_p, c_void_p,             # draft h/w, teacher h/w
             c_int64, c_int64, c_int64, c_int64, c_int,          # m h_draft h_teacher v dtype
             c_float, c_void_p, c_void_p, c_void_p,              # softcap losses draft_lse teacher_lse
+            c_void_p,                                           # teacher_probabilities (or null)
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_kl_teacher_probabilities_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int64, c_int]),
     "tlce_kl_backward": (
         c_int,
         [
             c_void_p, c_void_p, c_void_p, c_void_p,             # draft h/w, teacher h/w
             c_void_p, c_void_p, c_void_p,                       # draft_lse teacher_lse grad_output
+            c_void_p,                                           # teacher_probabilities (or null)
             c_int64, c_int64, c_int64, c_int64, c_int,          # m h_draft h_teacher v dtype
             c_float, c_void_p,                                  # softcap grad_hidden
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream

@@ -1144,10 +1144,15 @@ def dflash_kl_forward(
     teacher_hidden: torch.Tensor,
     teacher_weight: torch.Tensor,
     logit_softcap: float,
-) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    keep_teacher_probabilities: bool = False,
+) -> tuple[torch.Tensor, ...]:
     """``(losses, draft_lse, teacher_lse)``, float32 [N]: per-token forward KL
     of the teacher head against the draft head without a logits buffer
-    (reference shim, chunked_linear_ce_native.py:259-274)."""
+    (reference shim, chunked_linear_ce_native.py:259-274).
+
+    ``keep_teacher_probabilities``: also return the teacher probabilities of the
+    whole vocabulary (a uint8 buffer, 2 bytes per padded row and vocabulary entry)
+    for ``dflash_kl_backward`` to read instead of producing them a second time."""
     device, dh, dw, th, tw = _kl_operands(draft_hidden, draft_weight, teacher_hidden,
                                           teacher_weight)
     m, hd = dh.shape
@@ -1158,18 +1163,32 @@ def dflash_kl_forward(
         losses = torch.empty(m, dtype=torch.float32, device=device)
         draft_lse = torch.empty(m, dtype=torch.float32, device=device)
         teacher_lse = torch.empty(m, dtype=torch.float32, device=device)
+        kept = None
         if m == 0:
-            return losses, draft_lse, teacher_lse
+            return ((losses, draft_lse, teacher_lse, kept) if keep_teacher_probabilities
+                    else (losses, draft_lse, teacher_lse))
+        if keep_teacher_probabilities:
+            kept = torch.empty(lib.tlce_kl_teacher_probabilities_bytes(m, hd, ht, v, code),
+                               dtype=torch.uint8, device=device)
         ws = _workspace(lib.tlce_kl_workspace_bytes(m, hd, ht, v, code, get_panel_bytes()), device)
         _lib.check(
             lib.tlce_kl_forward(
                 _ptr(dh), _ptr(dw), _ptr(th), _ptr(tw), m, hd, ht, v, code,
                 float(logit_softcap), _ptr(losses), _ptr(draft_lse), _ptr(teacher_lse),
-                get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
+                _ptr(kept), get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_kl_forward",
         )
+    if keep_teacher_probabilities:
+        return losses, draft_lse, teacher_lse, kept
     return losses, draft_lse, teacher_lse
+
+
+def kl_teacher_probabilities_bytes(draft_hidden, draft_weight, teacher_hidden) -> int:
+    """Size of the buffer ``dflash_kl_forward(keep_teacher_probabilities=True)`` fills."""
+    m, hd = draft_hidden.shape
+    return int(_lib.library().tlce_kl_teacher_probabilities_bytes(
+        m, hd, teacher_hidden.shape[1], draft_weight.shape[0], _dtype_code(draft_hidden)))
 
 
 def dflash_kl_backward(
@@ -1181,9 +1200,11 @@ def dflash_kl_backward(
     teacher_lse: torch.Tensor,
     grad_output: torch.Tensor,
     logit_softcap: float,
+    teacher_probabilities: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """Gradient of the per-token KL with respect to the draft hidden states
-    (reference shim, chunked_linear_ce_native.py:277-296)."""
+    (reference shim, chunked_linear_ce_native.py:277-296).  ``teacher_probabilities``:
+    what the forward kept for these operands, or None to produce them again."""
     device, dh, dw, th, tw = _kl_operands(draft_hidden, draft_weight, teacher_hidden,
                                           teacher_weight)
     _require_device(draft_lse, teacher_lse, grad_output)
@@ -1196,6 +1217,13 @@ def dflash_kl_backward(
     draft_lse = draft_lse.reshape(-1).to(torch.float32).contiguous()
     teacher_lse = teacher_lse.reshape(-1).to(torch.float32).contiguous()
     lib = _lib.library()
+    if teacher_probabilities is not None:
+        _require_device(teacher_probabilities)
+        need = lib.tlce_kl_teacher_probabilities_bytes(m, hd, ht, v, code)
+        if (teacher_probabilities.dtype != torch.uint8 or not teacher_probabilities.is_contiguous()
+                or teacher_probabilities.numel() < need):
+            raise RuntimeError("teacher_probabilities must be the uint8 buffer the forward kept "
+                               f"for these operands ({need} bytes)")
     with torch.cuda.device(device):
         grad_hidden = torch.empty((m, hd), dtype=dh.dtype, device=device)
         if m == 0:
@@ -1205,7 +1233,7 @@ def dflash_kl_backward(
             lib.tlce_kl_backward(
                 _ptr(dh), _ptr(dw), _ptr(th), _ptr(tw),
                 _ptr(draft_lse), _ptr(teacher_lse), _ptr(grad_output),
-                m, hd, ht, v, code, float(logit_softcap), _ptr(grad_hidden),
+                _ptr(teacher_probabilities), m, hd, ht, v, code, float(logit_softcap), _ptr(grad_hidden),
                 get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
             ),
             "tlce_kl_backward",

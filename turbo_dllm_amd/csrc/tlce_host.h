@@ -657,7 +657,24 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
              const float* teacher_lse, const float* ones, const float* scale, int64_t m,
              int64_t hd, int64_t ht, int64_t v, float softcap, int64_t v0, int64_t width,
              void* g, float* loss_part, float* tsum_part, float* part_max, float* part_sum,
-             int mode, hipStream_t stream) {
+             int mode, hipStream_t stream, void* kept = nullptr, int64_t kept_ld = 0,
+             bool kept_is_written = false) {
+  // kept: a buffer over the whole vocabulary [mp, kept_ld] that holds the teacher
+  // probabilities between forward and backward.  The forward produces each panel into
+  // it (and reads it there); the backward (kept_is_written) skips the producer and
+  // reads the panel from it, writing the logit gradients to g.
+  void* teacher_panel = kept != nullptr ? static_cast<char*>(kept) + v0 * (int64_t)sizeof(typename E::T) : g;
+  const int64_t teacher_ld = kept != nullptr ? kept_ld : pd.vc;
+  KlPanelArgs ka;
+  ka.hidden = draft_hidden; ka.weight = draft_weight; ka.lse = draft_lse; ka.scale = scale;
+  ka.m = (int)m; ka.h = (int)hd; ka.v = (int)v; ka.softcap = softcap;
+  ka.v0 = (int)v0; ka.n_ttiles = pd.n_ttiles; ka.n_ptiles = (int)(width / pd.tile);
+  ka.loss_part = loss_part; ka.tsum_part = tsum_part;
+  ka.part_max = part_max; ka.part_sum = part_sum; ka.part_ld = (int)pd.mp; ka.mode = mode;
+  if (kept != nullptr && kept_is_written) {
+    ka.panel = g; ka.ld = pd.vc; ka.panel_in = teacher_panel; ka.ld_in = teacher_ld;
+    return launch_kl_panel<E>(ka, stream);
+  }
   GradLogitsArgs ga;
   ga.hidden = teacher_hidden; ga.weight = teacher_weight; ga.bias = nullptr;
   ga.labels = nullptr; ga.lse = teacher_lse; ga.scale = ones;
@@ -666,15 +683,10 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
   ga.label_offset = 0; ga.probabilities = 1; ga.cap_grad = 0; ga.logit_scale = 1.0f;
   ga.v0 = (int)v0;
   ga.n_ttiles = pd.n_ttiles; ga.n_ptiles = (int)(width / pd.tile);
-  ga.g = g; ga.ldg = pd.vc; ga.gt = nullptr; ga.ldgt = 0;
+  ga.g = teacher_panel; ga.ldg = teacher_ld; ga.gt = nullptr; ga.ldgt = 0;
   ga.grad_bias = nullptr;
   if (int rc = launch_grad_logits<E>(ga, stream)) return rc;
-  KlPanelArgs ka;
-  ka.hidden = draft_hidden; ka.weight = draft_weight; ka.lse = draft_lse; ka.scale = scale;
-  ka.m = (int)m; ka.h = (int)hd; ka.v = (int)v; ka.softcap = softcap;
-  ka.v0 = (int)v0; ka.n_ttiles = pd.n_ttiles; ka.n_ptiles = (int)(width / pd.tile);
-  ka.panel = g; ka.ld = pd.vc; ka.loss_part = loss_part; ka.tsum_part = tsum_part;
-  ka.part_max = part_max; ka.part_sum = part_sum; ka.part_ld = (int)pd.mp; ka.mode = mode;
+  ka.panel = teacher_panel; ka.ld = teacher_ld;
   return launch_kl_panel<E>(ka, stream);
 }
 
@@ -683,7 +695,7 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
                     const void* draft_weight, const void* teacher_hidden,
                     const void* teacher_weight, int64_t m, int64_t hd, int64_t ht, int64_t v,
                     int dtype, float softcap, float* losses, float* draft_lse, float* teacher_lse,
-                    char* ws, hipStream_t stream) {
+                    char* ws, hipStream_t stream, void* kept_teacher = nullptr) {
   using T = typename E::T;
   // teacher statistics first: its probabilities need the teacher lse
   if (int rc = forward_impl<E>(pt, teacher_hidden, teacher_weight, nullptr, nullptr, nullptr, m,
@@ -710,7 +722,7 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
     if (int rc = kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight,
                              nullptr, teacher_lse, ones, nullptr, m, hd, ht, v, softcap, v0,
                              width, g, loss_part, tsum_part, part_max, part_sum, kKlLoss,
-                             stream))
+                             stream, kept_teacher, pd.vp, false))
       return rc;
   }
   CombineArgs ca;
@@ -738,7 +750,8 @@ int kl_backward_impl(const Plan& pd, const KlLayout& l, const void* draft_hidden
                      const void* draft_weight, const void* teacher_hidden,
                      const void* teacher_weight, const float* draft_lse, const float* teacher_lse,
                      const float* grad_output, int64_t m, int64_t hd, int64_t ht, int64_t v,
-                     int dtype, float softcap, void* grad_hidden, char* ws, hipStream_t stream) {
+                     int dtype, float softcap, void* grad_hidden, char* ws, hipStream_t stream,
+                     const void* kept_teacher = nullptr) {
   float* ones = reinterpret_cast<float*>(ws + l.ones);
   char* bws = ws + l.backward;
   const BackwardLayout bl = backward_layout(pd, m, hd, dtype, false);
@@ -753,7 +766,8 @@ int kl_backward_impl(const Plan& pd, const KlLayout& l, const void* draft_hidden
   auto produce = [&](int64_t v0, int64_t width, void* g, void*) -> int {
     return kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight, draft_lse,
                        teacher_lse, ones, scale, m, hd, ht, v, softcap, v0, width, g, nullptr,
-                       nullptr, nullptr, nullptr, kKlGrad, stream);
+                       nullptr, nullptr, nullptr, kKlGrad, stream,
+                       const_cast<void*>(kept_teacher), pd.vp, kept_teacher != nullptr);
   };
   return panel_contractions<E>(pd, bl, draft_hidden, draft_weight, nullptr, m, m, hd, v, dtype,
                                grad_hidden, nullptr, bws, stream, produce);
@@ -995,11 +1009,11 @@ int soft_embedding_impl(const Plan& fp, const Plan& bp, const SoftEmbeddingLayou
                                float, void*, char*, hipStream_t);                               \
   X int kl_forward_impl<E>(const Plan&, const Plan&, const KlLayout&, const void*, const void*, \
                            const void*, const void*, int64_t, int64_t, int64_t, int64_t, int,   \
-                           float, float*, float*, float*, char*, hipStream_t);                  \
+                           float, float*, float*, float*, char*, hipStream_t, void*);           \
   X int kl_backward_impl<E>(const Plan&, const KlLayout&, const void*, const void*,             \
                             const void*, const void*, const float*, const float*, const float*, \
                             int64_t, int64_t, int64_t, int64_t, int, float, void*, char*,       \
-                            hipStream_t);                                                       \
+                            hipStream_t, const void*);                                          \
   X int topk_forward_impl<E>(const TopkPlan&, const void*, const void*, const int64_t*,         \
                              int64_t, int64_t, int64_t, int, float, float, float*, float*,      \
                              float*, int64_t*, float*, char*, hipStream_t,                      \

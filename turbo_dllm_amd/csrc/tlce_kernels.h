@@ -642,6 +642,8 @@ struct KlPanelArgs {
   int n_ttiles, n_ptiles;
   void* panel;          // [mp, ld] teacher probabilities in, logit gradients out
   int64_t ld;
+  const void* panel_in = nullptr;   // non-null: the teacher probabilities are read here
+  int64_t ld_in = 0;                // ([mp, ld_in]) and `panel` only receives the gradients
   float* loss_part;     // kKlLoss: [n vocabulary tiles, part_ld] loss terms of the tile
   float* tsum_part;     // kKlLoss: [n vocabulary tiles, part_ld] teacher mass of the tile
   float* part_max;      // kKlLoss: [n vocabulary tiles, part_ld] base-2 tile maxima
@@ -700,6 +702,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
     }
   }
   T* panel = static_cast<T*>(p.panel);
+  const T* panel_in = p.panel_in != nullptr ? static_cast<const T*>(p.panel_in) : panel;
+  const int64_t ld_in = p.panel_in != nullptr ? p.ld_in : p.ld;
   const int prow = pv * E::kTile;   // first panel column of this tile
   constexpr bool kCanStage = E::kHasKMajor && sizeof(T) == 2;
 
@@ -744,8 +748,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
       const int tok = c >> 5;
       const int ch = c & 31;
       *reinterpret_cast<uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)) =
-          *reinterpret_cast<const uint4*>(panel + ((int64_t)tt * E::kTile + tok) * p.ld + prow +
-                                          ch * 8);
+          *reinterpret_cast<const uint4*>(panel_in + ((int64_t)tt * E::kTile + tok) * ld_in +
+                                          prow + ch * 8);
     }
     __syncthreads();
 #pragma unroll
@@ -793,11 +797,13 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
 #pragma unroll
     for (int j = 0; j < E::kCols; ++j) {
       T* cell0 = panel + ((int64_t)tt * E::kTile + eng.col(j)) * p.ld + prow;
+      const T* in0 = panel_in + ((int64_t)tt * E::kTile + eng.col(j)) * ld_in + prow;
 #pragma unroll
       for (int i4 = 0; i4 < E::kRows; i4 += 4) {
         T* cell = cell0 + eng.row(i4);
-        const float t[4] = {to_float<T>(cell[0]), to_float<T>(cell[1]), to_float<T>(cell[2]),
-                            to_float<T>(cell[3])};
+        const T* in = in0 + eng.row(i4);
+        const float t[4] = {to_float<T>(in[0]), to_float<T>(in[1]), to_float<T>(in[2]),
+                            to_float<T>(in[3])};
         float g[4];
         process(j, i4, t, g);
         if (grad) store4<T>(cell, g[0], g[1], g[2], g[3]);

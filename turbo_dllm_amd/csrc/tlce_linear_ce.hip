@@ -598,7 +598,8 @@ extern "C" int tlce_kl_forward(const void* draft_hidden, const void* draft_weigh
                                const void* teacher_hidden, const void* teacher_weight, int64_t m,
                                int64_t h_draft, int64_t h_teacher, int64_t v, int dtype,
                                float logit_softcap, float* losses, float* draft_lse,
-                               float* teacher_lse, int64_t panel_bytes, void* workspace,
+                               float* teacher_lse, void* teacher_probabilities,
+                               int64_t panel_bytes, void* workspace,
                                int64_t workspace_bytes, void* stream_) {
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   if (int rc = kl_validate(draft_hidden, draft_weight, teacher_hidden, teacher_weight, m,
@@ -606,6 +607,8 @@ extern "C" int tlce_kl_forward(const void* draft_hidden, const void* draft_weigh
     return rc;
   if (m == 0) return 0;
   TLCE_REQUIRE(losses && draft_lse && teacher_lse && workspace, "kl_forward: null pointer");
+  TLCE_REQUIRE(((uintptr_t)teacher_probabilities & 255) == 0,
+               "kl_forward: teacher_probabilities must be 256-byte aligned");
   const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes);
   TLCE_REQUIRE(workspace_bytes >= k.layout.total, "kl_forward: workspace too small (%lld < %lld)",
                (long long)workspace_bytes, (long long)k.layout.total);
@@ -614,13 +617,22 @@ extern "C" int tlce_kl_forward(const void* draft_hidden, const void* draft_weigh
                 kl_forward_impl<E>(k.draft, k.teacher, k.layout, draft_hidden, draft_weight,
                                    teacher_hidden, teacher_weight, m, h_draft, h_teacher, v, dtype,
                                    logit_softcap, losses, draft_lse, teacher_lse,
-                                   static_cast<char*>(workspace), stream));
+                                   static_cast<char*>(workspace), stream,
+                                   teacher_probabilities));
+}
+
+extern "C" int64_t tlce_kl_teacher_probabilities_bytes(int64_t m, int64_t h_draft,
+                                                       int64_t h_teacher, int64_t v, int dtype) {
+  if (m <= 0 || h_draft <= 0 || h_teacher <= 0 || v <= 0) return 0;
+  const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, 0);
+  return k.draft.mp * k.draft.vp * dtype_bytes(dtype);
 }
 
 extern "C" int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
                                 const void* teacher_hidden, const void* teacher_weight,
                                 const float* draft_lse, const float* teacher_lse,
-                                const float* grad_output, int64_t m, int64_t h_draft,
+                                const float* grad_output,
+                                const void* teacher_probabilities, int64_t m, int64_t h_draft,
                                 int64_t h_teacher, int64_t v, int dtype, float logit_softcap,
                                 void* grad_hidden, int64_t panel_bytes, void* workspace,
                                 int64_t workspace_bytes, void* stream_) {
@@ -640,7 +652,8 @@ extern "C" int tlce_kl_backward(const void* draft_hidden, const void* draft_weig
                 kl_backward_impl<E>(k.draft, k.layout, draft_hidden, draft_weight, teacher_hidden,
                                     teacher_weight, draft_lse, teacher_lse, grad_output, m,
                                     h_draft, h_teacher, v, dtype, logit_softcap, grad_hidden,
-                                    static_cast<char*>(workspace), stream));
+                                    static_cast<char*>(workspace), stream,
+                                    teacher_probabilities));
 }
 
 // ---------------------------------------------------- cross entropy + top-k --

@@ -13,6 +13,10 @@ import torch
 import torch.nn.functional as F
 
 
+# the teacher probabilities kept between forward and backward may take this much
+KEPT_TEACHER_BYTES = 5 << 29
+
+
 class _FrozenLinearKL(torch.autograd.Function):
     """Autograd node around the library's KL forward / backward entry points."""
 
@@ -22,8 +26,24 @@ class _FrozenLinearKL(torch.autograd.Function):
 
         operands = tuple(t.contiguous() for t in (draft_hidden, draft_weight, teacher_hidden,
                                                   teacher_weight))
-        losses, draft_lse, teacher_lse = native.dflash_kl_forward(*operands, float(logit_softcap))
-        ctx.save_for_backward(*operands, draft_lse, teacher_lse)
+        # The teacher probabilities of the whole vocabulary stay in memory until the
+        # backward when they fit the budget of the other kept panels (2.5 GiB: 8192 rows at
+        # V = 151936): the backward then reads them instead of contracting the teacher
+        # head a second time (5 contractions per step instead of 6).
+        from . import options
+        keep = (bool(ctx.needs_input_grad[0]) and options.get_gradient_mode() == "forward"
+                and operands[0].shape[0] > 0
+                and native.kl_teacher_probabilities_bytes(operands[0], operands[1], operands[2])
+                <= KEPT_TEACHER_BYTES)
+        if keep:
+            losses, draft_lse, teacher_lse, kept = native.dflash_kl_forward(
+                *operands, float(logit_softcap), keep_teacher_probabilities=True)
+        else:
+            losses, draft_lse, teacher_lse = native.dflash_kl_forward(*operands,
+                                                                      float(logit_softcap))
+            kept = None
+        ctx.kept = keep
+        ctx.save_for_backward(*operands, draft_lse, teacher_lse, *((kept,) if keep else ()))
         ctx.logit_softcap = float(logit_softcap)
         ctx.panel_bytes = native.get_panel_bytes()   # the backward may run on another thread
         return losses
@@ -32,10 +52,13 @@ class _FrozenLinearKL(torch.autograd.Function):
     def backward(ctx, grad_output):
         from . import chunked_linear_ce_native as native
 
-        *operands, draft_lse, teacher_lse = ctx.saved_tensors
+        saved = list(ctx.saved_tensors)
+        kept = saved.pop() if ctx.kept else None
+        *operands, draft_lse, teacher_lse = saved
         with native.panel_budget(ctx.panel_bytes):
             grad_hidden = native.dflash_kl_backward(*operands, draft_lse, teacher_lse,
-                                                    grad_output.contiguous(), ctx.logit_softcap)
+                                                    grad_output.contiguous(), ctx.logit_softcap,
+                                                    teacher_probabilities=kept)
         return grad_hidden, None, None, None, None
 
 
