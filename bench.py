@@ -379,9 +379,9 @@ def bench_next_objective(args) -> int:
             draft_h.grad = None
             frozen_linear_kl(draft_h, draft_w, teacher_h, teacher_w).sum().backward()
 
-        # 3 forward + 2 backward: the teacher probabilities are kept for the backward
-        # (--gradients recompute: 3 + 3, produced a second time)
-        contractions = 5 if args.gradients == "forward" else 6
+        # teacher statistics, teacher panels, draft pass, and the gradient contraction in
+        # the same forward; the backward scales rows (--gradients recompute: 3 + 3)
+        contractions = 4 if args.gradients == "forward" else 6
         name = "frozen-head KL fwd+bwd"
         shape = f"M={m}, H_draft=H_teacher={h}, V={v}"
     elif args.objective == "ce_topk":

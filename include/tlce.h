@@ -377,6 +377,34 @@ int tlce_kl_forward(const void* draft_hidden, const void* draft_weight,
 int64_t tlce_kl_teacher_probabilities_bytes(int64_t m, int64_t h_draft,
                                             int64_t h_teacher, int64_t v, int dtype);
 
+/* The forward with the gradient formed in it: 4 contractions per forward +
+ * backward.  The draft pass, which holds every draft logit in registers, also
+ * writes exp2(logit2 - the exact maximum of the token's 256-entry vocabulary
+ * tile) <= 1 in bf16 into a second panel over the whole vocabulary beside the
+ * teacher probabilities; once the draft lse is known one elementwise pass forms
+ *   g[r, v] = entry * exp2(tile maximum - lse2_draft[r]) - p_t[r, v]
+ * and one contraction with the draft head leaves
+ *   unit_grad_hidden_f32[r, :] = d losses[r] / d draft_hidden[r, :]   float32 [m, h_draft].
+ * The backward is tlce_apply_grad_output(unit, NULL, NULL, NULL, grad_output, NULL,
+ * m, m, h_draft, v, dtype, TLCE_REDUCTION_NONE, grad_hidden, NULL, stream).
+ * bf16, no soft cap, both hidden sizes and v multiples of 64, all rows in one block
+ * of the 2.5 GiB panel budget (tlce_kl_gradient_in_forward_supported); the workspace
+ * holds both panels (2 x 2 bytes per padded row and vocabulary entry). */
+int tlce_kl_gradient_in_forward_supported(int64_t m, int64_t h_draft,
+                                          int64_t h_teacher, int64_t v, int dtype,
+                                          float logit_softcap);
+
+int64_t tlce_kl_forward_with_gradient_workspace_bytes(int64_t m, int64_t h_draft,
+                                                      int64_t h_teacher, int64_t v,
+                                                      int dtype, int64_t panel_bytes);
+
+int tlce_kl_forward_with_gradient(
+    const void* draft_hidden, const void* draft_weight, const void* teacher_hidden,
+    const void* teacher_weight, int64_t m, int64_t h_draft, int64_t h_teacher,
+    int64_t v, int dtype, float logit_softcap, float* losses, float* draft_lse,
+    float* teacher_lse, float* unit_grad_hidden_f32, int64_t panel_bytes,
+    void* workspace, int64_t workspace_bytes, void* stream);
+
 int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
                      const void* teacher_hidden, const void* teacher_weight,
                      const float* draft_lse, const float* teacher_lse,

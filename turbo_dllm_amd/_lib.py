@@ -232,6 +232,20 @@ SIGNATURES = {
             c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
         ],
     ),
+    "tlce_kl_gradient_in_forward_supported": (
+        c_int, [c_int64, c_int64, c_int64, c_int64, c_int, c_float]),
+    "tlce_kl_forward_with_gradient_workspace_bytes": (
+        c_int64, [c_int64, c_int64, c_int64, c_int64, c_int, c_int64]),
+    "tlce_kl_forward_with_gradient": (
+        c_int,
+        [
+            c_void_p, c_void_p, c_void_p, c_void_p,             # draft h/w, teacher h/w
+            c_int64, c_int64, c_int64, c_int64, c_int,          # m h_draft h_teacher v dtype
+            c_float, c_void_p, c_void_p, c_void_p,              # softcap losses draft_lse teacher_lse
+            c_void_p,                                           # unit_grad_hidden_f32
+            c_int64, c_void_p, c_int64, c_void_p,               # panel_bytes workspace bytes stream
+        ],
+    ),
     "tlce_kl_teacher_probabilities_bytes": (
         c_int64, [c_int64, c_int64, c_int64, c_int64, c_int]),
     "tlce_kl_backward": (

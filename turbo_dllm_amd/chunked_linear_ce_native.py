@@ -1184,6 +1184,56 @@ def dflash_kl_forward(
     return losses, draft_lse, teacher_lse
 
 
+def kl_gradient_in_forward_supported(draft_hidden, draft_weight, teacher_hidden,
+                                     logit_softcap: float) -> bool:
+    """Whether ``dflash_kl_forward_with_gradient`` takes these operands (bf16, no soft
+    cap, hidden sizes and V multiples of 64, all rows in one block of the panel budget)."""
+    if draft_hidden.dtype != torch.bfloat16 or draft_hidden.shape[0] == 0:
+        return False
+    return bool(_lib.library().tlce_kl_gradient_in_forward_supported(
+        draft_hidden.shape[0], draft_hidden.shape[1], teacher_hidden.shape[1],
+        draft_weight.shape[0], _lib.DTYPE_BF16, float(logit_softcap)))
+
+
+def dflash_kl_forward_with_gradient(
+    draft_hidden: torch.Tensor,
+    draft_weight: torch.Tensor,
+    teacher_hidden: torch.Tensor,
+    teacher_weight: torch.Tensor,
+    logit_softcap: float,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(losses, draft_lse, teacher_lse, unit)``: ``dflash_kl_forward`` plus
+    ``d losses / d draft_hidden`` as a float32 ``[N, D]`` tensor formed in the same
+    forward (4 contractions per step); the backward multiplies row ``r`` by its
+    upstream gradient (``apply_grad_output(..., reduction="none")``)."""
+    device, dh, dw, th, tw = _kl_operands(draft_hidden, draft_weight, teacher_hidden,
+                                          teacher_weight)
+    m, hd = dh.shape
+    ht, v = th.shape[1], dw.shape[0]
+    code = _dtype_code(dh)
+    lib = _lib.library()
+    with torch.cuda.device(device):
+        losses = torch.empty(m, dtype=torch.float32, device=device)
+        draft_lse = torch.empty(m, dtype=torch.float32, device=device)
+        teacher_lse = torch.empty(m, dtype=torch.float32, device=device)
+        unit = torch.empty((m, hd), dtype=torch.float32, device=device)
+        nbytes = lib.tlce_kl_forward_with_gradient_workspace_bytes(m, hd, ht, v, code,
+                                                                    get_panel_bytes())
+        if nbytes < 0:
+            raise RuntimeError("the KL forward that leaves the gradient does not take these "
+                               "operands (kl_gradient_in_forward_supported)")
+        ws = _workspace(nbytes, device)
+        _lib.check(
+            lib.tlce_kl_forward_with_gradient(
+                _ptr(dh), _ptr(dw), _ptr(th), _ptr(tw), m, hd, ht, v, code,
+                float(logit_softcap), _ptr(losses), _ptr(draft_lse), _ptr(teacher_lse),
+                _ptr(unit), get_panel_bytes(), ws.data_ptr(), ws.numel(), _stream(device),
+            ),
+            "tlce_kl_forward_with_gradient",
+        )
+    return losses, draft_lse, teacher_lse, unit
+
+
 def kl_teacher_probabilities_bytes(draft_hidden, draft_weight, teacher_hidden) -> int:
     """Size of the buffer ``dflash_kl_forward(keep_teacher_probabilities=True)`` fills."""
     m, hd = draft_hidden.shape

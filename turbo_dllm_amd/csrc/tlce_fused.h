@@ -751,7 +751,109 @@ int topk_forward_with_gradient_impl(const TopkPlan& t, const FusedPlan& p, const
   return launch_reduce_slabs(rs, stream);
 }
 
+// ---- frozen-head KL: the gradient formed in the forward (4 contractions, not 6) ----
+// The draft pass of the forward already holds every draft logit in registers.  In its
+// emitting variant (lce_kl_panel_kernel<.., kEmit>) it also writes exp2(z2 - tile
+// maximum) <= 1 of every entry in bf16 into a second panel over the whole vocabulary,
+// beside the teacher probabilities.  When the pass is over the draft lse is known,
+// one elementwise pass turns the two panels into the logit gradient
+//   g[r, v] = e[r, v] * exp2(part_max[tile(v), r] - lse2_draft[r]) - t[r, v]
+// (lce_kl_grad_from_exp_kernel), and one contraction with the draft head leaves
+//   unit[r, :] = d loss[r] / d draft_hidden[r, :]       float32 [m, h].
+// The backward multiplies row r by its upstream gradient and rounds once.  No soft cap
+// (its derivative would have to be re-derived from the rounded entries).
+struct KlGradFromExpArgs {
+  void* exp_panel;           // bf16 [mp, ld]: e in, logit gradient out
+  const void* teacher;       // bf16 [mp, ld] teacher probabilities
+  int64_t ld;
+  int m, mp;
+  const float* part_max;     // [n_vtiles, part_ld] base-2 tile maxima
+  int part_ld;
+  const float* draft_lse;    // [m] natural units
+};
+int launch_kl_grad_from_exp(const KlGradFromExpArgs& a, int n_vtiles, hipStream_t stream);
+
+struct KlFusedLayout {
+  int64_t kl, teacher, exp_panel, slabs, total;
+};
+
+template <class E>
+int launch_kl_panel_emit(const KlPanelArgs& a, hipStream_t stream) {
+  static LdsOptIn lds;
+  constexpr int kLdsBytes = E::kSmemBytes + E::kShare * E::kTile * (int)sizeof(float);
+  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, false, false, true>, kLdsBytes, lds))
+    return rc;
+  const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
+  ScopedTimer timer(kClassGradLogits, stream);
+  lce_kl_panel_kernel<E, false, false, true><<<grid, E::kThreads, kLdsBytes, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
+inline bool kl_gradient_in_forward_supported(int64_t m, int64_t hd, int64_t ht, int64_t v,
+                                             int dtype, float softcap) {
+  return softcap <= 0.0f && fused_gradients_supported(hd, v, dtype) &&
+         engine_class(ht, dtype) == 2 && make_fused_plan(m, hd, v, dtype, 0).n_blocks == 1;
+}
+
+inline KlFusedLayout kl_fused_layout(const KlLayout& kl, const Plan& pd, const FusedPlan& p,
+                                     int64_t hd) {
+  KlFusedLayout l;
+  int64_t off = 0;
+  l.kl = off;         off += align256(kl.total);
+  l.teacher = off;    off += align256(pd.mp * pd.vp * 2);
+  l.exp_panel = off;  off += align256(pd.mp * pd.vp * 2);
+  l.slabs = off;      off += align256((int64_t)p.dh_ksplit * pd.mp * hd * 4);
+  l.total = off;
+  return l;
+}
+
+template <class E>
+int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout& kl,
+                                  const FusedPlan& fp, const void* draft_hidden,
+                                  const void* draft_weight, const void* teacher_hidden,
+                                  const void* teacher_weight, int64_t m, int64_t hd, int64_t ht,
+                                  int64_t v, int dtype, float* losses, float* draft_lse,
+                                  float* teacher_lse, float* unit_grad, char* ws,
+                                  hipStream_t stream) {
+  using T = typename E::T;
+  const KlFusedLayout l = kl_fused_layout(kl, pd, fp, hd);
+  char* kws = ws + l.kl;
+  T* teacher = reinterpret_cast<T*>(ws + l.teacher);
+  T* exp_panel = reinterpret_cast<T*>(ws + l.exp_panel);
+  float* slabs = reinterpret_cast<float*>(ws + l.slabs);
+  // the forward as ever, its teacher panels going to `teacher` and its draft pass
+  // leaving exp2(z2 - tile maximum) in `exp_panel`
+  if (int rc = kl_forward_impl<E>(pd, pt, kl, draft_hidden, draft_weight, teacher_hidden,
+                                  teacher_weight, m, hd, ht, v, dtype, 0.0f, losses, draft_lse,
+                                  teacher_lse, kws, stream, teacher, exp_panel))
+    return rc;
+  const float* part_max = reinterpret_cast<const float*>(kws + kl.stats);
+  KlGradFromExpArgs ga;
+  ga.exp_panel = exp_panel; ga.teacher = teacher; ga.ld = pd.vp;
+  ga.m = (int)m; ga.mp = (int)pd.mp;
+  ga.part_max = part_max; ga.part_ld = (int)pd.mp; ga.draft_lse = draft_lse;
+  if (int rc = launch_kl_grad_from_exp(ga, pd.n_vtiles, stream)) return rc;
+
+  const float* ones = reinterpret_cast<const float*>(kws + kl.ones);
+  GemmArgs g;
+  g.a = draft_weight; g.lda = hd; g.a_rows = (int)hd;
+  g.b = exp_panel; g.ldb = pd.vp; g.b_rows = (int)pd.mp;
+  g.k = (int)round_up(v, 64); g.k_per_split = 0;
+  g.ni = fp.n_htiles; g.nj = (int)(pd.mp / E::kTile);
+  g.c = slabs; g.ldc = hd; g.c_rows = (int)pd.mp; g.c_cols = (int)hd;
+  g.c_split_stride = pd.mp * hd;
+  g.mode = kStoreF32;
+  if (int rc = launch_gemm<E, true, false>(g, fp.dh_ksplit, kClassGradHidden, stream)) return rc;
+  ReduceSlabsArgs rs;
+  rs.slabs = slabs; rs.n_splits = fp.dh_ksplit; rs.split_stride = pd.mp * hd;
+  rs.row_scale = ones; rs.m = (int)m; rs.h = (int)hd;
+  rs.out = unit_grad;
+  return launch_reduce_slabs(rs, stream);
+}
+
 #define TLCE_LAUNCHERS_EXP_PANEL(X, E)                                                  \
+  X int launch_kl_panel_emit<E>(const KlPanelArgs&, hipStream_t);                       \
   X int launch_exp_panel_variant<E, false, false>(const ExpPanelArgs&, hipStream_t);    \
   X int launch_exp_panel_variant<E, true, false>(const ExpPanelArgs&, hipStream_t);     \
   X int launch_exp_panel_variant<E, true, true>(const ExpPanelArgs&, hipStream_t);
@@ -767,6 +869,11 @@ int topk_forward_with_gradient_impl(const TopkPlan& t, const FusedPlan& p, const
                                            const void*, const int64_t*, int64_t, int64_t,        \
                                            int64_t, int, float, float, float*, float*, float*,   \
                                            int64_t*, float*, float*, char*, hipStream_t);        \
+  X int kl_forward_with_gradient_impl<E>(const Plan&, const Plan&, const KlLayout&,              \
+                                         const FusedPlan&, const void*, const void*,             \
+                                         const void*, const void*, int64_t, int64_t, int64_t,    \
+                                         int64_t, int, float*, float*, float*, float*, char*,    \
+                                         hipStream_t);                                           \
   X int deferred_grad_weight_impl<E>(const FusedPlan&, const void*, int64_t, int64_t, int64_t,   \
                                      int, const float*, const float*, int, const int64_t*,       \
                                      const int64_t*, void*, char*, hipStream_t);

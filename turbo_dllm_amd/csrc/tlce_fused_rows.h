@@ -199,6 +199,34 @@ __global__ __launch_bounds__(256) void lce_reduce_scaled_slabs_kernel(ReduceSlab
   }
 }
 
+// blockIdx.x = row, blockIdx.y = a group of 8 vocabulary tiles: 32 threads per tile, 8
+// columns each.  The logit gradient of the frozen-head KL from the two panels the
+// forward left (rows from m on get zeros).
+__global__ __launch_bounds__(256) void lce_kl_grad_from_exp_kernel(KlGradFromExpArgs p,
+                                                                   int n_vtiles) {
+  const int r = blockIdx.x;
+  const int tile = blockIdx.y * 8 + (threadIdx.x >> 5);
+  if (tile >= n_vtiles) return;
+  const int64_t c = (int64_t)tile * 256 + (threadIdx.x & 31) * 8;
+  __bf16* e = static_cast<__bf16*>(p.exp_panel) + (int64_t)r * p.ld + c;
+  typedef __bf16 v8_t __attribute__((ext_vector_type(8)));
+  v8_t out;
+  if (r < p.m) {
+    const float f = exp2f(p.part_max[(int64_t)tile * p.part_ld + r] -
+                          p.draft_lse[r] * TLCE_LOG2E);
+    const v8_t ev = *reinterpret_cast<const v8_t*>(e);
+    const v8_t tv = *reinterpret_cast<const v8_t*>(static_cast<const __bf16*>(p.teacher) +
+                                                   (int64_t)r * p.ld + c);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      out[i] = from_float<__bf16>(to_float<__bf16>(ev[i]) * f - to_float<__bf16>(tv[i]));
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = from_float<__bf16>(0.0f);
+  }
+  *reinterpret_cast<v8_t*>(e) = out;
+}
+
 // One row and 2048 columns per workgroup, 8 columns per thread.
 __global__ __launch_bounds__(256) void lce_exp_from_logits_kernel(ExpFromLogitsArgs p) {
   const int r = blockIdx.x;

@@ -629,6 +629,14 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 //   mode kKlGrad: panel[token, v] = (exp(lp) - t) * scale[token] * cap'(z_draft)
 //                 in place, rounded to the input dtype: the logit gradient that
 //                 feeds the grad-hidden contraction.
+//   kEmit (with kKlLoss): additionally panel[token, v] = exp2(z2 - tile maximum of
+//                 the token) rounded to the input dtype, the teacher tile being
+//                 read from panel_in.  The tile maximum (part_max) is the exact
+//                 maximum over the tile's 256 vocabulary rows, found through LDS
+//                 before the exponentials, so every entry is <= 1; once the draft
+//                 lse is known, softmax = entry * exp2(part_max - lse2) per
+//                 (token, tile): the logit gradient can be formed from the two
+//                 panels without contracting the draft head again.
 enum { kKlLoss = 0, kKlGrad = 1 };
 
 struct KlPanelArgs {
@@ -652,8 +660,9 @@ struct KlPanelArgs {
   int mode;
 };
 
-template <class E, bool kSoftcap, bool kGrad>
+template <class E, bool kSoftcap, bool kGrad, bool kEmit = false>
 __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p) {
+  static_assert(!(kGrad && kEmit), "kEmit belongs to the loss mode");
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
   const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
@@ -700,6 +709,22 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
         tile_max[j] = fmaxf(tile_max[j], z);
       }
     }
+    if constexpr (kEmit) {
+      // the maximum over all of the tile's vocabulary rows per token, through the LDS
+      // beyond the engine's stages (the launch allocates it), before any exponential
+      float* all_max = reinterpret_cast<float*>(smem + E::kSmemBytes);
+      const int slot = eng.share_slot();
+#pragma unroll
+      for (int j = 0; j < E::kCols; ++j) all_max[slot * E::kTile + eng.col(j)] = tile_max[j];
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < E::kCols; ++j) {
+        float mx = all_max[eng.col(j)];
+#pragma unroll
+        for (int sl = 1; sl < E::kShare; ++sl) mx = fmaxf(mx, all_max[sl * E::kTile + eng.col(j)]);
+        tile_max[j] = mx;
+      }
+    }
   }
   T* panel = static_cast<T*>(p.panel);
   const T* panel_in = p.panel_in != nullptr ? static_cast<const T*>(p.panel_in) : panel;
@@ -731,6 +756,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
         const float tv = t[u];
         const float e = exp2_of<E::kPrecise>(z - tile_max[j]);
         tile_sum[j] += vok ? e : 0.0f;
+        if (kEmit) g[u] = (vok && tile_max[j] > -INFINITY) ? e : 0.0f;
         const bool use = vok && tv > 0.0f;
         const float term = tv * ((log2_of<E::kPrecise>(tv) - z) * TLCE_LN2) - tv;
         partial[j] += use ? term : 0.0f;
@@ -766,9 +792,9 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
                             to_float<T>(tv[3])};
         float g[4];
         process(j, i4, t, g);
-        if (grad) store4<T>(cell, g[0], g[1], g[2], g[3]);
+        if (grad || kEmit) store4<T>(cell, g[0], g[1], g[2], g[3]);
       }
-      if (grad) {
+      if (grad || kEmit) {
         // the tokens with owned index j are complete: their rows go out while
         // the next quarter of the tile is being processed
         __syncthreads();
@@ -806,7 +832,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
                             to_float<T>(in[3])};
         float g[4];
         process(j, i4, t, g);
-        if (grad) store4<T>(cell, g[0], g[1], g[2], g[3]);
+        if (grad || kEmit) store4<T>(cell, g[0], g[1], g[2], g[3]);
       }
     }
   }

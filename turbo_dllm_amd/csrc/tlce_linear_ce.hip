@@ -89,6 +89,14 @@ int launch_scale_rows(const ScaleRowsArgs& a, hipStream_t stream) {
   return 0;
 }
 
+int launch_kl_grad_from_exp(const KlGradFromExpArgs& a, int n_vtiles, hipStream_t stream) {
+  ScopedTimer timer(kClassOther, stream);
+  lce_kl_grad_from_exp_kernel<<<dim3((unsigned)a.mp, (unsigned)ceil_div(n_vtiles, 8)), 256, 0,
+                                stream>>>(a, n_vtiles);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
 int launch_exp_from_logits(const ExpFromLogitsArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassOther, stream);
   lce_exp_from_logits_kernel<<<dim3((unsigned)a.m_pad, (unsigned)ceil_div(a.width, 2048)), 256, 0,
@@ -626,6 +634,55 @@ extern "C" int64_t tlce_kl_teacher_probabilities_bytes(int64_t m, int64_t h_draf
   if (m <= 0 || h_draft <= 0 || h_teacher <= 0 || v <= 0) return 0;
   const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, 0);
   return k.draft.mp * k.draft.vp * dtype_bytes(dtype);
+}
+
+extern "C" int tlce_kl_gradient_in_forward_supported(int64_t m, int64_t h_draft,
+                                                     int64_t h_teacher, int64_t v, int dtype,
+                                                     float logit_softcap) {
+  if (m <= 0 || h_draft <= 0 || h_teacher <= 0 || v <= 0) return 0;
+  return kl_gradient_in_forward_supported(m, h_draft, h_teacher, v, dtype, logit_softcap) ? 1 : 0;
+}
+
+extern "C" int64_t tlce_kl_forward_with_gradient_workspace_bytes(int64_t m, int64_t h_draft,
+                                                                 int64_t h_teacher, int64_t v,
+                                                                 int dtype, int64_t panel_bytes) {
+  if (!tlce_kl_gradient_in_forward_supported(m, h_draft, h_teacher, v, dtype, 0.0f)) return -1;
+  const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes);
+  return kl_fused_layout(k.layout, k.draft, make_fused_plan(m, h_draft, v, dtype, 0), h_draft)
+      .total;
+}
+
+extern "C" int tlce_kl_forward_with_gradient(
+    const void* draft_hidden, const void* draft_weight, const void* teacher_hidden,
+    const void* teacher_weight, int64_t m, int64_t h_draft, int64_t h_teacher, int64_t v,
+    int dtype, float logit_softcap, float* losses, float* draft_lse, float* teacher_lse,
+    float* unit_grad_hidden_f32, int64_t panel_bytes, void* workspace, int64_t workspace_bytes,
+    void* stream_) {
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  if (int rc = kl_validate(draft_hidden, draft_weight, teacher_hidden, teacher_weight, m,
+                           h_draft, h_teacher, v, dtype))
+    return rc;
+  if (m == 0) return 0;
+  TLCE_REQUIRE(kl_gradient_in_forward_supported(m, h_draft, h_teacher, v, dtype, logit_softcap),
+               "kl_forward_with_gradient: needs bf16 inputs, no soft cap, both hidden sizes and v "
+               "multiples of 64, and all rows in one block of the panel budget (m=%lld, v=%lld)",
+               (long long)m, (long long)v);
+  TLCE_REQUIRE(losses && draft_lse && teacher_lse && unit_grad_hidden_f32 && workspace,
+               "kl_forward_with_gradient: null pointer");
+  TLCE_REQUIRE(((uintptr_t)unit_grad_hidden_f32 & 15) == 0,
+               "kl_forward_with_gradient: the gradient buffer must be 16-byte aligned");
+  const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes);
+  const FusedPlan fp = make_fused_plan(m, h_draft, v, dtype, 0);
+  const int64_t need = kl_fused_layout(k.layout, k.draft, fp, h_draft).total;
+  TLCE_REQUIRE(workspace_bytes >= need,
+               "kl_forward_with_gradient: workspace too small (%lld < %lld)",
+               (long long)workspace_bytes, (long long)need);
+  TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
+               "kl_forward_with_gradient: workspace must be 256-byte aligned");
+  return kl_forward_with_gradient_impl<MfmaDirect4Engine<__bf16>>(
+      k.draft, k.teacher, k.layout, fp, draft_hidden, draft_weight, teacher_hidden,
+      teacher_weight, m, h_draft, h_teacher, v, dtype, losses, draft_lse, teacher_lse,
+      unit_grad_hidden_f32, static_cast<char*>(workspace), stream);
 }
 
 extern "C" int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,

@@ -26,13 +26,27 @@ class _FrozenLinearKL(torch.autograd.Function):
 
         operands = tuple(t.contiguous() for t in (draft_hidden, draft_weight, teacher_hidden,
                                                   teacher_weight))
-        # The teacher probabilities of the whole vocabulary stay in memory until the
-        # backward when they fit the budget of the other kept panels (2.5 GiB: 8192 rows at
-        # V = 151936): the backward then reads them instead of contracting the teacher
-        # head a second time (5 contractions per step instead of 6).
         from . import options
-        keep = (bool(ctx.needs_input_grad[0]) and options.get_gradient_mode() == "forward"
-                and operands[0].shape[0] > 0
+        wants = (bool(ctx.needs_input_grad[0]) and options.get_gradient_mode() == "forward"
+                 and operands[0].shape[0] > 0)
+        # bf16 without a soft cap, all rows in one block of the panel budget: the draft
+        # pass of the forward leaves what the logit gradient needs, and one contraction
+        # more in the forward leaves d loss / d draft_hidden (4 contractions per step);
+        # the backward only multiplies each row by its upstream gradient
+        ctx.fused = wants and native.kl_gradient_in_forward_supported(
+            operands[0], operands[1], operands[2], float(logit_softcap))
+        if ctx.fused:
+            losses, _, _, unit = native.dflash_kl_forward_with_gradient(*operands,
+                                                                        float(logit_softcap))
+            ctx.kept = False
+            ctx.save_for_backward(unit)
+            ctx.grad_dtype = operands[0].dtype
+            return losses
+        # Otherwise the teacher probabilities of the whole vocabulary stay in memory until
+        # the backward when they fit the budget of the other kept panels (2.5 GiB: 8192 rows
+        # at V = 151936): the backward then reads them instead of contracting the teacher
+        # head a second time (5 contractions per step instead of 6).
+        keep = (wants
                 and native.kl_teacher_probabilities_bytes(operands[0], operands[1], operands[2])
                 <= KEPT_TEACHER_BYTES)
         if keep:
@@ -52,6 +66,12 @@ class _FrozenLinearKL(torch.autograd.Function):
     def backward(ctx, grad_output):
         from . import chunked_linear_ce_native as native
 
+        if ctx.fused:
+            (unit,) = ctx.saved_tensors
+            grad_hidden, _ = native.apply_grad_output(
+                unit, None, grad_output.contiguous(), None, reduction="none",
+                dtype=ctx.grad_dtype)
+            return grad_hidden, None, None, None, None
         saved = list(ctx.saved_tensors)
         kept = saved.pop() if ctx.kept else None
         *operands, draft_lse, teacher_lse = saved
