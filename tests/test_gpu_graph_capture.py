@@ -242,3 +242,87 @@ def test_gradients_formed_in_the_forward_graph_replays_match_eager(gpu_device, n
         for name, a, b in zip(("losses", "grad_hidden", "grad_weight"), got, eager):
             assert torch.equal(a, b), (replay, name)
         assert torch.isfinite(got[0]).all() and torch.isfinite(got[1].float()).all()
+
+
+def _replay_against_eager(dev, run, make, static, names, replays=4):
+    """Captures run(*static) once, then replays it for fresh inputs with eager work and
+    synchronisations in between; every replay must equal the eager result bit for bit."""
+    first = make()
+    for s, t in zip(static, first):
+        s.copy_(t)
+    run(*static)                                  # warm-up: one-time kernel attributes
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outputs = run(*static)
+    torch.cuda.synchronize()
+    for replay in range(replays):
+        case = first if replay == 0 else make()
+        for s, t in zip(static, case):
+            s.copy_(t)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outputs]
+        eager = run(*[t.to(dev) for t in case])   # eager work between replays
+        torch.cuda.synchronize()
+        for name, a, b in zip(names, got, eager):
+            assert torch.equal(a, b), (replay, name)
+
+
+def test_frozen_kl_gradient_in_the_forward_graph_replays_match_eager(gpu_device, set_panel_budget):
+    """The KL forward that leaves d loss / d hidden, and the row scaling that is its
+    backward, from one graph (kernels and device-to-device work only)."""
+    print("[case] KL gradient-in-forward graph capture", flush=True)
+    dev = gpu_device
+    n, hd, ht, v = 300, 128, 64, 1536
+    set_panel_budget(512 * 512 * 2)
+    gen = torch.Generator().manual_seed(5)
+    draft_w = (torch.randn(v, hd, generator=gen) * 0.2).bfloat16().to(dev)
+    teacher_w = (torch.randn(v, ht, generator=gen) * 0.2).bfloat16().to(dev)
+
+    def make():
+        return (torch.randn(n, hd, generator=gen).bfloat16(),
+                torch.randn(n, ht, generator=gen).bfloat16(),
+                torch.rand(n, generator=gen) + 0.5)
+
+    def run(draft_h, teacher_h, go):
+        losses, _, _, unit = native.dflash_kl_forward_with_gradient(draft_h, draft_w, teacher_h,
+                                                                    teacher_w, 0.0)
+        grad, _ = native.apply_grad_output(unit, None, go, None, reduction="none",
+                                           dtype=torch.bfloat16)
+        return losses, grad
+
+    static = [torch.zeros(n, hd, dtype=torch.bfloat16, device=dev),
+              torch.zeros(n, ht, dtype=torch.bfloat16, device=dev),
+              torch.zeros(n, dtype=torch.float32, device=dev)]
+    _replay_against_eager(dev, run, make, static, ("losses", "grad_hidden"))
+
+
+def test_ce_topk_gradient_in_the_forward_graph_replays_match_eager(gpu_device, set_panel_budget):
+    """Frozen-head cross entropy with top-k, d lse / d hidden formed in the forward over
+    several float32 logits panels (with the rescaling of panels written before a row's
+    maximum grew), and the row pass that is its backward, from one graph."""
+    print("[case] CE top-k gradient-in-forward graph capture", flush=True)
+    dev = gpu_device
+    n, h, v, k = 260, 128, 4096, 8
+    set_panel_budget(512 * 1024 * 4)
+    gen = torch.Generator().manual_seed(6)
+    weight = (torch.randn(v, h, generator=gen) * 0.5).bfloat16().to(dev)
+
+    def make():
+        return (torch.randn(n, h, generator=gen).bfloat16(),
+                torch.randint(0, v, (n,), generator=gen),
+                torch.randn(n, generator=gen), torch.randn(n, generator=gen),
+                torch.randn(n, k, generator=gen))
+
+    def run(hidden, labels, gl, gp, gv):
+        loss, prob, vals, ids, _, unit = native.dflash_ce_topk_forward_with_gradient(
+            hidden, weight, labels, top_k=k, output_multiplier=0.8, logit_softcap=0.0)
+        grad = native.dflash_ce_topk_apply_gradient(unit, hidden, weight, labels, prob, ids, gl, gp,
+                                                    gv, output_multiplier=0.8, logit_softcap=0.0)
+        return loss, vals, ids, grad
+
+    static = [torch.zeros(n, h, dtype=torch.bfloat16, device=dev),
+              torch.zeros(n, dtype=torch.long, device=dev),
+              torch.zeros(n, device=dev), torch.zeros(n, device=dev), torch.zeros(n, k, device=dev)]
+    _replay_against_eager(dev, run, make, static, ("loss", "top_values", "top_ids", "grad_hidden"))
