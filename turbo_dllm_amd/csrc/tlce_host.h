@@ -742,9 +742,13 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
   // softmax partials (the teacher partials above are dead by now)
   const BackwardLayout bl = backward_layout(pd, m, hd, dtype, false);
   void* g = ws + l.backward + bl.g;
-  for (int panel = 0; panel < pd.n_panels; ++panel) {
-    const int64_t v0 = (int64_t)panel * pd.vc;
-    const int64_t width = std::min<int64_t>(pd.vc, pd.vp - v0);
+  // teacher probabilities that go to a buffer over the whole vocabulary need no bounded
+  // panel: one launch of each kernel covers all of it (fewer partly filled last rounds)
+  const int n_panels = kept_teacher != nullptr ? 1 : pd.n_panels;
+  const int64_t panel_width = kept_teacher != nullptr ? pd.vp : pd.vc;
+  for (int panel = 0; panel < n_panels; ++panel) {
+    const int64_t v0 = (int64_t)panel * panel_width;
+    const int64_t width = std::min<int64_t>(panel_width, pd.vp - v0);
     if (int rc = kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight,
                              nullptr, teacher_lse, ones, nullptr, m, hd, ht, v, softcap, v0,
                              width, g, loss_part, tsum_part, part_max, part_sum, kKlLoss,
