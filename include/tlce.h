@@ -387,9 +387,10 @@ int64_t tlce_kl_teacher_probabilities_bytes(int64_t m, int64_t h_draft,
  *   unit_grad_hidden_f32[r, :] = d losses[r] / d draft_hidden[r, :]   float32 [m, h_draft].
  * The backward is tlce_apply_grad_output(unit, NULL, NULL, NULL, grad_output, NULL,
  * m, m, h_draft, v, dtype, TLCE_REDUCTION_NONE, grad_hidden, NULL, stream).
- * bf16, no soft cap, both hidden sizes and v multiples of 64, all rows in one block
- * of the 2.5 GiB panel budget (tlce_kl_gradient_in_forward_supported); the workspace
- * holds both panels (2 x 2 bytes per padded row and vocabulary entry). */
+ * bf16, no soft cap, both hidden sizes and v multiples of 64
+ * (tlce_kl_gradient_in_forward_supported); rows are taken in blocks of the 2.5 GiB
+ * panel budget one after the other, and the workspace holds both panels of a block
+ * (2 x 2 bytes per padded row and vocabulary entry). */
 int tlce_kl_gradient_in_forward_supported(int64_t m, int64_t h_draft,
                                           int64_t h_teacher, int64_t v, int dtype,
                                           float logit_softcap);
@@ -468,9 +469,10 @@ int tlce_ce_topk_backward(const void* hidden, const void* weight,
  *                       - ce_scale[r] * dz/draw[label] * weight[label]
  *                       + sum_j grad_top_values[r,j] * dz/draw[id_j] * weight[id_j]
  * rounded once: 2 contractions per step instead of 3.  bf16, h and v multiples
- * of 64, and all rows in one block of the 2.5 GiB panel budget (8192 rows at
- * v = 151936): tlce_ce_topk_gradient_in_forward_supported; panel_bytes bounds
- * the float32 logits panels as in tlce_ce_topk_forward. */
+ * of 64 (tlce_ce_topk_gradient_in_forward_supported); rows are taken in blocks
+ * of the 2.5 GiB panel budget (8192 rows at v = 151936), one after the other on
+ * one workspace; panel_bytes bounds the float32 logits panels as in
+ * tlce_ce_topk_forward. */
 int tlce_ce_topk_gradient_in_forward_supported(int64_t m, int64_t h, int64_t v,
                                                int dtype);
 

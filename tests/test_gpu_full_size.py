@@ -447,3 +447,44 @@ def test_small_head_full_size_against_the_dense_oracle(gpu_device):
     err_w = oracle.relative_max_error(weight.grad.cpu(), rdw)
     say(f"loss rel {rel:.2e} dH {err_h:.2e} dW {err_w:.2e}")
     assert rel <= 1e-3 and err_h <= 2e-2 and err_w <= 2e-2
+
+
+def test_row_blocks_of_the_objectives_whose_gradient_is_formed_in_the_forward(gpu_device):
+    """12000 rows at V = 151936 exceed one block of the panel budget (8192 rows): the KL
+    and the cross entropy with top-k take them as two blocks, each a call of its own on a
+    part of every per-row buffer.  Rows are independent, so the result equals, bit for
+    bit, the two parts run on their own (which the smaller tests hold to the oracle)."""
+    from turbo_dllm_amd import _lib
+    from turbo_dllm_amd.dflash_kl import frozen_linear_kl
+    from turbo_dllm_amd.dflash_linear_topk import frozen_linear_ce_topk
+    dev = gpu_device
+    m, h, v, k = 12000, 256, 151936, 4
+    block = _lib.query_fused_plan(m, h, v, _lib.DTYPE_BF16, 0)["block_rows"]
+    say("row blocks", m, "rows in blocks of", block)
+    assert 0 < block < m
+    gen = torch.Generator().manual_seed(12)
+    draft_h, teacher_h = _randn(gen, m, h, 1.0, dev), _randn(gen, m, h, 1.0, dev)
+    draft_w, teacher_w = _randn(gen, v, h, 0.05, dev), _randn(gen, v, h, 0.05, dev)
+    labels = torch.randint(0, v, (m,), generator=gen).to(dev)
+    go = (torch.rand(m, generator=gen) + 0.5).to(dev)
+
+    def kl(rows):
+        x = draft_h[rows].clone().requires_grad_(True)
+        loss = frozen_linear_kl(x, draft_w, teacher_h[rows], teacher_w)
+        loss.backward(go[rows])
+        return loss.detach(), x.grad
+
+    def topk(rows):
+        x = draft_h[rows].clone().requires_grad_(True)
+        loss, prob, vals, ids = frozen_linear_ce_topk(x, draft_w, labels[rows], top_k=k)
+        (loss * go[rows]).sum().backward()
+        return loss.detach(), vals.detach(), ids, x.grad
+
+    for name, fn in (("KL", kl), ("CE top-k", topk)):
+        whole = fn(slice(0, m))
+        parts = [fn(slice(0, block)), fn(slice(block, m))]
+        torch.cuda.synchronize()
+        for i, out in enumerate(whole):
+            assert bool(torch.isfinite(out.float()).all()) if out.is_floating_point() else True
+            assert torch.equal(out, torch.cat([parts[0][i], parts[1][i]])), (name, i)
+        say(name, "two blocks equal the parts run alone")

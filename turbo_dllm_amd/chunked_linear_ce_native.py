@@ -1187,7 +1187,7 @@ def dflash_kl_forward(
 def kl_gradient_in_forward_supported(draft_hidden, draft_weight, teacher_hidden,
                                      logit_softcap: float) -> bool:
     """Whether ``dflash_kl_forward_with_gradient`` takes these operands (bf16, no soft
-    cap, hidden sizes and V multiples of 64, all rows in one block of the panel budget)."""
+    cap, hidden sizes and V multiples of 64; rows go in blocks of the panel budget)."""
     if draft_hidden.dtype != torch.bfloat16 or draft_hidden.shape[0] == 0:
         return False
     return bool(_lib.library().tlce_kl_gradient_in_forward_supported(
@@ -1343,8 +1343,8 @@ def dflash_ce_topk_forward(
 
 def ce_topk_gradient_in_forward_supported(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether ``dflash_ce_topk_forward_with_gradient`` takes these operands: bf16,
-    H and V multiples of 64, and all rows in one block of the panel of exponentiated
-    logits (2.5 GiB over the whole vocabulary: 8192 rows at V = 151936)."""
+    H and V multiples of 64 (rows are taken in blocks of the panel of exponentiated
+    logits, 2.5 GiB over the whole vocabulary: 8192 rows at V = 151936)."""
     if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or hidden.shape[0] == 0:
         return False
     return bool(_lib.library().tlce_ce_topk_gradient_in_forward_supported(

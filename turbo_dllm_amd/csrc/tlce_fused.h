@@ -681,11 +681,17 @@ struct TopkFusedLayout {
   int64_t forward, panel, ref_used, row_scale, slabs, total;
 };
 
-// All rows must form one block of the panel budget of the forward that leaves the
-// gradients (its default: panel_bytes bounds the float32 logits panels here).
+// Rows are taken in blocks of the panel budget of the forward that leaves the gradients
+// (its default; panel_bytes bounds the float32 logits panels here): rows are independent,
+// so a block is a call of its own on a part of every per-row buffer.
 inline bool topk_gradient_in_forward_supported(int64_t m, int64_t h, int64_t v, int dtype) {
-  return fused_gradients_supported(h, v, dtype) &&
-         make_fused_plan(m, h, v, dtype, 0).n_blocks == 1;
+  (void)m;
+  return fused_gradients_supported(h, v, dtype);
+}
+
+// Rows per block of the objectives that take whole blocks of rows one after the other.
+inline int64_t fused_row_block(int64_t m, int64_t h, int64_t v, int dtype) {
+  return make_fused_plan(m, h, v, dtype, 0).block_rows;
 }
 
 inline TopkFusedLayout topk_fused_layout(const TopkPlan& t, const FusedPlan& p, int64_t h) {
@@ -792,8 +798,9 @@ int launch_kl_panel_emit(const KlPanelArgs& a, hipStream_t stream) {
 
 inline bool kl_gradient_in_forward_supported(int64_t m, int64_t hd, int64_t ht, int64_t v,
                                              int dtype, float softcap) {
+  (void)m;   // rows beyond one block of the panel budget are taken block by block
   return softcap <= 0.0f && fused_gradients_supported(hd, v, dtype) &&
-         engine_class(ht, dtype) == 2 && make_fused_plan(m, hd, v, dtype, 0).n_blocks == 1;
+         engine_class(ht, dtype) == 2;
 }
 
 inline KlFusedLayout kl_fused_layout(const KlLayout& kl, const Plan& pd, const FusedPlan& p,

@@ -647,8 +647,9 @@ extern "C" int64_t tlce_kl_forward_with_gradient_workspace_bytes(int64_t m, int6
                                                                  int64_t h_teacher, int64_t v,
                                                                  int dtype, int64_t panel_bytes) {
   if (!tlce_kl_gradient_in_forward_supported(m, h_draft, h_teacher, v, dtype, 0.0f)) return -1;
-  const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes);
-  return kl_fused_layout(k.layout, k.draft, make_fused_plan(m, h_draft, v, dtype, 0), h_draft)
+  const int64_t rows = std::min(m, fused_row_block(m, h_draft, v, dtype));   // the largest block
+  const KlPlans k = kl_plans(rows, h_draft, h_teacher, v, dtype, panel_bytes);
+  return kl_fused_layout(k.layout, k.draft, make_fused_plan(rows, h_draft, v, dtype, 0), h_draft)
       .total;
 }
 
@@ -665,24 +666,35 @@ extern "C" int tlce_kl_forward_with_gradient(
   if (m == 0) return 0;
   TLCE_REQUIRE(kl_gradient_in_forward_supported(m, h_draft, h_teacher, v, dtype, logit_softcap),
                "kl_forward_with_gradient: needs bf16 inputs, no soft cap, both hidden sizes and v "
-               "multiples of 64, and all rows in one block of the panel budget (m=%lld, v=%lld)",
-               (long long)m, (long long)v);
+               "multiples of 64 (h_draft=%lld, h_teacher=%lld, v=%lld)", (long long)h_draft,
+               (long long)h_teacher, (long long)v);
   TLCE_REQUIRE(losses && draft_lse && teacher_lse && unit_grad_hidden_f32 && workspace,
                "kl_forward_with_gradient: null pointer");
   TLCE_REQUIRE(((uintptr_t)unit_grad_hidden_f32 & 15) == 0,
                "kl_forward_with_gradient: the gradient buffer must be 16-byte aligned");
-  const KlPlans k = kl_plans(m, h_draft, h_teacher, v, dtype, panel_bytes);
-  const FusedPlan fp = make_fused_plan(m, h_draft, v, dtype, 0);
-  const int64_t need = kl_fused_layout(k.layout, k.draft, fp, h_draft).total;
+  const int64_t need = tlce_kl_forward_with_gradient_workspace_bytes(m, h_draft, h_teacher, v,
+                                                                     dtype, panel_bytes);
   TLCE_REQUIRE(workspace_bytes >= need,
                "kl_forward_with_gradient: workspace too small (%lld < %lld)",
                (long long)workspace_bytes, (long long)need);
   TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
                "kl_forward_with_gradient: workspace must be 256-byte aligned");
-  return kl_forward_with_gradient_impl<MfmaDirect4Engine<__bf16>>(
-      k.draft, k.teacher, k.layout, fp, draft_hidden, draft_weight, teacher_hidden,
-      teacher_weight, m, h_draft, h_teacher, v, dtype, losses, draft_lse, teacher_lse,
-      unit_grad_hidden_f32, static_cast<char*>(workspace), stream);
+  // rows are independent: blocks of the panel budget one after the other
+  const int64_t block = fused_row_block(m, h_draft, v, dtype);
+  const int64_t es = dtype_bytes(dtype);
+  for (int64_t r0 = 0; r0 < m; r0 += block) {
+    const int64_t rows = std::min(block, m - r0);
+    const KlPlans k = kl_plans(rows, h_draft, h_teacher, v, dtype, panel_bytes);
+    const FusedPlan fp = make_fused_plan(rows, h_draft, v, dtype, 0);
+    if (int rc = kl_forward_with_gradient_impl<MfmaDirect4Engine<__bf16>>(
+            k.draft, k.teacher, k.layout, fp,
+            static_cast<const char*>(draft_hidden) + r0 * h_draft * es, draft_weight,
+            static_cast<const char*>(teacher_hidden) + r0 * h_teacher * es, teacher_weight, rows,
+            h_draft, h_teacher, v, dtype, losses + r0, draft_lse + r0, teacher_lse + r0,
+            unit_grad_hidden_f32 + r0 * h_draft, static_cast<char*>(workspace), stream))
+      return rc;
+  }
+  return 0;
 }
 
 extern "C" int tlce_kl_backward(const void* draft_hidden, const void* draft_weight,
@@ -772,8 +784,9 @@ extern "C" int64_t tlce_ce_topk_forward_with_gradient_workspace_bytes(int64_t m,
                                                                       int64_t v, int dtype,
                                                                       int64_t panel_bytes) {
   if (m <= 0 || h <= 0 || v <= 0 || !topk_gradient_in_forward_supported(m, h, v, dtype)) return -1;
-  return topk_fused_layout(topk_plan(m, h, v, dtype, panel_bytes),
-                           make_fused_plan(m, h, v, dtype, 0), h).total;
+  const int64_t rows = std::min(m, fused_row_block(m, h, v, dtype));   // the largest block
+  return topk_fused_layout(topk_plan(rows, h, v, dtype, panel_bytes),
+                           make_fused_plan(rows, h, v, dtype, 0), h).total;
 }
 
 extern "C" int tlce_ce_topk_forward_with_gradient(
@@ -786,26 +799,34 @@ extern "C" int tlce_ce_topk_forward_with_gradient(
   if (int rc = topk_validate(hidden, weight, labels, m, h, v, dtype, top_k)) return rc;
   if (m == 0) return 0;
   TLCE_REQUIRE(topk_gradient_in_forward_supported(m, h, v, dtype),
-               "ce_topk_forward_with_gradient: needs bf16 inputs, h and v multiples of 64 and all "
-               "rows in one block of the exponentiated-logits panel (m=%lld, v=%lld)",
-               (long long)m, (long long)v);
+               "ce_topk_forward_with_gradient: needs bf16 inputs with h and v multiples of 64 "
+               "(h=%lld, v=%lld)", (long long)h, (long long)v);
   TLCE_REQUIRE(losses && probabilities && top_values && top_ids && lse && unit_grad_hidden_f32 &&
                    workspace,
                "ce_topk_forward_with_gradient: null pointer");
   TLCE_REQUIRE(((uintptr_t)unit_grad_hidden_f32 & 15) == 0,
                "ce_topk_forward_with_gradient: the gradient buffer must be 16-byte aligned");
-  const TopkPlan t = topk_plan(m, h, v, dtype, panel_bytes);
-  const FusedPlan p = make_fused_plan(m, h, v, dtype, 0);
-  const int64_t need = topk_fused_layout(t, p, h).total;
+  const int64_t need =
+      tlce_ce_topk_forward_with_gradient_workspace_bytes(m, h, v, dtype, panel_bytes);
   TLCE_REQUIRE(workspace_bytes >= need,
                "ce_topk_forward_with_gradient: workspace too small (%lld < %lld)",
                (long long)workspace_bytes, (long long)need);
   TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
                "ce_topk_forward_with_gradient: workspace must be 256-byte aligned");
-  return topk_forward_with_gradient_impl<MfmaDirect4Engine<__bf16>>(
-      t, p, hidden, weight, labels, m, h, v, top_k, output_multiplier, logit_softcap, losses,
-      probabilities, top_values, top_ids, lse, unit_grad_hidden_f32,
-      static_cast<char*>(workspace), stream);
+  const int64_t block = fused_row_block(m, h, v, dtype);
+  const char* hidden_b = static_cast<const char*>(hidden);
+  for (int64_t r0 = 0; r0 < m; r0 += block) {
+    const int64_t rows = std::min(block, m - r0);
+    const TopkPlan t = topk_plan(rows, h, v, dtype, panel_bytes);
+    const FusedPlan p = make_fused_plan(rows, h, v, dtype, 0);
+    if (int rc = topk_forward_with_gradient_impl<MfmaDirect4Engine<__bf16>>(
+            t, p, hidden_b + r0 * h * dtype_bytes(dtype), weight, labels + r0, rows, h, v, top_k,
+            output_multiplier, logit_softcap, losses + r0, probabilities + r0,
+            top_values + r0 * top_k, top_ids + r0 * top_k, lse + r0,
+            unit_grad_hidden_f32 + r0 * h, static_cast<char*>(workspace), stream))
+      return rc;
+  }
+  return 0;
 }
 
 extern "C" int tlce_ce_topk_apply_gradient(const float* unit_grad_hidden_f32, const void* hidden,
