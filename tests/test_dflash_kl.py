@@ -161,20 +161,23 @@ def test_kept_teacher_probabilities_give_the_same_gradient(gpu_device, dtype, hd
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("m,hd,ht,v,std", [
-    (300, 128, 192, 4096, 0.2),
-    (700, 64, 64, 2048, 1.5),        # logits tens of nats apart: entries far below their tile maximum
-    (1, 256, 128, 576, 0.3),
+@pytest.mark.parametrize("m,hd,ht,v,std,softcap", [
+    (300, 128, 192, 4096, 0.2, None),
+    (700, 64, 64, 2048, 1.5, None),  # logits tens of nats apart: entries far below their tile maximum
+    (1, 256, 128, 576, 0.3, None),
+    (300, 128, 128, 2048, 0.3, 6.0),
+    (520, 64, 128, 4096, 3.0, 30.0),  # logits deep in the cap on both sides
 ])
-def test_gradient_formed_in_the_forward(gpu_device, m, hd, ht, v, std, set_panel_budget):
-    """bf16 without a soft cap: the draft pass of the forward leaves exp2(z2 - tile
-    maximum), and d loss / d draft_hidden is contracted in the forward (its grad_hidden
+def test_gradient_formed_in_the_forward(gpu_device, m, hd, ht, v, std, softcap,
+                                        set_panel_budget):
+    """bf16 (with a soft cap of at most 40, or none): the draft pass of the forward leaves
+    exp2(z2 - tile maximum), and d loss / d draft_hidden is contracted in the forward (its grad_hidden
     contraction shows in the forward's launch counts); the backward scales rows.  Loss and
     gradient against the float64 oracle, over several vocabulary panels; the loss agrees
     with the plain forward's to float32 rounding (the draft's tile sums are taken against
     the tile's exact maximum instead of per-thread maxima)."""
     from turbo_dllm_amd import _lib, options
-    print("[case] KL gradient in the forward", m, hd, ht, v, std, flush=True)
+    print("[case] KL gradient in the forward", m, hd, ht, v, std, softcap, flush=True)
     set_panel_budget(512 * 512 * 2)
     gen = torch.Generator().manual_seed(m + v)
     cpu = [torch.randn(m, hd, generator=gen), torch.randn(v, hd, generator=gen) * std,
@@ -184,17 +187,18 @@ def test_gradient_formed_in_the_forward(gpu_device, m, hd, ht, v, std, set_panel
     go = torch.rand(m, generator=gen) + 0.1
     x = ops[0].clone().requires_grad_(True)
     with _lib.kernel_profile() as prof:
-        losses = frozen_linear_kl(x, ops[1], ops[2], ops[3])
+        losses = frozen_linear_kl(x, ops[1], ops[2], ops[3], logit_softcap=softcap)
         torch.cuda.synchronize()
     assert prof.launches["grad_hidden_gemm"] == 1
     losses.backward(go.to(gpu_device))
     torch.cuda.synchronize()
     with options.gradient_mode("recompute"):
-        plain = frozen_linear_kl(ops[0], ops[1], ops[2], ops[3])
+        plain = frozen_linear_kl(ops[0], ops[1], ops[2], ops[3], logit_softcap=softcap)
     torch.testing.assert_close(losses.detach().cpu(), plain.cpu(), rtol=1e-5, atol=1e-5)
-    ref_loss = oracle.dense_frozen_kl(cpu[0], cpu[1], cpu[2], cpu[3])
+    ref_loss = oracle.dense_frozen_kl(cpu[0], cpu[1], cpu[2], cpu[3], logit_softcap=softcap)
     torch.testing.assert_close(losses.detach().cpu().double(), ref_loss, rtol=2e-2, atol=1e-3)
-    ref_grad = oracle.dense_frozen_kl_grad(cpu[0], cpu[1], cpu[2], cpu[3], go)
+    ref_grad = oracle.dense_frozen_kl_grad(cpu[0], cpu[1], cpu[2], cpu[3], go,
+                                           logit_softcap=softcap)
     err = oracle.relative_max_error(x.grad.cpu(), ref_grad)
     print("[case] grad rel max err", f"{err:.2e}", flush=True)
     assert bool(torch.isfinite(x.grad.float()).all())

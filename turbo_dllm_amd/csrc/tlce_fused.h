@@ -766,8 +766,10 @@ int topk_forward_with_gradient_impl(const TopkPlan& t, const FusedPlan& p, const
 //   g[r, v] = e[r, v] * exp2(part_max[tile(v), r] - lse2_draft[r]) - t[r, v]
 // (lce_kl_grad_from_exp_kernel), and one contraction with the draft head leaves
 //   unit[r, :] = d loss[r] / d draft_hidden[r, :]       float32 [m, h].
-// The backward multiplies row r by its upstream gradient and rounds once.  No soft cap
-// (its derivative would have to be re-derived from the rounded entries).
+// The backward multiplies row r by its upstream gradient and rounds once.  Under a soft
+// cap the gradient also carries cap'(z) = 1 - (z / cap)^2, with z re-derived from the
+// entry (z2 = log2(entry) + tile maximum; the rounding of the entry moves z by less than
+// 0.003); a cap of at most kSoftEmbeddingMaxCap keeps every entry a normal bf16 number.
 struct KlGradFromExpArgs {
   void* exp_panel;           // bf16 [mp, ld]: e in, logit gradient out
   const void* teacher;       // bf16 [mp, ld] teacher probabilities
@@ -776,6 +778,7 @@ struct KlGradFromExpArgs {
   const float* part_max;     // [n_vtiles, part_ld] base-2 tile maxima
   int part_ld;
   const float* draft_lse;    // [m] natural units
+  float softcap = 0.0f;      // > 0: the gradient is multiplied by cap'(z)
 };
 int launch_kl_grad_from_exp(const KlGradFromExpArgs& a, int n_vtiles, hipStream_t stream);
 
@@ -783,23 +786,29 @@ struct KlFusedLayout {
   int64_t kl, teacher, exp_panel, slabs, total;
 };
 
-template <class E>
-int launch_kl_panel_emit(const KlPanelArgs& a, hipStream_t stream) {
+template <class E, bool kSoftcap>
+int launch_kl_panel_emit_variant(const KlPanelArgs& a, hipStream_t stream) {
   static LdsOptIn lds;
   constexpr int kLdsBytes = E::kSmemBytes + E::kShare * E::kTile * (int)sizeof(float);
-  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, false, false, true>, kLdsBytes, lds))
+  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap, false, true>, kLdsBytes, lds))
     return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
   ScopedTimer timer(kClassGradLogits, stream);
-  lce_kl_panel_kernel<E, false, false, true><<<grid, E::kThreads, kLdsBytes, stream>>>(a);
+  lce_kl_panel_kernel<E, kSoftcap, false, true><<<grid, E::kThreads, kLdsBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
+}
+
+template <class E>
+int launch_kl_panel_emit(const KlPanelArgs& a, hipStream_t stream) {
+  return a.softcap > 0.0f ? launch_kl_panel_emit_variant<E, true>(a, stream)
+                          : launch_kl_panel_emit_variant<E, false>(a, stream);
 }
 
 inline bool kl_gradient_in_forward_supported(int64_t m, int64_t hd, int64_t ht, int64_t v,
                                              int dtype, float softcap) {
   (void)m;   // rows beyond one block of the panel budget are taken block by block
-  return softcap <= 0.0f && fused_gradients_supported(hd, v, dtype) &&
+  return softcap <= kSoftEmbeddingMaxCap && fused_gradients_supported(hd, v, dtype) &&
          engine_class(ht, dtype) == 2;
 }
 
@@ -820,9 +829,9 @@ int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout
                                   const FusedPlan& fp, const void* draft_hidden,
                                   const void* draft_weight, const void* teacher_hidden,
                                   const void* teacher_weight, int64_t m, int64_t hd, int64_t ht,
-                                  int64_t v, int dtype, float* losses, float* draft_lse,
-                                  float* teacher_lse, float* unit_grad, char* ws,
-                                  hipStream_t stream) {
+                                  int64_t v, int dtype, float softcap, float* losses,
+                                  float* draft_lse, float* teacher_lse, float* unit_grad,
+                                  char* ws, hipStream_t stream) {
   using T = typename E::T;
   const KlFusedLayout l = kl_fused_layout(kl, pd, fp, hd);
   char* kws = ws + l.kl;
@@ -832,7 +841,7 @@ int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout
   // the forward as ever, its teacher panels going to `teacher` and its draft pass
   // leaving exp2(z2 - tile maximum) in `exp_panel`
   if (int rc = kl_forward_impl<E>(pd, pt, kl, draft_hidden, draft_weight, teacher_hidden,
-                                  teacher_weight, m, hd, ht, v, dtype, 0.0f, losses, draft_lse,
+                                  teacher_weight, m, hd, ht, v, dtype, softcap, losses, draft_lse,
                                   teacher_lse, kws, stream, teacher, exp_panel))
     return rc;
   const float* part_max = reinterpret_cast<const float*>(kws + kl.stats);
@@ -840,6 +849,7 @@ int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout
   ga.exp_panel = exp_panel; ga.teacher = teacher; ga.ld = pd.vp;
   ga.m = (int)m; ga.mp = (int)pd.mp;
   ga.part_max = part_max; ga.part_ld = (int)pd.mp; ga.draft_lse = draft_lse;
+  ga.softcap = softcap;
   if (int rc = launch_kl_grad_from_exp(ga, pd.n_vtiles, stream)) return rc;
 
   const float* ones = reinterpret_cast<const float*>(kws + kl.ones);
@@ -879,8 +889,8 @@ int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout
   X int kl_forward_with_gradient_impl<E>(const Plan&, const Plan&, const KlLayout&,              \
                                          const FusedPlan&, const void*, const void*,             \
                                          const void*, const void*, int64_t, int64_t, int64_t,    \
-                                         int64_t, int, float*, float*, float*, float*, char*,    \
-                                         hipStream_t);                                           \
+                                         int64_t, int, float, float*, float*, float*, float*,    \
+                                         char*, hipStream_t);                                    \
   X int deferred_grad_weight_impl<E>(const FusedPlan&, const void*, int64_t, int64_t, int64_t,   \
                                      int, const float*, const float*, int, const int64_t*,       \
                                      const int64_t*, void*, char*, hipStream_t);

@@ -647,6 +647,7 @@ extern "C" int64_t tlce_kl_forward_with_gradient_workspace_bytes(int64_t m, int6
                                                                  int64_t h_teacher, int64_t v,
                                                                  int dtype, int64_t panel_bytes) {
   if (!tlce_kl_gradient_in_forward_supported(m, h_draft, h_teacher, v, dtype, 0.0f)) return -1;
+  // (the soft cap does not change the layout)
   const int64_t rows = std::min(m, fused_row_block(m, h_draft, v, dtype));   // the largest block
   const KlPlans k = kl_plans(rows, h_draft, h_teacher, v, dtype, panel_bytes);
   return kl_fused_layout(k.layout, k.draft, make_fused_plan(rows, h_draft, v, dtype, 0), h_draft)
@@ -665,9 +666,9 @@ extern "C" int tlce_kl_forward_with_gradient(
     return rc;
   if (m == 0) return 0;
   TLCE_REQUIRE(kl_gradient_in_forward_supported(m, h_draft, h_teacher, v, dtype, logit_softcap),
-               "kl_forward_with_gradient: needs bf16 inputs, no soft cap, both hidden sizes and v "
-               "multiples of 64 (h_draft=%lld, h_teacher=%lld, v=%lld)", (long long)h_draft,
-               (long long)h_teacher, (long long)v);
+               "kl_forward_with_gradient: needs bf16 inputs, a soft cap of at most 40 or none, both "
+               "hidden sizes and v multiples of 64 (h_draft=%lld, h_teacher=%lld, v=%lld)",
+               (long long)h_draft, (long long)h_teacher, (long long)v);
   TLCE_REQUIRE(losses && draft_lse && teacher_lse && unit_grad_hidden_f32 && workspace,
                "kl_forward_with_gradient: null pointer");
   TLCE_REQUIRE(((uintptr_t)unit_grad_hidden_f32 & 15) == 0,
@@ -690,7 +691,8 @@ extern "C" int tlce_kl_forward_with_gradient(
             k.draft, k.teacher, k.layout, fp,
             static_cast<const char*>(draft_hidden) + r0 * h_draft * es, draft_weight,
             static_cast<const char*>(teacher_hidden) + r0 * h_teacher * es, teacher_weight, rows,
-            h_draft, h_teacher, v, dtype, losses + r0, draft_lse + r0, teacher_lse + r0,
+            h_draft, h_teacher, v, dtype, logit_softcap, losses + r0, draft_lse + r0,
+            teacher_lse + r0,
             unit_grad_hidden_f32 + r0 * h_draft, static_cast<char*>(workspace), stream))
       return rc;
   }
