@@ -379,9 +379,10 @@ def bench_next_objective(args) -> int:
             draft_h.grad = None
             frozen_linear_kl(draft_h, draft_w, teacher_h, teacher_w).sum().backward()
 
-        # teacher statistics, teacher panels, draft pass, and the gradient contraction in
-        # the same forward; the backward scales rows (--gradients recompute: 3 + 3)
-        contractions = 4 if args.gradients == "forward" else 6
+        # one pass over the teacher head, one over the draft head, and the gradient
+        # contraction, all in the forward; the backward scales rows
+        # (--gradients recompute: 3 + 3)
+        contractions = 3 if args.gradients == "forward" else 6
         name = "frozen-head KL fwd+bwd"
         shape = f"M={m}, H_draft=H_teacher={h}, V={v}"
     elif args.objective == "ce_topk":

@@ -377,12 +377,16 @@ int tlce_kl_forward(const void* draft_hidden, const void* draft_weight,
 int64_t tlce_kl_teacher_probabilities_bytes(int64_t m, int64_t h_draft,
                                             int64_t h_teacher, int64_t v, int dtype);
 
-/* The forward with the gradient formed in it: 4 contractions per forward +
- * backward.  The draft pass, which holds every draft logit in registers, also
+/* The forward with the gradient formed in it: 3 contractions per forward +
+ * backward.  A pass over a head holds every logit of a tile in registers; it
  * writes exp2(logit2 - the exact maximum of the token's 256-entry vocabulary
- * tile) <= 1 in bf16 into a second panel over the whole vocabulary beside the
- * teacher probabilities; once the draft lse is known one elementwise pass forms
- *   g[r, v] = entry * exp2(tile maximum - lse2_draft[r]) - p_t[r, v]
+ * tile) <= 1 in bf16 into a panel over the whole vocabulary and leaves the
+ * tile's (maximum, sum), so that softmax = entry * exp2(tile maximum - lse2)
+ * per (token, tile) once the lse is merged.  One such pass over the teacher
+ * head replaces its statistics pass and its probabilities pass; the draft pass
+ * reads the teacher's entries, accumulates the loss terms and writes its own
+ * entries into a second panel; one elementwise pass then forms
+ *   g[r, v] = entry_d * exp2(max_d - lse2_d[r]) - entry_t * exp2(max_t - lse2_t[r])
  * (times cap'(z) under a soft cap, z re-derived from the entry), and one
  * contraction with the draft head leaves
  *   unit_grad_hidden_f32[r, :] = d losses[r] / d draft_hidden[r, :]   float32 [m, h_draft].

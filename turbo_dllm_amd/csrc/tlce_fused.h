@@ -757,13 +757,18 @@ int topk_forward_with_gradient_impl(const TopkPlan& t, const FusedPlan& p, const
   return launch_reduce_slabs(rs, stream);
 }
 
-// ---- frozen-head KL: the gradient formed in the forward (4 contractions, not 6) ----
-// The draft pass of the forward already holds every draft logit in registers.  In its
-// emitting variant (lce_kl_panel_kernel<.., kEmit>) it also writes exp2(z2 - tile
-// maximum) <= 1 of every entry in bf16 into a second panel over the whole vocabulary,
-// beside the teacher probabilities.  When the pass is over the draft lse is known,
-// one elementwise pass turns the two panels into the logit gradient
-//   g[r, v] = e[r, v] * exp2(part_max[tile(v), r] - lse2_draft[r]) - t[r, v]
+// ---- frozen-head KL: the gradient formed in the forward (3 contractions, not 6) ----
+// A pass over a head holds every logit of a tile in registers.  The emitting variant of
+// the KL panel kernel (lce_kl_panel_kernel<.., kEmit>) finds the exact maximum of each
+// token over the tile's 256 vocabulary rows and writes e = exp2(z2 - tile maximum) <= 1
+// in bf16 into a panel over the whole vocabulary, beside the tile's softmax partials:
+// softmax = e * exp2(tile maximum - lse2) per (token, tile) once the lse is known, and
+// nothing has to be known beforehand.  One such pass over the teacher head (no teacher
+// tile to read: kNoTeacher) replaces its statistics pass and its probabilities pass;
+// the draft pass reads the teacher's entries, scales them to probabilities per (token,
+// tile), accumulates the loss terms and emits its own entries.  One elementwise pass
+// then turns the two panels into the logit gradient
+//   g[r, v] = e_d * exp2(max_d[tile, r] - lse2_d[r]) - e_t * exp2(max_t[tile, r] - lse2_t[r])
 // (lce_kl_grad_from_exp_kernel), and one contraction with the draft head leaves
 //   unit[r, :] = d loss[r] / d draft_hidden[r, :]       float32 [m, h].
 // The backward multiplies row r by its upstream gradient and rounds once.  Under a soft
@@ -775,34 +780,43 @@ struct KlGradFromExpArgs {
   const void* teacher;       // bf16 [mp, ld] teacher probabilities
   int64_t ld;
   int m, mp;
-  const float* part_max;     // [n_vtiles, part_ld] base-2 tile maxima
+  const float* part_max;     // [n_vtiles, part_ld] base-2 tile maxima of the draft
   int part_ld;
   const float* draft_lse;    // [m] natural units
   float softcap = 0.0f;      // > 0: the gradient is multiplied by cap'(z)
+  const float* t_part_max = nullptr;   // non-null: `teacher` holds entries of the same kind,
+  const float* t_lse = nullptr;        // these are the teacher's tile maxima and lse
 };
 int launch_kl_grad_from_exp(const KlGradFromExpArgs& a, int n_vtiles, hipStream_t stream);
 
 struct KlFusedLayout {
-  int64_t kl, teacher, exp_panel, slabs, total;
+  int64_t kl, teacher_parts, teacher, exp_panel, slabs, total;
 };
 
-template <class E, bool kSoftcap>
+template <class E, bool kSoftcap, bool kNoTeacher>
 int launch_kl_panel_emit_variant(const KlPanelArgs& a, hipStream_t stream) {
   static LdsOptIn lds;
   constexpr int kLdsBytes = E::kSmemBytes + E::kShare * E::kTile * (int)sizeof(float);
-  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap, false, true>, kLdsBytes, lds))
+  if (int rc = enable_large_lds(lce_kl_panel_kernel<E, kSoftcap, false, true, kNoTeacher>,
+                                kLdsBytes, lds))
     return rc;
   const int grid = xcd_grid((int64_t)a.n_ttiles * a.n_ptiles);
   ScopedTimer timer(kClassGradLogits, stream);
-  lce_kl_panel_kernel<E, kSoftcap, false, true><<<grid, E::kThreads, kLdsBytes, stream>>>(a);
+  lce_kl_panel_kernel<E, kSoftcap, false, true, kNoTeacher>
+      <<<grid, E::kThreads, kLdsBytes, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
 
+// panel_in == null: the pass over a head on its own (no teacher tile is read)
 template <class E>
 int launch_kl_panel_emit(const KlPanelArgs& a, hipStream_t stream) {
-  return a.softcap > 0.0f ? launch_kl_panel_emit_variant<E, true>(a, stream)
-                          : launch_kl_panel_emit_variant<E, false>(a, stream);
+  if (a.panel_in == nullptr) {
+    return a.softcap > 0.0f ? launch_kl_panel_emit_variant<E, true, true>(a, stream)
+                            : launch_kl_panel_emit_variant<E, false, true>(a, stream);
+  }
+  return a.softcap > 0.0f ? launch_kl_panel_emit_variant<E, true, false>(a, stream)
+                          : launch_kl_panel_emit_variant<E, false, false>(a, stream);
 }
 
 inline bool kl_gradient_in_forward_supported(int64_t m, int64_t hd, int64_t ht, int64_t v,
@@ -817,6 +831,7 @@ inline KlFusedLayout kl_fused_layout(const KlLayout& kl, const Plan& pd, const F
   KlFusedLayout l;
   int64_t off = 0;
   l.kl = off;         off += align256(kl.total);
+  l.teacher_parts = off;  off += 2 * kl.tile_part;
   l.teacher = off;    off += align256(pd.mp * pd.vp * 2);
   l.exp_panel = off;  off += align256(pd.mp * pd.vp * 2);
   l.slabs = off;      off += align256((int64_t)p.dh_ksplit * pd.mp * hd * 4);
@@ -838,21 +853,74 @@ int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout
   T* teacher = reinterpret_cast<T*>(ws + l.teacher);
   T* exp_panel = reinterpret_cast<T*>(ws + l.exp_panel);
   float* slabs = reinterpret_cast<float*>(ws + l.slabs);
-  // the forward as ever, its teacher panels going to `teacher` and its draft pass
-  // leaving exp2(z2 - tile maximum) in `exp_panel`
-  if (int rc = kl_forward_impl<E>(pd, pt, kl, draft_hidden, draft_weight, teacher_hidden,
-                                  teacher_weight, m, hd, ht, v, dtype, softcap, losses, draft_lse,
-                                  teacher_lse, kws, stream, teacher, exp_panel))
+  float* part_max = reinterpret_cast<float*>(kws + kl.stats);
+  float* part_sum = reinterpret_cast<float*>(kws + kl.stats + kl.tile_part);
+  float* loss_part = reinterpret_cast<float*>(kws + kl.stats + 2 * kl.tile_part);
+  float* tsum_part = reinterpret_cast<float*>(kws + kl.stats + 3 * kl.tile_part);
+  float* t_part_max = reinterpret_cast<float*>(ws + l.teacher_parts);
+  float* t_part_sum = reinterpret_cast<float*>(ws + l.teacher_parts + kl.tile_part);
+  float* ones = reinterpret_cast<float*>(kws + kl.ones);
+  (void)pt;
+  ScaleArgs sa;
+  sa.labels = nullptr; sa.row_idx = nullptr; sa.grad_output = nullptr; sa.valid_count = nullptr;
+  sa.m = (int)m; sa.mp = (int)pd.mp; sa.reduction = TLCE_REDUCTION_SUM; sa.ignore = 0;
+  sa.scale = ones; sa.constant = 1.0f; sa.multiplier = 1.0f;
+  if (int rc = launch_token_scale(sa, stream)) return rc;
+
+  auto lse_from_partials = [&](const void* hidden, const void* weight, int64_t h,
+                               const float* pmax, const float* psum, float* lse) -> int {
+    CombineArgs ca;
+    ca.hidden = hidden; ca.weight = weight; ca.bias = nullptr; ca.labels = nullptr;
+    ca.row_idx = nullptr;
+    ca.m = (int)m; ca.h = (int)h; ca.v = (int)v;
+    ca.ignore = 0; ca.exclude = -1; ca.softcap = softcap;
+    ca.part_max = pmax; ca.part_sum = psum;
+    ca.part_ld = (int)pd.mp; ca.nsplit = pd.n_vtiles;
+    ca.losses = nullptr; ca.lse = lse; ca.valid_count = nullptr;
+    ca.label_offset = 0; ca.local_max = nullptr; ca.local_sum = nullptr;
+    ca.target_logits = nullptr;
+    ScopedTimer timer(kClassCombine, stream);
+    lce_combine_loss_kernel<T><<<(int)ceil_div(m, kCombineRowsPerBlock), 256, 0, stream>>>(ca);
+    TLCE_LAUNCH_CHECK();
+    return 0;
+  };
+
+  KlPanelArgs ka;
+  ka.lse = nullptr; ka.scale = nullptr;
+  ka.m = (int)m; ka.v = (int)v; ka.softcap = softcap;
+  ka.v0 = 0; ka.n_ttiles = pd.n_ttiles; ka.n_ptiles = pd.n_vtiles;
+  ka.ld = pd.vp; ka.part_ld = (int)pd.mp; ka.mode = kKlLoss;
+  ka.loss_part = loss_part; ka.tsum_part = tsum_part;
+  // the teacher head on its own: entries and softmax partials in one contraction
+  ka.hidden = teacher_hidden; ka.weight = teacher_weight; ka.h = (int)ht;
+  ka.panel = teacher; ka.panel_in = nullptr;
+  ka.part_max = t_part_max; ka.part_sum = t_part_sum;
+  if (int rc = launch_kl_panel_emit<E>(ka, stream)) return rc;
+  if (int rc = lse_from_partials(teacher_hidden, teacher_weight, ht, t_part_max, t_part_sum,
+                                 teacher_lse))
     return rc;
-  const float* part_max = reinterpret_cast<const float*>(kws + kl.stats);
+  // the draft head against it: loss terms, softmax partials and its own entries
+  ka.hidden = draft_hidden; ka.weight = draft_weight; ka.h = (int)hd;
+  ka.panel = exp_panel; ka.panel_in = teacher; ka.ld_in = pd.vp;
+  ka.t_part_max = t_part_max; ka.t_lse = teacher_lse;
+  ka.part_max = part_max; ka.part_sum = part_sum;
+  if (int rc = launch_kl_panel_emit<E>(ka, stream)) return rc;
+  if (int rc = lse_from_partials(draft_hidden, draft_weight, hd, part_max, part_sum, draft_lse))
+    return rc;
+  {
+    ScopedTimer timer(kClassCombine, stream);
+    if (int rc = launch_kl_finish(losses, loss_part, tsum_part, pd.n_vtiles, pd.mp, draft_lse, m,
+                                  stream))
+      return rc;
+  }
   KlGradFromExpArgs ga;
   ga.exp_panel = exp_panel; ga.teacher = teacher; ga.ld = pd.vp;
   ga.m = (int)m; ga.mp = (int)pd.mp;
   ga.part_max = part_max; ga.part_ld = (int)pd.mp; ga.draft_lse = draft_lse;
   ga.softcap = softcap;
+  ga.t_part_max = t_part_max; ga.t_lse = teacher_lse;
   if (int rc = launch_kl_grad_from_exp(ga, pd.n_vtiles, stream)) return rc;
 
-  const float* ones = reinterpret_cast<const float*>(kws + kl.ones);
   GemmArgs g;
   g.a = draft_weight; g.lda = hd; g.a_rows = (int)hd;
   g.b = exp_panel; g.ldb = pd.vp; g.b_rows = (int)pd.mp;

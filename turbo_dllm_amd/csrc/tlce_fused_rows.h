@@ -214,6 +214,10 @@ __global__ __launch_bounds__(256) void lce_kl_grad_from_exp_kernel(KlGradFromExp
   if (r < p.m) {
     const float tile_max2 = p.part_max[(int64_t)tile * p.part_ld + r];
     const float f = exp2f(tile_max2 - p.draft_lse[r] * TLCE_LOG2E);
+    const float ft = p.t_part_max != nullptr
+                         ? exp2f(p.t_part_max[(int64_t)tile * p.part_ld + r] -
+                                 p.t_lse[r] * TLCE_LOG2E)
+                         : 1.0f;
     const float inv_cap = p.softcap > 0.0f ? TLCE_LN2 / p.softcap : 0.0f;
     const v8_t ev = *reinterpret_cast<const v8_t*>(e);
     const v8_t tv = *reinterpret_cast<const v8_t*>(static_cast<const __bf16*>(p.teacher) +
@@ -221,7 +225,7 @@ __global__ __launch_bounds__(256) void lce_kl_grad_from_exp_kernel(KlGradFromExp
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float ei = to_float<__bf16>(ev[i]);
-      float g = ei * f - to_float<__bf16>(tv[i]);
+      float g = ei * f - to_float<__bf16>(tv[i]) * ft;
       if (p.softcap > 0.0f) {
         // (an entry of 0 is a column past the vocabulary: its gradient is 0 anyway)
         const float t = ei > 0.0f ? (log2f(ei) + tile_max2) * inv_cap : 0.0f;

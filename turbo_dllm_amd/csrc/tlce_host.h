@@ -23,7 +23,6 @@
 #include <algorithm>
 #include <atomic>
 #include <functional>
-#include <type_traits>
 #include <vector>
 
 #include "tlce_common.h"
@@ -651,22 +650,6 @@ int launch_kl_panel(const KlPanelArgs& a, hipStream_t stream) {
               : launch_kl_panel_variant<E, false, false>(a, stream);
 }
 
-// The emitting variant of the draft pass exists for the four-wave bf16 engine only
-// (defined beside the forward that leaves the gradients).
-template <class E>
-int launch_kl_panel_emit(const KlPanelArgs& a, hipStream_t stream);
-
-template <class E>
-int launch_kl_panel_emit_if(const KlPanelArgs& a, hipStream_t stream) {
-  if constexpr (E::kHasKMajor && sizeof(typename E::T) == 2 && E::kCols == 4 &&
-                std::is_same<typename E::T, __bf16>::value) {
-    return launch_kl_panel_emit<E>(a, stream);
-  } else {
-    (void)a; (void)stream;
-    return fail("kl: the emitting draft pass needs the bf16 direct engine");
-  }
-}
-
 // Teacher probabilities of the panel [v0, v0 + width), then the draft pass over it.
 template <class E>
 int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
@@ -675,7 +658,7 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
              int64_t hd, int64_t ht, int64_t v, float softcap, int64_t v0, int64_t width,
              void* g, float* loss_part, float* tsum_part, float* part_max, float* part_sum,
              int mode, hipStream_t stream, void* kept = nullptr, int64_t kept_ld = 0,
-             bool kept_is_written = false, void* emit = nullptr) {
+             bool kept_is_written = false) {
   // kept: a buffer over the whole vocabulary [mp, kept_ld] that holds the teacher
   // probabilities between forward and backward.  The forward produces each panel into
   // it (and reads it there); the backward (kept_is_written) skips the producer and
@@ -704,14 +687,6 @@ int kl_panel(const Plan& pd, const void* draft_hidden, const void* draft_weight,
   ga.grad_bias = nullptr;
   if (int rc = launch_grad_logits<E>(ga, stream)) return rc;
   ka.panel = teacher_panel; ka.ld = teacher_ld;
-  if (emit != nullptr) {
-    // the draft pass also leaves exp2(z2 - tile maximum) in a second panel laid out
-    // like the kept teacher panel (direct bf16 engine only)
-    ka.panel_in = teacher_panel; ka.ld_in = teacher_ld;
-    ka.panel = static_cast<char*>(emit) + v0 * (int64_t)sizeof(typename E::T);
-    ka.ld = kept_ld;
-    return launch_kl_panel_emit_if<E>(ka, stream);
-  }
   return launch_kl_panel<E>(ka, stream);
 }
 
@@ -720,8 +695,7 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
                     const void* draft_weight, const void* teacher_hidden,
                     const void* teacher_weight, int64_t m, int64_t hd, int64_t ht, int64_t v,
                     int dtype, float softcap, float* losses, float* draft_lse, float* teacher_lse,
-                    char* ws, hipStream_t stream, void* kept_teacher = nullptr,
-                    void* emit_exp = nullptr) {
+                    char* ws, hipStream_t stream, void* kept_teacher = nullptr) {
   using T = typename E::T;
   // teacher statistics first: its probabilities need the teacher lse
   if (int rc = forward_impl<E>(pt, teacher_hidden, teacher_weight, nullptr, nullptr, nullptr, m,
@@ -752,7 +726,7 @@ int kl_forward_impl(const Plan& pd, const Plan& pt, const KlLayout& l, const voi
     if (int rc = kl_panel<E>(pd, draft_hidden, draft_weight, teacher_hidden, teacher_weight,
                              nullptr, teacher_lse, ones, nullptr, m, hd, ht, v, softcap, v0,
                              width, g, loss_part, tsum_part, part_max, part_sum, kKlLoss,
-                             stream, kept_teacher, pd.vp, false, emit_exp))
+                             stream, kept_teacher, pd.vp, false))
       return rc;
   }
   CombineArgs ca;
@@ -1039,7 +1013,7 @@ int soft_embedding_impl(const Plan& fp, const Plan& bp, const SoftEmbeddingLayou
                                float, void*, char*, hipStream_t);                               \
   X int kl_forward_impl<E>(const Plan&, const Plan&, const KlLayout&, const void*, const void*, \
                            const void*, const void*, int64_t, int64_t, int64_t, int64_t, int,   \
-                           float, float*, float*, float*, char*, hipStream_t, void*, void*);    \
+                           float, float*, float*, float*, char*, hipStream_t, void*);           \
   X int kl_backward_impl<E>(const Plan&, const KlLayout&, const void*, const void*,             \
                             const void*, const void*, const float*, const float*, const float*, \
                             int64_t, int64_t, int64_t, int64_t, int, float, void*, char*,       \

@@ -637,6 +637,11 @@ __global__ __launch_bounds__(E::kThreads) void lce_grad_logits_panel_kernel(Grad
 //                 lse is known, softmax = entry * exp2(part_max - lse2) per
 //                 (token, tile): the logit gradient can be formed from the two
 //                 panels without contracting the draft head again.
+//   kNoTeacher (with kEmit): no teacher tile is read (t = 0, the loss outputs are
+//                 meaningless): the pass only emits and leaves the softmax partials.
+//                 Run on the teacher head, it replaces the teacher's statistics pass
+//                 and its probabilities pass by one contraction; the draft pass then
+//                 takes t = entry * exp2(t_part_max - t_lse2) per (token, tile).
 enum { kKlLoss = 0, kKlGrad = 1 };
 
 struct KlPanelArgs {
@@ -652,6 +657,10 @@ struct KlPanelArgs {
   int64_t ld;
   const void* panel_in = nullptr;   // non-null: the teacher probabilities are read here
   int64_t ld_in = 0;                // ([mp, ld_in]) and `panel` only receives the gradients
+  // non-null: the teacher panel holds exp2(z2 - tile maximum) of the teacher head, these
+  // are its tile maxima [n vocabulary tiles, part_ld] and its lse [m] (natural units)
+  const float* t_part_max = nullptr;
+  const float* t_lse = nullptr;
   float* loss_part;     // kKlLoss: [n vocabulary tiles, part_ld] loss terms of the tile
   float* tsum_part;     // kKlLoss: [n vocabulary tiles, part_ld] teacher mass of the tile
   float* part_max;      // kKlLoss: [n vocabulary tiles, part_ld] base-2 tile maxima
@@ -660,9 +669,10 @@ struct KlPanelArgs {
   int mode;
 };
 
-template <class E, bool kSoftcap, bool kGrad, bool kEmit = false>
+template <class E, bool kSoftcap, bool kGrad, bool kEmit = false, bool kNoTeacher = false>
 __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p) {
   static_assert(!(kGrad && kEmit), "kEmit belongs to the loss mode");
+  static_assert(kEmit || !kNoTeacher, "kNoTeacher belongs to the emitting pass");
   extern __shared__ __align__(16) char smem[];
   using T = typename E::T;
   const int logical = xcd_logical_block(blockIdx.x, gridDim.x);
@@ -676,6 +686,7 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
   constexpr bool grad = kGrad;   // p.mode, fixed at compile time: no mode test per group of 4
   float lse2[E::kCols], scale[E::kCols], partial[E::kCols], tsum[E::kCols];
   float tile_max[E::kCols], tile_sum[E::kCols];
+  float tscale[E::kCols];   // teacher entry -> teacher probability
   bool live[E::kCols];
   // the per-row operands are loaded before the contraction: their latency passes under it
 #pragma unroll
@@ -689,6 +700,11 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
     tsum[j] = 0.0f;
     tile_max[j] = -INFINITY;
     tile_sum[j] = 0.0f;
+    tscale[j] = 1.0f;
+    if (kEmit && !kNoTeacher && p.t_part_max != nullptr) {
+      const float pm = p.t_part_max[(int64_t)(vbase / E::kTile) * p.part_ld + rc];
+      tscale[j] = exp2_of<E::kPrecise>(pm - p.t_lse[rc] * TLCE_LOG2E);
+    }
   }
   eng.mainloop_set(static_cast<const T*>(p.weight), p.h, vbase, p.v,
                    static_cast<const T*>(p.hidden), p.h, tt * E::kTile, p.m, 0, p.h, acc, smem);
@@ -753,11 +769,13 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
       } else {
         // z already is the capped draft logit in base-2 units (-inf past the vocabulary)
         // selects, not branches: the lanes of a wave disagree on tv > 0
-        const float tv = t[u];
+        const float tv = kNoTeacher ? 0.0f : t[u] * tscale[j];
         const float e = exp2_of<E::kPrecise>(z - tile_max[j]);
         tile_sum[j] += vok ? e : 0.0f;
         if (kEmit) g[u] = (vok && tile_max[j] > -INFINITY) ? e : 0.0f;
-        const bool use = vok && tv > 0.0f;
+        // (a product of an entry and a tile scale can be a denormal, whose fast log2 is
+        // -inf: probabilities below the smallest normal number carry no loss)
+        const bool use = vok && tv >= 1.17549435e-38f;
         const float term = tv * ((log2_of<E::kPrecise>(tv) - z) * TLCE_LN2) - tv;
         partial[j] += use ? term : 0.0f;
         tsum[j] += use ? tv : 0.0f;
@@ -768,16 +786,18 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
   if constexpr (kCanStage) {
     // the tile of the panel goes through LDS in whole 512-byte token rows
     // (16-byte chunk c of token t in slot c ^ (t & 31)), both ways
+    if constexpr (!kNoTeacher) {
 #pragma unroll 4
-    for (int it = 0; it < (E::kTile * 32) / E::kThreads; ++it) {
-      const int c = it * E::kThreads + threadIdx.x;
-      const int tok = c >> 5;
-      const int ch = c & 31;
-      *reinterpret_cast<uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)) =
-          *reinterpret_cast<const uint4*>(panel_in + ((int64_t)tt * E::kTile + tok) * ld_in +
-                                          prow + ch * 8);
+      for (int it = 0; it < (E::kTile * 32) / E::kThreads; ++it) {
+        const int c = it * E::kThreads + threadIdx.x;
+        const int tok = c >> 5;
+        const int ch = c & 31;
+        *reinterpret_cast<uint4*>(smem + tok * 512 + ((ch ^ (tok & 31)) * 16)) =
+            *reinterpret_cast<const uint4*>(panel_in + ((int64_t)tt * E::kTile + tok) * ld_in +
+                                            prow + ch * 8);
+      }
+      __syncthreads();
     }
-    __syncthreads();
 #pragma unroll
     for (int j = 0; j < E::kCols; ++j) {
       const int tok = eng.col(j);
@@ -787,7 +807,8 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
         T* cell = reinterpret_cast<T*>(smem + tok * 512 + (((vq >> 1) ^ (tok & 31)) * 16) +
                                        (vq & 1) * 8);
         typedef T v4_t __attribute__((ext_vector_type(4)));
-        const v4_t tv = *reinterpret_cast<const v4_t*>(cell);
+        v4_t tv = {};
+        if constexpr (!kNoTeacher) tv = *reinterpret_cast<const v4_t*>(cell);
         const float t[4] = {to_float<T>(tv[0]), to_float<T>(tv[1]), to_float<T>(tv[2]),
                             to_float<T>(tv[3])};
         float g[4];
