@@ -329,7 +329,11 @@ int tlce_backward_local(const void* hidden, const void* weight, const float* bia
  * two suffice: capped logits lie in [-cap, cap], so exp(logit - cap) needs no
  * row maximum; it is written for a block of rows over the whole vocabulary
  * into a panel of panel_bytes (0: 2.5 GiB), contracted with the weight rows, and
- * the result divided by the row's sum.  The workspace query covers both.
+ * the result divided by the row's sum.  Without such a cap the same operands
+ * take two contractions as well: one pass writes exp2(logit2 - the exact maximum
+ * of the token's 256-entry vocabulary tile) with the tile's softmax partials,
+ * the entries are normalised per (token, tile) once the lse is merged, then
+ * contracted.  The workspace query covers every sequence.
  *   hidden [m,h], weight [v,h], out [m,h], all `dtype`. */
 int64_t tlce_soft_embedding_workspace_bytes(int64_t m, int64_t h, int64_t v,
                                             int dtype, int64_t panel_bytes);

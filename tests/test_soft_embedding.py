@@ -93,17 +93,22 @@ def test_device_path_matches_dense(gpu_device, case):
     (30.0, 0, 3.0),      # the production cap, one block of rows
     (30.0, 1, 3.0),      # three blocks of rows
     (30.0, 0, 60.0),     # logits far into the cap on both sides: exp(z - cap) spans exp(-60)..1
-    (40.0, 2, 8.0),      # the largest cap the two-contraction sequence takes
-    (50.0, 0, 8.0),      # beyond it: statistics pass first, three contractions
+    (40.0, 2, 8.0),      # the largest cap that sequence takes
+    (50.0, 0, 8.0),      # beyond it, and without a cap: one emitting pass (entries relative
+    (None, 1, 3.0),      # to exact tile maxima), an elementwise normalisation, the contraction
+    (None, 0, 40.0),     # logits hundreds of nats apart
 ])
-def test_capped_soft_embedding_takes_two_contractions(gpu_device, softcap, tiles_per_block, std):
+def test_soft_embedding_takes_two_contractions(gpu_device, softcap, tiles_per_block, std):
     """Capped logits lie in [-cap, cap]: exp(z - cap) needs no row maximum, so the
     device path writes it to the panel in one contraction and normalises after the
-    second (which sequence ran is read from the library's per-class launch counts)."""
+    second.  Without a usable cap one pass over the head emits exp2(z2 - tile maximum)
+    with the softmax partials, and the entries are normalised per (token, tile) before
+    the second contraction.  No statistics pass either way (which sequence ran is read
+    from the library's per-class launch counts)."""
     from turbo_dllm_amd import _lib, options
     print("[case] capped soft embedding", softcap, tiles_per_block, std, flush=True)
     m, hdim, v = 700, 128, 2048
-    gen = torch.Generator().manual_seed(int(softcap) + tiles_per_block)
+    gen = torch.Generator().manual_seed(int(softcap or 0) + tiles_per_block)
     h = torch.randn(m, hdim, generator=gen).to(torch.bfloat16)
     w = (torch.randn(v, hdim, generator=gen) * (std / hdim ** 0.5)).to(torch.bfloat16)
     with options.panel_budget(tiles_per_block * 256 * v * 2), _lib.kernel_profile() as prof:
@@ -111,12 +116,12 @@ def test_capped_soft_embedding_takes_two_contractions(gpu_device, softcap, tiles
                                        vocab_chunk_size=256, logit_softcap=softcap,
                                        embedding_scale=2.0)
         torch.cuda.synchronize()
-    two_contractions = softcap <= 40.0
-    assert (prof.launches["exp_logits_panel"] > 0) == two_contractions
-    assert (prof.launches["forward_stats"] == 0) == two_contractions
-    if two_contractions:
-        assert prof.launches["exp_logits_panel"] == (1 if tiles_per_block == 0 else
-                                                     -(-m // (256 * tiles_per_block)))
+    blocks = 1 if tiles_per_block == 0 else -(-m // (256 * tiles_per_block))
+    capped = softcap is not None and softcap <= 40.0
+    assert prof.launches["forward_stats"] == 0
+    assert prof.launches["exp_logits_panel"] == (blocks if capped else 0)
+    assert prof.launches["grad_logits_panel"] == (0 if capped else blocks)   # the emitting pass
+    assert prof.launches["grad_hidden_gemm"] == blocks
     assert bool(torch.isfinite(got.float()).all())
     err = rel_max(got.cpu(), dense(h, w, softcap, 2.0))
     print("[case] rel max err", f"{err:.2e}", flush=True)

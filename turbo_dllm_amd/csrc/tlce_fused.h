@@ -786,7 +786,23 @@ struct KlGradFromExpArgs {
   float softcap = 0.0f;      // > 0: the gradient is multiplied by cap'(z)
   const float* t_part_max = nullptr;   // non-null: `teacher` holds entries of the same kind,
   const float* t_lse = nullptr;        // these are the teacher's tile maxima and lse
+  // teacher == null: the entries are only normalised (softmax of the rows, times
+  // exp(-draft_lse offset) if the caller folded a factor into draft_lse)
 };
+
+// lse[r] - log(scale) from the per-tile (maximum, sum) partials of an emitting pass
+// (so that exp2(tile maximum - lse2) carries the factor `scale`), and row_scale = 1
+// (0 from m on) for the slab reduction that follows.
+struct EmitRowsArgs {
+  const float* part_max;   // [n_vtiles, part_ld] base-2 tile maxima
+  const float* part_sum;   // [n_vtiles, part_ld] sums of exp2(z2 - tile maximum)
+  int part_ld, n_vtiles;
+  int m, m_pad;
+  float scale;             // > 0
+  float* lse;              // [m_pad]
+  float* row_scale;        // [m_pad]
+};
+int launch_emit_rows(const EmitRowsArgs& a, hipStream_t stream);
 int launch_kl_grad_from_exp(const KlGradFromExpArgs& a, int n_vtiles, hipStream_t stream);
 
 struct KlFusedLayout {
@@ -937,6 +953,77 @@ int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout
   return launch_reduce_slabs(rs, stream);
 }
 
+// Soft embedding without a usable soft cap (none, or one above kSoftEmbeddingMaxCap), in
+// two contractions as well: one emitting pass over the head (entries relative to exact
+// tile maxima, softmax partials), the lse merged from the partials with the embedding
+// scale folded in, one elementwise pass that normalises the entries per (token, tile),
+// and the contraction with the weight rows.
+template <class E>
+int soft_embedding_emit_impl(const FusedPlan& p, const void* hidden, const void* weight,
+                             int64_t m, int64_t h, int64_t v, int dtype, float softcap,
+                             float scale, void* out, char* ws, hipStream_t stream) {
+  using T = typename E::T;
+  const FusedLayout l = fused_layout(p, m, h, dtype, false);
+  T* panel = reinterpret_cast<T*>(ws + l.panel);
+  float* part_sum = reinterpret_cast<float*>(ws + l.part_sum);
+  float* part_max = reinterpret_cast<float*>(ws + l.part_max);
+  float* lse = reinterpret_cast<float*>(ws + l.ref_next);
+  float* row_scale = reinterpret_cast<float*>(ws + l.row_scale);
+  float* slabs = reinterpret_cast<float*>(ws + l.slabs);
+  const T* hidden_t = static_cast<const T*>(hidden);
+  for (int block = 0; block < p.n_blocks; ++block) {
+    const int64_t r0 = (int64_t)block * p.block_rows;
+    const int64_t rows = std::min<int64_t>(p.block_rows, m - r0);
+    if (rows <= 0) break;
+    const int n_ttiles = (int)ceil_div(rows, E::kTile);
+    const int64_t rows_p = (int64_t)n_ttiles * E::kTile;
+
+    KlPanelArgs ka;
+    ka.hidden = hidden_t + r0 * h; ka.weight = weight; ka.lse = nullptr; ka.scale = nullptr;
+    ka.m = (int)rows; ka.h = (int)h; ka.v = (int)v; ka.softcap = softcap;
+    ka.v0 = 0; ka.n_ttiles = n_ttiles; ka.n_ptiles = p.n_vtiles;
+    ka.panel = panel; ka.ld = p.vp; ka.panel_in = nullptr;
+    ka.loss_part = nullptr; ka.tsum_part = nullptr;
+    ka.part_max = part_max; ka.part_sum = part_sum; ka.part_ld = (int)p.block_rows;
+    ka.mode = kKlLoss;
+    if (int rc = launch_kl_panel_emit<E>(ka, stream)) return rc;
+
+    EmitRowsArgs er;
+    er.part_max = part_max; er.part_sum = part_sum; er.part_ld = (int)p.block_rows;
+    er.n_vtiles = p.n_vtiles; er.m = (int)rows; er.m_pad = (int)rows_p; er.scale = scale;
+    er.lse = lse; er.row_scale = row_scale;
+    if (int rc = launch_emit_rows(er, stream)) return rc;
+
+    KlGradFromExpArgs ga;
+    ga.exp_panel = panel; ga.teacher = nullptr; ga.ld = p.vp;
+    ga.m = (int)rows; ga.mp = (int)rows_p;
+    ga.part_max = part_max; ga.part_ld = (int)p.block_rows; ga.draft_lse = lse;
+    ga.softcap = 0.0f;     // a forward value: no cap'
+    if (int rc = launch_kl_grad_from_exp(ga, p.n_vtiles, stream)) return rc;
+
+    GemmArgs g;
+    g.a = weight; g.lda = h; g.a_rows = (int)h;
+    g.b = panel; g.ldb = p.vp; g.b_rows = (int)rows_p;
+    g.k = (int)round_up(v, 64); g.k_per_split = 0;
+    g.ni = p.n_htiles; g.nj = n_ttiles;
+    g.c = slabs; g.ldc = h; g.c_rows = (int)rows_p; g.c_cols = (int)h;
+    g.c_split_stride = p.block_rows * h;
+    g.mode = kStoreF32;
+    const int ksplit = (rows_p == p.block_rows)
+                           ? p.dh_ksplit
+                           : std::min(p.dh_ksplit,
+                                      grad_hidden_k_splits((int64_t)n_ttiles * p.n_htiles,
+                                                           p.dh_ksplit, p.vp / 64, rows_p * h));
+    if (int rc = launch_gemm<E, true, false>(g, ksplit, kClassGradHidden, stream)) return rc;
+    ReduceSlabsArgs rs;
+    rs.slabs = slabs; rs.n_splits = ksplit; rs.split_stride = p.block_rows * h;
+    rs.row_scale = row_scale; rs.m = (int)rows; rs.h = (int)h;
+    rs.out = nullptr; rs.out_t = static_cast<T*>(out) + r0 * h;
+    if (int rc = launch_reduce_slabs(rs, stream)) return rc;
+  }
+  return 0;
+}
+
 #define TLCE_LAUNCHERS_EXP_PANEL(X, E)                                                  \
   X int launch_kl_panel_emit<E>(const KlPanelArgs&, hipStream_t);                       \
   X int launch_exp_panel_variant<E, false, false>(const ExpPanelArgs&, hipStream_t);    \
@@ -950,6 +1037,9 @@ int kl_forward_with_gradient_impl(const Plan& pd, const Plan& pt, const KlLayout
   X int soft_embedding_fused_impl<E>(const FusedPlan&, const void*, const void*, int64_t,        \
                                      int64_t, int64_t, int, float, float, void*, char*,          \
                                      hipStream_t);                                               \
+  X int soft_embedding_emit_impl<E>(const FusedPlan&, const void*, const void*, int64_t,         \
+                                    int64_t, int64_t, int, float, float, void*, char*,           \
+                                    hipStream_t);                                                \
   X int topk_forward_with_gradient_impl<E>(const TopkPlan&, const FusedPlan&, const void*,       \
                                            const void*, const int64_t*, int64_t, int64_t,        \
                                            int64_t, int, float, float, float*, float*, float*,   \

@@ -211,7 +211,14 @@ __global__ __launch_bounds__(256) void lce_kl_grad_from_exp_kernel(KlGradFromExp
   __bf16* e = static_cast<__bf16*>(p.exp_panel) + (int64_t)r * p.ld + c;
   typedef __bf16 v8_t __attribute__((ext_vector_type(8)));
   v8_t out;
-  if (r < p.m) {
+  if (r < p.m && p.teacher == nullptr) {
+    // only normalise: softmax (times what the caller folded into draft_lse)
+    const float f = exp2f(p.part_max[(int64_t)tile * p.part_ld + r] -
+                          p.draft_lse[r] * TLCE_LOG2E);
+    const v8_t ev = *reinterpret_cast<const v8_t*>(e);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = from_float<__bf16>(to_float<__bf16>(ev[i]) * f);
+  } else if (r < p.m) {
     const float tile_max2 = p.part_max[(int64_t)tile * p.part_ld + r];
     const float f = exp2f(tile_max2 - p.draft_lse[r] * TLCE_LOG2E);
     const float ft = p.t_part_max != nullptr
@@ -357,6 +364,27 @@ __global__ __launch_bounds__(256) void lce_topk_apply_kernel(TopkApplyArgs p) {
     }
     out[k] = from_float<T>(acc);
   }
+}
+
+// One thread per row, 64 rows per workgroup: the tiles' (maximum, sum) pairs merged in
+// tile order.
+__global__ __launch_bounds__(64) void lce_emit_rows_kernel(EmitRowsArgs p) {
+  const int r = blockIdx.x * 64 + threadIdx.x;
+  if (r >= p.m_pad) return;
+  if (r >= p.m) {
+    p.lse[r] = 0.0f;
+    p.row_scale[r] = 0.0f;
+    return;
+  }
+  float mx = -INFINITY;
+  for (int t = 0; t < p.n_vtiles; ++t) mx = fmaxf(mx, p.part_max[(int64_t)t * p.part_ld + r]);
+  float sum = 0.0f;
+  for (int t = 0; t < p.n_vtiles; ++t) {
+    const float pm = p.part_max[(int64_t)t * p.part_ld + r];
+    if (pm > -INFINITY) sum += p.part_sum[(int64_t)t * p.part_ld + r] * exp2f(pm - mx);
+  }
+  p.lse[r] = (mx + log2f(sum)) * TLCE_LN2 - logf(p.scale);
+  p.row_scale[r] = 1.0f;
 }
 
 // 64 rows per workgroup of 16 waves, the rows across the lanes (the partials are

@@ -891,8 +891,10 @@ __global__ __launch_bounds__(E::kThreads) void lce_kl_panel_kernel(KlPanelArgs p
       const int64_t o = (int64_t)tile_index * p.part_ld + tt * E::kTile + c;
       p.part_max[o] = mx;
       p.part_sum[o] = sum;
-      p.loss_part[o] = loss;
-      p.tsum_part[o] = mass;
+      if (p.loss_part != nullptr) {   // (null: a pass that only emits)
+        p.loss_part[o] = loss;
+        p.tsum_part[o] = mass;
+      }
     }
   }
 }

@@ -127,6 +127,13 @@ int launch_topk_apply(const TopkApplyArgs& a, hipStream_t stream) {
   return 0;
 }
 
+int launch_emit_rows(const EmitRowsArgs& a, hipStream_t stream) {
+  ScopedTimer timer(kClassCombine, stream);
+  lce_emit_rows_kernel<<<(int)ceil_div(a.m_pad, 64), 64, 0, stream>>>(a);
+  TLCE_LAUNCH_CHECK();
+  return 0;
+}
+
 int launch_soft_rows(const SoftRowsArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassCombine, stream);
   lce_soft_rows_kernel<<<(int)ceil_div(a.m_pad, 64), 64 * kSoftRowsWaves, 0, stream>>>(a);
@@ -544,16 +551,22 @@ extern "C" int tlce_soft_embedding(const void* hidden, const void* weight, int64
   if (m == 0) return 0;
   TLCE_REQUIRE(out != nullptr && workspace != nullptr, "soft_embedding: null pointer");
   TLCE_REQUIRE(((uintptr_t)out & 15) == 0, "soft_embedding: out must be 16-byte aligned");
-  if (logit_softcap > 0.0f && logit_softcap <= kSoftEmbeddingMaxCap &&
-      fused_gradients_supported(h, v, dtype)) {
-    // under a soft cap no row maximum is needed: two contractions instead of three
+  if (fused_gradients_supported(h, v, dtype) && embedding_scale > 0.0f) {
+    // two contractions instead of three: under a soft cap of at most 40 no row maximum is
+    // needed at all; otherwise one pass emits entries relative to exact tile maxima
+    const bool capped = logit_softcap > 0.0f && logit_softcap <= kSoftEmbeddingMaxCap;
     const FusedPlan p = make_fused_plan(m, h, v, dtype, panel_bytes);
     const int64_t need = fused_layout(p, m, h, dtype, false).total;
     TLCE_REQUIRE(workspace_bytes >= need, "soft_embedding: workspace too small (%lld < %lld)",
                  (long long)workspace_bytes, (long long)need);
     TLCE_REQUIRE(((uintptr_t)workspace & 255) == 0,
                  "soft_embedding: workspace must be 256-byte aligned");
-    return soft_embedding_fused_impl<MfmaDirect4Engine<__bf16>>(
+    if (capped) {
+      return soft_embedding_fused_impl<MfmaDirect4Engine<__bf16>>(
+          p, hidden, weight, m, h, v, dtype, logit_softcap, embedding_scale, out,
+          static_cast<char*>(workspace), stream);
+    }
+    return soft_embedding_emit_impl<MfmaDirect4Engine<__bf16>>(
         p, hidden, weight, m, h, v, dtype, logit_softcap, embedding_scale, out,
         static_cast<char*>(workspace), stream);
   }
