@@ -353,38 +353,30 @@ __global__ __launch_bounds__(256) void lce_topk_apply_kernel(TopkApplyArgs p) {
     }
   }
   __syncthreads();
+  // eight consecutive columns per thread and step (h is a multiple of 64 on this path):
+  // 16-byte reads of the weight rows, 16-byte store
   const float* unit = p.unit + (int64_t)r * p.h;
   T* out = static_cast<T*>(p.grad_hidden) + (int64_t)r * p.h;
-  for (int k = t; k < p.h; k += 256) {
-    float acc = scale * unit[k];
+  typedef T v8_t __attribute__((ext_vector_type(8)));
+  for (int k = t * 8; k < p.h; k += 256 * 8) {
+    const f32x4_t u0 = *reinterpret_cast<const f32x4_t*>(unit + k);
+    const f32x4_t u1 = *reinterpret_cast<const f32x4_t*>(unit + k + 4);
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = scale * (i < 4 ? u0[i] : u1[i - 4]);
     for (int e = 0; e < n_entries; ++e) {
-      if (coef[e] != 0.0f)
-        acc = fmaf(coef[e], to_float<T>(static_cast<const T*>(p.weight)[ids[e] * (int64_t)p.h + k]),
-                   acc);
+      const float c = coef[e];
+      if (c == 0.0f) continue;   // workgroup-uniform
+      const v8_t w = *reinterpret_cast<const v8_t*>(static_cast<const T*>(p.weight) +
+                                                    ids[e] * (int64_t)p.h + k);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(c, to_float<T>(w[i]), acc[i]);
     }
-    out[k] = from_float<T>(acc);
+    v8_t o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = from_float<T>(acc[i]);
+    *reinterpret_cast<v8_t*>(out + k) = o;
   }
-}
-
-// One thread per row, 64 rows per workgroup: the tiles' (maximum, sum) pairs merged in
-// tile order.
-__global__ __launch_bounds__(64) void lce_emit_rows_kernel(EmitRowsArgs p) {
-  const int r = blockIdx.x * 64 + threadIdx.x;
-  if (r >= p.m_pad) return;
-  if (r >= p.m) {
-    p.lse[r] = 0.0f;
-    p.row_scale[r] = 0.0f;
-    return;
-  }
-  float mx = -INFINITY;
-  for (int t = 0; t < p.n_vtiles; ++t) mx = fmaxf(mx, p.part_max[(int64_t)t * p.part_ld + r]);
-  float sum = 0.0f;
-  for (int t = 0; t < p.n_vtiles; ++t) {
-    const float pm = p.part_max[(int64_t)t * p.part_ld + r];
-    if (pm > -INFINITY) sum += p.part_sum[(int64_t)t * p.part_ld + r] * exp2f(pm - mx);
-  }
-  p.lse[r] = (mx + log2f(sum)) * TLCE_LN2 - logf(p.scale);
-  p.row_scale[r] = 1.0f;
 }
 
 // 64 rows per workgroup of 16 waves, the rows across the lanes (the partials are
@@ -409,6 +401,47 @@ __global__ __launch_bounds__(64 * kSoftRowsWaves) void lce_soft_rows_kernel(Soft
 #pragma unroll
   for (int w = 0; w < kSoftRowsWaves; ++w) sum += sh[w][lane];
   p.row_scale[r] = (r < p.m && sum > 0.0f) ? p.scale / sum : 0.0f;
+}
+
+// The tiles' (maximum, sum) pairs of an emitting pass merged into lse - log(scale), the
+// same way: 64 rows per workgroup of 16 waves, wave w merging the tiles w, w + 16, ...
+// in ascending order, the 16 partial pairs merged in wave order.
+__global__ __launch_bounds__(64 * kSoftRowsWaves) void lce_emit_rows_kernel(EmitRowsArgs p) {
+  __shared__ float sh_max[kSoftRowsWaves][64];
+  __shared__ float sh_sum[kSoftRowsWaves][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = blockIdx.x * 64 + lane;
+  float mx = -INFINITY, sum = 0.0f;
+  if (r < p.m) {
+    for (int t = wave; t < p.n_vtiles; t += kSoftRowsWaves) {
+      const float pm = p.part_max[(int64_t)t * p.part_ld + r];
+      const float ps = p.part_sum[(int64_t)t * p.part_ld + r];
+      if (pm > -INFINITY) {
+        const float nm = fmaxf(mx, pm);
+        sum = sum * exp2f(mx - nm) + ps * exp2f(pm - nm);   // (exp2f(-inf) = 0 the first time)
+        mx = nm;
+      }
+    }
+  }
+  sh_max[wave][lane] = mx;
+  sh_sum[wave][lane] = sum;
+  __syncthreads();
+  if (wave != 0 || r >= p.m_pad) return;
+  if (r >= p.m) {
+    p.lse[r] = 0.0f;
+    p.row_scale[r] = 0.0f;
+    return;
+  }
+  mx = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < kSoftRowsWaves; ++w) mx = fmaxf(mx, sh_max[w][lane]);
+  sum = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kSoftRowsWaves; ++w)
+    if (sh_max[w][lane] > -INFINITY) sum += sh_sum[w][lane] * exp2f(sh_max[w][lane] - mx);
+  p.lse[r] = (mx + log2f(sum)) * TLCE_LN2 - logf(p.scale);
+  p.row_scale[r] = 1.0f;
 }
 
 template <typename T>

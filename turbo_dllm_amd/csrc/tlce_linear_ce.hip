@@ -46,8 +46,8 @@ int launch_token_scale(const ScaleArgs& sa, hipStream_t stream) {
 
 int launch_kl_finish(float* losses, const float* loss_part, const float* tsum_part, int n_tiles,
                      int64_t part_ld, const float* lse, int64_t m, hipStream_t stream) {
-  lce_kl_finish_kernel<<<(int)ceil_div(m, 256), 256, 0, stream>>>(losses, loss_part, tsum_part,
-                                                                  n_tiles, part_ld, lse, (int)m);
+  lce_kl_finish_kernel<<<(int)ceil_div(m, 64), 64 * kKlFinishWaves, 0, stream>>>(
+      losses, loss_part, tsum_part, n_tiles, part_ld, lse, (int)m);
   TLCE_LAUNCH_CHECK();
   return 0;
 }
@@ -129,7 +129,7 @@ int launch_topk_apply(const TopkApplyArgs& a, hipStream_t stream) {
 
 int launch_emit_rows(const EmitRowsArgs& a, hipStream_t stream) {
   ScopedTimer timer(kClassCombine, stream);
-  lce_emit_rows_kernel<<<(int)ceil_div(a.m_pad, 64), 64, 0, stream>>>(a);
+  lce_emit_rows_kernel<<<(int)ceil_div(a.m_pad, 64), 64 * kSoftRowsWaves, 0, stream>>>(a);
   TLCE_LAUNCH_CHECK();
   return 0;
 }

@@ -83,18 +83,37 @@ __global__ __launch_bounds__(256) void lce_segment_weighted_sum_kernel(
   if (threadIdx.x == 0) out[blockIdx.x] = part[0];
 }
 
-// losses[r] = sum_t loss_part[t][r] + (sum_t tsum_part[t][r]) * lse_draft[r] + 1, the
-// vocabulary tiles t added in ascending order (see lce_kl_panel_kernel).
-__global__ __launch_bounds__(256) void lce_kl_finish_kernel(float* losses, const float* loss_part,
-                                                            const float* tsum_part, int n_tiles,
-                                                            int64_t part_ld, const float* lse,
-                                                            int m) {
-  const int r = blockIdx.x * 256 + threadIdx.x;
-  if (r >= m) return;
+// losses[r] = sum_t loss_part[t][r] + (sum_t tsum_part[t][r]) * lse_draft[r] + 1 over the
+// vocabulary tiles t (see lce_kl_panel_kernel), in a fixed order: 64 rows per workgroup of
+// 16 waves, the rows across the lanes; wave w adds the tiles w, w + 16, ... in ascending
+// order and the 16 sums are merged in wave order.
+constexpr int kKlFinishWaves = 16;
+
+__global__ __launch_bounds__(64 * kKlFinishWaves) void lce_kl_finish_kernel(
+    float* losses, const float* loss_part, const float* tsum_part, int n_tiles, int64_t part_ld,
+    const float* lse, int m) {
+  __shared__ float sh_loss[kKlFinishWaves][64];
+  __shared__ float sh_mass[kKlFinishWaves][64];
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  const int r = blockIdx.x * 64 + lane;
   float loss = 0.0f, mass = 0.0f;
-  for (int t = 0; t < n_tiles; ++t) {
-    loss += loss_part[(int64_t)t * part_ld + r];
-    mass += tsum_part[(int64_t)t * part_ld + r];
+  if (r < m) {
+    for (int t = wave; t < n_tiles; t += kKlFinishWaves) {
+      loss += loss_part[(int64_t)t * part_ld + r];
+      mass += tsum_part[(int64_t)t * part_ld + r];
+    }
+  }
+  sh_loss[wave][lane] = loss;
+  sh_mass[wave][lane] = mass;
+  __syncthreads();
+  if (wave != 0 || r >= m) return;
+  loss = 0.0f;
+  mass = 0.0f;
+#pragma unroll
+  for (int w = 0; w < kKlFinishWaves; ++w) {
+    loss += sh_loss[w][lane];
+    mass += sh_mass[w][lane];
   }
   losses[r] = loss + mass * lse[r] + 1.0f;
 }
