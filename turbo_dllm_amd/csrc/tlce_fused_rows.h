@@ -310,13 +310,12 @@ __global__ __launch_bounds__(256) void lce_topk_row_scale_kernel(TopkRowScaleArg
 //   - ce_scale[r] * d'(label) * W[label] + sum_j grad_top_values[r, j] * d'(id_j) * W[id_j]
 // (dflash_linear_topk.py:196-225) with d'(v) = multiplier * (1 - tanh^2(multiplier *
 // h.W[v] / cap)) (multiplier alone without a cap), rounded once.  The coefficients
-// of the single-row terms are formed first (one dot product each), then every
-// column is summed in float32.
+// of the single-row terms are formed first (under a soft cap one dot product each, a
+// wave per entry), then every column is summed in float32.
 constexpr int kTopkApplyMaxEntries = 257;   // top_k <= 256, plus the label
 
 template <typename T>
 __global__ __launch_bounds__(256) void lce_topk_apply_kernel(TopkApplyArgs p) {
-  __shared__ float red[4];
   __shared__ float coef[kTopkApplyMaxEntries];
   __shared__ int64_t ids[kTopkApplyMaxEntries];
   const int t = threadIdx.x;
@@ -325,30 +324,21 @@ __global__ __launch_bounds__(256) void lce_topk_apply_kernel(TopkApplyArgs p) {
   const T* hrow = static_cast<const T*>(p.hidden) + (int64_t)r * p.h;
   const float scale = p.ce_scale[r];
   const int n_entries = (p.grad_top_values != nullptr ? p.k : 0) + 1;
-  for (int e = 0; e < n_entries; ++e) {
+  // one wave per entry, the waves taking every fourth: the raw logit is needed only for
+  // the soft cap's derivative
+  for (int e = wave; e < n_entries; e += 4) {
     const bool is_label = e == n_entries - 1;
     const int64_t id = is_label ? p.labels[r] : p.top_ids[(int64_t)r * p.k + e];
     const float weight_in = is_label ? -scale : p.grad_top_values[(int64_t)r * p.k + e];
-    float c = 0.0f;
-    if (weight_in != 0.0f) {   // workgroup-uniform
+    float deriv = p.logit_scale;
+    if (p.softcap > 0.0f && weight_in != 0.0f) {   // wave-uniform
       const T* wrow = static_cast<const T*>(p.weight) + id * (int64_t)p.h;
-      float dot = 0.0f;
-      for (int k = t; k < p.h; k += 256)
-        dot = fmaf(to_float<T>(hrow[k]), to_float<T>(wrow[k]), dot);
-      dot = wave_sum(dot);
-      if (lane == 0) red[wave] = dot;
-      __syncthreads();
-      const float raw = (red[0] + red[1] + red[2] + red[3]) * p.logit_scale;
-      __syncthreads();
-      float deriv = p.logit_scale;
-      if (p.softcap > 0.0f) {
-        const float th = tanhf(raw / p.softcap);
-        deriv *= 1.0f - th * th;
-      }
-      c = weight_in * deriv;
+      const float raw = wave_dot<T>(hrow, wrow, p.h, lane) * p.logit_scale;
+      const float th = tanhf(raw / p.softcap);
+      deriv *= 1.0f - th * th;
     }
-    if (t == 0) {
-      coef[e] = c;
+    if (lane == 0) {
+      coef[e] = weight_in * deriv;
       ids[e] = id;
     }
   }
