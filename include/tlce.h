@@ -396,7 +396,7 @@ int64_t tlce_kl_teacher_probabilities_bytes(int64_t m, int64_t h_draft,
  *   unit_grad_hidden_f32[r, :] = d losses[r] / d draft_hidden[r, :]   float32 [m, h_draft].
  * The backward is tlce_apply_grad_output(unit, NULL, NULL, NULL, grad_output, NULL,
  * m, m, h_draft, v, dtype, TLCE_REDUCTION_NONE, grad_hidden, NULL, stream).
- * bf16, a soft cap of at most 40 or none, both hidden sizes and v multiples of 64
+ * bf16, a soft cap between 10 and 40 or none, both hidden sizes and v multiples of 64
  * (tlce_kl_gradient_in_forward_supported); rows are taken in blocks of the 2.5 GiB
  * panel budget one after the other, and the workspace holds both panels of a block
  * (2 x 2 bytes per padded row and vocabulary entry). */

@@ -167,12 +167,12 @@ def test_kept_teacher_probabilities_give_the_same_gradient(gpu_device, dtype, hd
     (300, 128, 192, 4096, 0.2, None),
     (700, 64, 64, 2048, 1.5, None),  # logits tens of nats apart: entries far below their tile maximum
     (1, 256, 128, 576, 0.3, None),
-    (300, 128, 128, 2048, 0.3, 6.0),
+    (300, 128, 128, 2048, 0.3, 12.0),
     (520, 64, 128, 4096, 3.0, 30.0),  # logits deep in the cap on both sides
 ])
 def test_gradient_formed_in_the_forward(gpu_device, m, hd, ht, v, std, softcap,
                                         set_panel_budget):
-    """bf16 (with a soft cap of at most 40, or none): the draft pass of the forward leaves
+    """bf16 (with a soft cap between 10 and 40, or none): the draft pass of the forward leaves
     exp2(z2 - tile maximum), and d loss / d draft_hidden is contracted in the forward (its grad_hidden
     contraction shows in the forward's launch counts); the backward scales rows.  Loss and
     gradient against the float64 oracle; the loss is held to the plain forward's distance

@@ -1187,7 +1187,7 @@ def dflash_kl_forward(
 def kl_gradient_in_forward_supported(draft_hidden, draft_weight, teacher_hidden,
                                      logit_softcap: float) -> bool:
     """Whether ``dflash_kl_forward_with_gradient`` takes these operands (bf16, a soft cap
-    of at most 40 or none, hidden sizes and V multiples of 64; rows go in blocks of the
+    between 10 and 40 or none, hidden sizes and V multiples of 64; rows go in blocks of the
     panel budget)."""
     if draft_hidden.dtype != torch.bfloat16 or draft_hidden.shape[0] == 0:
         return False

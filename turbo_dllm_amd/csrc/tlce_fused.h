@@ -805,6 +805,8 @@ struct EmitRowsArgs {
 int launch_emit_rows(const EmitRowsArgs& a, hipStream_t stream);
 int launch_kl_grad_from_exp(const KlGradFromExpArgs& a, int n_vtiles, hipStream_t stream);
 
+constexpr float kKlMinCap = 10.0f;
+
 struct KlFusedLayout {
   int64_t kl, teacher_parts, teacher, exp_panel, slabs, total;
 };
@@ -838,8 +840,13 @@ int launch_kl_panel_emit(const KlPanelArgs& a, hipStream_t stream) {
 inline bool kl_gradient_in_forward_supported(int64_t m, int64_t hd, int64_t ht, int64_t v,
                                              int dtype, float softcap) {
   (void)m;   // rows beyond one block of the panel budget are taken block by block
-  return softcap <= kSoftEmbeddingMaxCap && fused_gradients_supported(hd, v, dtype) &&
-         engine_class(ht, dtype) == 2;
+  // cap'(z) is re-derived from entries rounded to bf16, which moves z by up to 0.003 and
+  // cap' = 1 - (z / cap)^2 by up to 0.006 / cap: negligible beside the entries whose cap'
+  // is of order one, but under a small cap with every logit deep in it nothing else is
+  // left (measured: 2 % of the gradient's largest entry at cap 3): caps below 10 keep the
+  // sequence that evaluates cap' on the float32 logit
+  const bool cap_ok = softcap <= 0.0f || (softcap >= kKlMinCap && softcap <= kSoftEmbeddingMaxCap);
+  return cap_ok && fused_gradients_supported(hd, v, dtype) && engine_class(ht, dtype) == 2;
 }
 
 inline KlFusedLayout kl_fused_layout(const KlLayout& kl, const Plan& pd, const FusedPlan& p,

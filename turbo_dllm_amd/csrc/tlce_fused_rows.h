@@ -236,7 +236,7 @@ __global__ __launch_bounds__(256) void lce_kl_grad_from_exp_kernel(KlGradFromExp
       if (p.softcap > 0.0f) {
         // (an entry of 0 is a column past the vocabulary: its gradient is 0 anyway)
         const float t = ei > 0.0f ? (log2f(ei) + tile_max2) * inv_cap : 0.0f;
-        g *= 1.0f - t * t;
+        g *= fmaxf(1.0f - t * t, 0.0f);   // (|z| <= cap: a rounded entry can say otherwise)
       }
       out[i] = from_float<__bf16>(g);
     }

@@ -29,7 +29,7 @@ class _FrozenLinearKL(torch.autograd.Function):
         from . import options
         wants = (bool(ctx.needs_input_grad[0]) and options.get_gradient_mode() == "forward"
                  and operands[0].shape[0] > 0)
-        # bf16, a soft cap of at most 40 or none: the draft
+        # bf16, a soft cap between 10 and 40 or none: the draft
         # pass of the forward leaves what the logit gradient needs, and one contraction
         # more in the forward leaves d loss / d draft_hidden (4 contractions per step);
         # the backward only multiplies each row by its upstream gradient
