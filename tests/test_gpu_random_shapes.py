@@ -69,6 +69,16 @@ HARD_CASES = {
                 why="float32, 1 row, V=3, bias: exp(z - lse) - 1 cancels"),
     37105: dict(widen=1.0, measured="1.6e-6 against 2e-5",
                 why="float32, 1 row, soft cap 2: was the tanh approximation"),
+    # a later run of draws 45 000 - 75 000: four more of the same kind, all float32 with V=3
+    # and one or two rows, where softmax(label) is within 1e-4 of 1 and exp(z - lse) - 1 cancels
+    54654: dict(widen=4.0, measured="2.05e-5 (bias gradient) and 5.6e-5 (masked loss grad_hidden) against 2e-5",
+                why="float32, 1 row, V=3, bias: exp(z - lse) - 1 cancels"),
+    61292: dict(widen=8.0, measured="1.2e-4 against 2e-5",
+                why="float32, 2 rows, V=3, soft cap 30: exp(z - lse) - 1 cancels"),
+    61720: dict(widen=24.0, measured="2.7e-4 (grad_hidden) and 3.4e-4 (grad_weight) against 2e-5 (masked loss)",
+                why="float32, 1 row, V=3, soft cap 30: exp(z - lse) - 1 cancels"),
+    74424: dict(widen=5.0, measured="5.0e-5 (grad_hidden) and 6.4e-5 (grad_weight) against 2e-5",
+                why="float32, 2 rows, V=3: exp(z - lse) - 1 cancels"),
 }
 
 
